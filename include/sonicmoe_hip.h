@@ -1,0 +1,150 @@
+/* C ABI of libsonicmoe_hip.so: the gfx950 (MI355X) kernels behind the `sonicmoe::*` operators of the MoE layer.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; the library never allocates device memory
+ *   - `stream` is a hipStream_t passed as void* (NULL = default stream); all work is asynchronous on it
+ *   - return value: 0 = SMOE_OK, otherwise an smoe_status; smoe_last_error() gives the message of the last
+ *     failing call on the calling thread
+ *   - activations / weights are bf16 (raw uint16 bits), routing scores fp32, all indices int32
+ *   - weights are addressed in the PARAMETER layout of the reference module: W1 (E, 2I, H) and W2 (E, H, I),
+ *     innermost dimension contiguous, with explicit expert and row strides in ELEMENTS (the reference hands its
+ *     kernels permuted views of exactly these buffers: sonicmoe/moe.py:223-225)
+ *   - rows of the grouped tensors z, y1, y2, dz, y1s, dx_expanded are in expert-sorted order: rows
+ *     [off[e], off[e+1]) belong to expert e; row m was routed from token x_gather_idx[m] and flat routing
+ *     slot s_scatter_idx[m]
+ *   - a `workspace` argument is scratch memory of at least the matching *_workspace_bytes(); contents are
+ *     undefined before and after the call
+ *
+ * File:line citations name the reference interface each entry point replaces (paths relative to the
+ * reference tree).
+ */
+#ifndef SONICMOE_HIP_H
+#define SONICMOE_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  SMOE_OK = 0,
+  SMOE_ERR_INVALID = 1,     /* bad argument (null pointer, negative size, ...) */
+  SMOE_ERR_UNSUPPORTED = 2, /* shape / dtype outside what the kernels support */
+  SMOE_ERR_HIP = 3,         /* a HIP runtime call or launch failed */
+  SMOE_ERR_WORKSPACE = 4    /* workspace too small */
+} smoe_status;
+
+typedef enum { SMOE_DT_BF16 = 0, SMOE_DT_F16 = 1, SMOE_DT_F32 = 2 } smoe_dtype;
+
+/* sonicmoe/enums.py:18-26 */
+typedef enum {
+  SMOE_ACT_SWIGLU = 0,
+  SMOE_ACT_GEGLU = 1,
+  SMOE_ACT_REGLU = 2,
+  SMOE_ACT_RELU_SQ = 3,
+  SMOE_ACT_RELU = 4,
+  SMOE_ACT_GELU = 5,
+  SMOE_ACT_SILU = 6
+} smoe_activation;
+
+int smoe_version(void);
+const char* smoe_last_error(void);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Routing
+ * ------------------------------------------------------------------------------------------------------ */
+
+/* Expert histogram + INCLUSIVE prefix sum.  Replaces sonicmoe::count_cumsum_cuda
+ * (sonicmoe/count_cumsum/__init__.py:11-29, sonicmoe/count_cumsum/kernel.cu:92-205).
+ *   x        : n int32 (x_is_int64 = 0) or int64 (= 1) values in [0, E)
+ *   count    : E int32 out;  cumsum : E int32 out or NULL (do_cumsum = False)
+ * Limits: 1 <= E <= 65536 (the reference needs E % 4 == 0 and E <= 50000: kernel.cu:18, :161-162). */
+int smoe_count_cumsum(const void* x, int x_is_int64, int64_t n, int E, int32_t* count, int32_t* cumsum,
+                      void* stream);
+
+/* Fused top-K + softmax over router logits.  Replaces sonicmoe::_softmax_topk_fwd / sonicmoe::_topk_fwd
+ * (sonicmoe/functional/forward.py:20-50, :224-237; kernel sonicmoe/functional/topk_softmax.py:85-193).
+ *   logits (T, E) of `dtype` with row stride `row_stride` elements; scores (T, K) fp32; indices (T, K) int32
+ *   winners ordered by descending value, ties towards the lower column; softmax != 0 normalises the K winners
+ *   fp32 logits are compared with their low log2(next_pow2(E)) mantissa bits cleared, as the reference does
+ *   (topk_softmax.py:127-142).
+ * Limits: E <= 4096, K <= min(E, 64). */
+int smoe_topk_softmax_fwd(const void* logits, int dtype, int64_t T, int E, int K, int64_t row_stride,
+                          float* scores, int32_t* indices, int softmax, void* stream);
+
+/* dlogits[t, idx[t,k]] = s_k (ds_k - sum_j ds_j s_j); other entries are left untouched (caller zero-fills).
+ * Replaces sonicmoe::_softmax_topk_bwd (sonicmoe/functional/backward.py:487-556). dlogits has `dtype`. */
+int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const float* dscores, const float* scores,
+                          const int32_t* indices, int64_t T, int K, void* stream);
+
+/* Routing metadata by a stable counting sort over expert ids.  Replaces TC_topk_router_metadata and
+ * general_routing_router_metadata incl. their count_cumsum / argsort / index kernels
+ * (sonicmoe/functional/__init__.py:19-46, :49-82).
+ *   expert_idx (TK) int32 in [0, E)
+ *   token_idx  (TK) int32 sorted ascending, or NULL for token-choice top-K where slot j belongs to token j / K
+ *   outputs: freq (E), off (E+1, leading 0), x_gather_idx / s_scatter_idx / s_reverse_scatter_idx (TK),
+ *            tok_off (T+1) per-token slot offsets (may be NULL)
+ * Limits: E <= 4096. */
+size_t smoe_routing_metadata_workspace_bytes(int64_t TK, int E);
+int smoe_routing_metadata(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T, int E, int K,
+                          int32_t* freq, int32_t* off, int32_t* x_gather_idx, int32_t* s_scatter_idx,
+                          int32_t* s_reverse_scatter_idx, int32_t* tok_off, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Grouped GEMMs (bf16 in, fp32 MFMA accumulate, bf16 out)
+ * ------------------------------------------------------------------------------------------------------ */
+
+/* Workspace needed by every grouped GEMM below (tile map built from `off` on the device). */
+size_t smoe_gemm_workspace_bytes(int64_t TK, int E);
+
+/* z[m] = x[x_gather_idx[m]] W1[e]^T ; y1[m] = act(z_even) * z_odd (GLU, gate = even columns) or act(z).
+ * Replaces sonicmoe::_up_projection_forward (sonicmoe/functional/forward.py:53-129).
+ *   x (T, H); w1 (E, N1, H) with N1 = 2I (GLU) or I; z (TK, N1) or NULL (inference: not stored); y1 (TK, I)
+ * Limits: H % 64 == 0, I % 64 == 0, SwiGLU only in this version, no bias. */
+int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* z,
+                               void* y1, const int32_t* off, const int32_t* x_gather_idx, int64_t T, int64_t TK,
+                               int H, int I, int E, int activation, void* workspace, size_t workspace_bytes,
+                               void* stream);
+
+/* y2[m] = y1[m] W2[e]^T.  Replaces sonicmoe::_down_projection_forward (sonicmoe/functional/forward.py:132-178).
+ *   y1 (TK, I); w2 (E, H, I); y2 (TK, H) */
+int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
+                                 void* y2, const int32_t* off, int64_t TK, int H, int I, int E, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
+/* out[t] = sum_{j in [tok_off[t], tok_off[t+1])} w[j] * src[ridx[j]]  (w == NULL: unweighted), fp32 accumulate.
+ * Replaces sonicmoe::_router_forward and sonicmoe::_token_broadcast_backward
+ * (sonicmoe/functional/forward.py:181-202, backward.py:464-484; kernel reduction_over_k_gather.py:441-517).
+ *   tok_off == NULL means fixed K slots per token (slot j of token t is t*K + j). */
+int smoe_gather_sum(const void* src, void* out, const float* w, const int32_t* ridx, const int32_t* tok_off,
+                    int64_t T, int K, int H, void* stream);
+
+/* Backward of down projection + combine.  Replaces sonicmoe::_down_projection_backward
+ * (sonicmoe/functional/backward.py:286-461).
+ *   dy1 = dout[x_gather_idx] W2[e] (never stored); with (g,u) = z pairs and s = scores[s_scatter_idx[m]]:
+ *   dz (TK, 2I), y1s = s*silu(g)*u (TK, I), ds[s_scatter_idx[m]] = sum_i dy1*y1 (fp32, flat-slot order),
+ *   dw2 (E, H, I) = sum_m dout[t_m]^T (x) y1s[m]  (zeros for empty experts).
+ *   ds_partial: fp32 scratch of TK * smoe_dz_partial_cols(I) elements. */
+int smoe_dz_partial_cols(int I);
+int smoe_down_projection_backward(const void* dout, const void* z, const void* w2, int64_t w2_stride_e,
+                                  int64_t w2_stride_row, void* dw2, int64_t dw2_stride_e, int64_t dw2_stride_row,
+                                  void* dz, void* y1s, float* ds, float* ds_partial, const float* scores,
+                                  const int32_t* off, const int32_t* x_gather_idx, const int32_t* s_scatter_idx,
+                                  int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                  size_t workspace_bytes, void* stream);
+
+/* dW1[e] = sum_m dz[m]^T (x) x[t_m];  dx_expanded[m] = dz[m] W1[e].
+ * Replaces sonicmoe::_up_projection_backward (sonicmoe/functional/backward.py:195-283). */
+int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
+                                const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row,
+                                void* dx_expanded, const int32_t* off, const int32_t* x_gather_idx, int64_t T,
+                                int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SONICMOE_HIP_H */

@@ -1,0 +1,61 @@
+// Shared host/device helpers for the gfx950 kernels of the MoE-layer hot path.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/sonicmoe_hip.h"
+
+namespace smoe {
+
+// ---- error reporting -------------------------------------------------------------------------------------
+void set_error(const char* fmt, ...);  // thread-local message behind smoe_last_error()
+
+#define SMOE_REQUIRE(cond, code, ...)    \
+  do {                                   \
+    if (!(cond)) {                       \
+      ::smoe::set_error(__VA_ARGS__);    \
+      return (code);                     \
+    }                                    \
+  } while (0)
+
+#define SMOE_HIP_CHECK(expr)                                                                  \
+  do {                                                                                        \
+    hipError_t _e = (expr);                                                                   \
+    if (_e != hipSuccess) {                                                                   \
+      ::smoe::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+      return SMOE_ERR_HIP;                                                                    \
+    }                                                                                         \
+  } while (0)
+
+#define SMOE_LAUNCH_CHECK() SMOE_HIP_CHECK(hipGetLastError())
+
+static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// ---- device-side types -----------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
+
+#define SMOE_DEV static __device__ __forceinline__
+
+// bf16 <-> fp32 on raw bits; round-to-nearest-even, NaN kept quiet
+SMOE_DEV float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+SMOE_DEV uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+// two floats -> one 32-bit word holding (lo, hi) bf16
+SMOE_DEV uint32_t pack_bf16x2(float lo, float hi) { return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16); }
+SMOE_DEV float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+SMOE_DEV float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+SMOE_DEV float fast_sigmoid(float x) { return __frcp_rn(1.0f + __expf(-x)); }
+
+}  // namespace smoe

@@ -1,0 +1,417 @@
+// Grouped GEMM over ragged token groups ("varlen-M"): for every expert e and every grouped row m of that expert
+//     C[m, n] = sum_k P[row(m), k] * Q_e[n, k]
+// with fused epilogues.  Four roles of the MoE layer share the main loop:
+//   up-projection forward    P = x rows gathered by x_gather_idx, Q = W1[e] (K-major)   -> z, y1 = SwiGLU(z)
+//   down-projection forward  P = y1 rows,                          Q = W2[e] (K-major)   -> y2
+//   down-proj activation grad P = dout rows gathered,              Q = W2[e] (MN-major)  -> dz, y1s, ds partials
+//   up-proj activation grad  P = dz rows,                          Q = W1[e] (MN-major)  -> dx_expanded
+#include "gemm_common.h"
+
+namespace smoe {
+
+enum Role { ROLE_UP_FWD = 0, ROLE_PLAIN = 1, ROLE_DZ = 2 };
+
+struct VarlenMParams {
+  const uint16_t* P;
+  int64_t p_stride;
+  const int32_t* gidx;  // nullable: P rows are the grouped rows themselves
+  const uint16_t* Q;
+  int64_t q_stride_e, q_stride_row;
+  const int32_t* off;
+  TileMap tm;
+  int N, Kdim, n_tiles;
+  uint16_t* out0;
+  int64_t out0_stride;
+  uint16_t* out1;
+  int64_t out1_stride;
+  const uint16_t* zin;
+  int64_t zin_stride;
+  const float* scores;
+  const int32_t* sidx;
+  float* ds_partial;
+  int ds_cols;
+};
+
+template <int BM_, int BN_, int WM_, int WN_, bool QMN_>
+struct Cfg {
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr bool QMN = QMN_;
+  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int TM = BM / WM, TN = BN / WN;
+  static constexpr int FM = TM / 32, FN = TN / 32;
+  static constexpr int P_STAGE = BM * BK * 2, Q_STAGE = BN * BK * 2;
+  static constexpr int STAGE = P_STAGE + Q_STAGE;
+  static constexpr int P_INSTR = P_STAGE / 1024 / NW;
+  static constexpr int Q_INSTR = Q_STAGE / 1024 / NW;
+  static constexpr int SMEM = 2 * STAGE;
+  // MN-major Q stage geometry
+  static constexpr int ROWB = BN * 2;     // bytes per k-row
+  static constexpr int LPR = ROWB / 16;   // lanes (16-byte pieces) per k-row
+  static constexpr int RPI = 64 / LPR;    // k-rows per load instruction
+  static constexpr int NG = ROWB / 32;    // 32-byte groups per k-row
+  static constexpr int SWM = (NG < 16 ? NG : 16) - 1;
+  static_assert(P_INSTR >= 1 && Q_INSTR >= 1, "tile too small for the wave count");
+  static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA");
+};
+
+template <class C, int ROLE>
+__global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int BN = C::BN, FM = C::FM, FN = C::FN;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % C::WM, wn = wave / C::WM;
+
+  const int num_m_tiles = p.tm.header[0];
+  const int64_t total = (int64_t)num_m_tiles * p.n_tiles;
+  const int64_t lin = xcd_linear_tile(total);
+  if (lin < 0) return;
+  constexpr int GM = 8;
+  const int64_t per_group = (int64_t)GM * p.n_tiles;
+  const int group = (int)(lin / per_group);
+  const int first_m = group * GM;
+  const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
+  const int within = (int)(lin - (int64_t)group * per_group);
+  const int mt = first_m + within % gm;
+  const int nt = within / gm;
+  const int e = p.tm.expert[mt];
+  const int row0 = p.tm.row0[mt];
+  const int row_end = p.off[e + 1];
+  const int n0 = nt * BN;
+
+  // ---- per-lane global source pointers (advance by one stage per k-step) ----
+  const uint16_t* p_src[C::P_INSTR];
+#pragma unroll
+  for (int i = 0; i < C::P_INSTR; i++) {
+    const int r = (wave * C::P_INSTR + i) * 8 + (lane >> 3);
+    int m = row0 + r;
+    m = m < row_end ? m : row_end - 1;
+    const int64_t src_row = p.gidx ? (int64_t)p.gidx[m] : (int64_t)m;
+    p_src[i] = p.P + src_row * p.p_stride + (((lane & 7) ^ kswz(r)) << 3);
+  }
+  const uint16_t* q_src[C::Q_INSTR];
+  const uint16_t* qe = p.Q + (int64_t)e * p.q_stride_e;
+  int64_t q_step;
+  if constexpr (!C::QMN) {
+#pragma unroll
+    for (int i = 0; i < C::Q_INSTR; i++) {
+      const int r = (wave * C::Q_INSTR + i) * 8 + (lane >> 3);
+      int n = n0 + r;
+      n = n < p.N ? n : p.N - 1;
+      q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane & 7) ^ kswz(r)) << 3);
+    }
+    q_step = BK;
+  } else {
+#pragma unroll
+    for (int i = 0; i < C::Q_INSTR; i++) {
+      const int kl = (wave * C::Q_INSTR + i) * C::RPI + lane / C::LPR;
+      const int phys16 = lane % C::LPR;
+      const int log32 = (phys16 >> 1) ^ (kl & C::SWM);
+      int n = n0 + ((log32 << 1) | (phys16 & 1)) * 8;
+      n = n <= p.N - 8 ? n : p.N - 8;
+      q_src[i] = qe + (int64_t)kl * p.q_stride_row + n;
+    }
+    q_step = (int64_t)BK * p.q_stride_row;
+  }
+
+  // ---- per-lane LDS fragment offsets (bytes inside a stage) ----
+  int p_off[4];
+  {
+    const int row = wm * C::TM + (lane & 31);
+    const int sw = kswz(row);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) p_off[ks] = row * 128 + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+  }
+  int q_off[C::QMN ? 2 * FN : 4];
+  if constexpr (!C::QMN) {
+    const int row = wn * C::TN + (lane & 31);
+    const int sw = kswz(row);
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) q_off[ks] = C::P_STAGE + row * 128 + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+  } else {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int kk = 8 * (grp >> 1) + (i16 >> 2);
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+      const int c32 = (wn * C::TN) / 16 + fn * 2 + (grp & 1);
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int k = kk + 4 * h;
+        q_off[fn * 2 + h] = C::P_STAGE + k * C::ROWB + ((c32 ^ (k & C::SWM)) << 5) + ((i16 & 3) << 3);
+      }
+    }
+  }
+
+  f32x16 acc[FN][FM];
+#pragma unroll
+  for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
+
+  auto issue = [&](int stage) {
+    char* base = smem + stage * C::STAGE;
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) {
+      load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
+      p_src[i] += BK;
+    }
+#pragma unroll
+    for (int i = 0; i < C::Q_INSTR; i++) {
+      load16_to_lds(q_src[i], base + C::P_STAGE + (wave * C::Q_INSTR + i) * 1024);
+      q_src[i] += q_step;
+    }
+  };
+
+  const int KT = p.Kdim / BK;
+  issue(0);
+  for (int kt = 0; kt < KT; kt++) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of stage kt have landed
+    __syncthreads();                     // everyone's pieces have landed; everyone is done reading the other stage
+    if (kt + 1 < KT) issue((kt + 1) & 1);
+    const char* st = smem + (kt & 1) * C::STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      bf16x8 pf[FM], qf[FN];
+#pragma unroll
+      for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(st + p_off[ks] + fm * 32 * 128);
+#pragma unroll
+      for (int fn = 0; fn < FN; fn++) {
+        if constexpr (!C::QMN) {
+          qf[fn] = lds_read_b128(st + q_off[ks] + fn * 32 * 128);
+        } else {
+          qf[fn] = lds_read_tr2(st + q_off[fn * 2] + ks * 16 * C::ROWB, st + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
+        }
+      }
+#pragma unroll
+      for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+        for (int fm = 0; fm < FM; fm++) acc[fn][fm] = mfma32(qf[fn], pf[fm], acc[fn][fm]);
+    }
+  }
+
+  // ---- epilogue: lane owns token column m = l%32 and 4 consecutive features per register quad ----
+  static_for<FM>([&](auto fm_c) {
+    constexpr int fm = decltype(fm_c)::value;
+    const int m = row0 + wm * C::TM + fm * 32 + (lane & 31);
+    const bool mvalid = m < row_end;
+    float s = 0.f, dsum = 0.f;
+    if constexpr (ROLE == ROLE_DZ) {
+      if (mvalid) s = p.scores[p.sidx[m]];
+    }
+    static_for<FN * 4>([&](auto q_c) {
+      constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+      const int n = n0 + wn * C::TN + fn * 32 + 8 * rg + 4 * (lane >> 5);
+      const bool ok = mvalid && n < p.N;
+      const float a0 = acc[fn][fm][4 * rg + 0], a1 = acc[fn][fm][4 * rg + 1], a2 = acc[fn][fm][4 * rg + 2],
+                  a3 = acc[fn][fm][4 * rg + 3];
+      if constexpr (ROLE == ROLE_PLAIN) {
+        if (ok) {
+          u32x2 v = {pack_bf16x2(a0, a1), pack_bf16x2(a2, a3)};
+          *(u32x2*)(p.out0 + (int64_t)m * p.out0_stride + n) = v;
+        }
+      } else if constexpr (ROLE == ROLE_UP_FWD) {
+        if (ok) {
+          if (p.out0) {
+            u32x2 v = {pack_bf16x2(a0, a1), pack_bf16x2(a2, a3)};
+            *(u32x2*)(p.out0 + (int64_t)m * p.out0_stride + n) = v;
+          }
+          const float y0 = a0 * fast_sigmoid(a0) * a1;
+          const float y1v = a2 * fast_sigmoid(a2) * a3;
+          *(uint32_t*)(p.out1 + (int64_t)m * p.out1_stride + (n >> 1)) = pack_bf16x2(y0, y1v);
+        }
+      } else {  // ROLE_DZ: n indexes the intermediate feature i; z holds (gate, up) pairs
+        if (ok) {
+          const u32x4 zz = *(const u32x4*)(p.zin + (int64_t)m * p.zin_stride + 2 * n);
+          const float dy0[4] = {a0, a1, a2, a3};
+          u32x4 dzv;
+          float ys[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
+            const float sig = fast_sigmoid(g);
+            const float silu = g * sig;
+            const float y1v = silu * u;
+            dsum += dy0[q] * y1v;
+            const float sd = s * dy0[q];
+            const float dg = sd * u * (silu * (1.f - sig) + sig);
+            const float du = sd * silu;
+            dzv[q] = pack_bf16x2(dg, du);
+            ys[q] = s * y1v;
+          }
+          *(u32x4*)(p.out0 + (int64_t)m * p.out0_stride + 2 * n) = dzv;
+          u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
+          *(u32x2*)(p.out1 + (int64_t)m * p.out1_stride + n) = yv;
+        }
+      }
+    });
+    if constexpr (ROLE == ROLE_DZ) {
+      dsum += __shfl_xor(dsum, 32, 64);
+      if (mvalid && lane < 32) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
+    }
+  });
+}
+
+template <class C, int ROLE>
+static int launch_varlen_m(const VarlenMParams& p, int64_t TK, int E, hipStream_t st) {
+  static bool attr_set = false;
+  auto kern = varlen_m_kernel<C, ROLE>;
+  if (!attr_set) {
+    SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
+    attr_set = true;
+  }
+  const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
+  const int64_t grid = ((max_tiles + 7) / 8) * 8;
+  SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+// tile configurations ------------------------------------------------------------------------------------------
+using CfgKM = Cfg<256, 256, 2, 2, false>;   // K-major weights (forward GEMMs)
+using CfgMN = Cfg<256, 256, 2, 2, true>;    // MN-major weights (activation-gradient GEMMs)
+
+}  // namespace smoe
+
+using namespace smoe;
+
+static int check_common(int64_t TK, int H, int I, int E, const void* ws, size_t ws_bytes, const char* who) {
+  SMOE_REQUIRE(TK >= 0 && TK < (1ll << 31), SMOE_ERR_INVALID, "%s: TK out of range", who);
+  SMOE_REQUIRE(E >= 1, SMOE_ERR_INVALID, "%s: E must be >= 1", who);
+  SMOE_REQUIRE(H >= 64 && H % 64 == 0, SMOE_ERR_UNSUPPORTED, "%s: H=%d must be a multiple of 64", who, H);
+  SMOE_REQUIRE(I >= 64 && I % 64 == 0, SMOE_ERR_UNSUPPORTED, "%s: I=%d must be a multiple of 64", who, I);
+  SMOE_REQUIRE(ws != nullptr && ws_bytes >= smoe_gemm_workspace_bytes(TK, E), SMOE_ERR_WORKSPACE,
+               "%s: workspace too small", who);
+  return SMOE_OK;
+}
+
+extern "C" size_t smoe_gemm_workspace_bytes(int64_t TK, int E) {
+  if (TK < 0 || E < 1) return 0;
+  return tile_map_bytes(TK, E);
+}
+
+extern "C" int smoe_dz_partial_cols(int I) { return (int)ceil_div(I, CfgMN::BN) * CfgMN::WN; }
+
+extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
+                                          void* z, void* y1, const int32_t* off, const int32_t* x_gather_idx,
+                                          int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "up_projection_forward");
+  if (rc) return rc;
+  SMOE_REQUIRE(activation == SMOE_ACT_SWIGLU, SMOE_ERR_UNSUPPORTED,
+               "up_projection_forward: only SwiGLU is implemented (activation=%d)", activation);
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(x && w1 && y1 && off && x_gather_idx, SMOE_ERR_INVALID, "up_projection_forward: null pointer");
+  SMOE_REQUIRE(T > 0, SMOE_ERR_INVALID, "up_projection_forward: T must be positive");
+  hipStream_t st = (hipStream_t)stream;
+  using C = CfgKM;
+  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
+  rc = launch_build_tile_map(off, E, C::BM, tm, st);
+  if (rc) return rc;
+  VarlenMParams p = {};
+  p.P = (const uint16_t*)x;
+  p.p_stride = H;
+  p.gidx = x_gather_idx;
+  p.Q = (const uint16_t*)w1;
+  p.q_stride_e = w1_stride_e;
+  p.q_stride_row = w1_stride_row;
+  p.off = off;
+  p.tm = tm;
+  p.N = 2 * I;
+  p.Kdim = H;
+  p.n_tiles = (int)ceil_div(2 * I, C::BN);
+  p.out0 = (uint16_t*)z;
+  p.out0_stride = 2 * I;
+  p.out1 = (uint16_t*)y1;
+  p.out1_stride = I;
+  return launch_varlen_m<C, ROLE_UP_FWD>(p, TK, E, st);
+}
+
+extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
+                                            void* y2, const int32_t* off, int64_t TK, int H, int I, int E,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "down_projection_forward");
+  if (rc) return rc;
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(y1 && w2 && y2 && off, SMOE_ERR_INVALID, "down_projection_forward: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  using C = CfgKM;
+  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
+  rc = launch_build_tile_map(off, E, C::BM, tm, st);
+  if (rc) return rc;
+  VarlenMParams p = {};
+  p.P = (const uint16_t*)y1;
+  p.p_stride = I;
+  p.Q = (const uint16_t*)w2;
+  p.q_stride_e = w2_stride_e;
+  p.q_stride_row = w2_stride_row;
+  p.off = off;
+  p.tm = tm;
+  p.N = H;
+  p.Kdim = I;
+  p.n_tiles = (int)ceil_div(H, C::BN);
+  p.out0 = (uint16_t*)y2;
+  p.out0_stride = H;
+  return launch_varlen_m<C, ROLE_PLAIN>(p, TK, E, st);
+}
+
+// activation-gradient halves of the two backward operators; the weight-gradient halves live in gemm_varlen_k.hip
+namespace smoe {
+
+int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
+              void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
+              const int32_t* sidx, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st) {
+  using C = CfgMN;
+  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
+  int rc = launch_build_tile_map(off, E, C::BM, tm, st);
+  if (rc) return rc;
+  VarlenMParams p = {};
+  p.P = (const uint16_t*)dout;
+  p.p_stride = H;
+  p.gidx = gidx;
+  p.Q = (const uint16_t*)w2;  // W2[e] is (H, I): k = h rows, n = i contiguous
+  p.q_stride_e = w2_stride_e;
+  p.q_stride_row = w2_stride_row;
+  p.off = off;
+  p.tm = tm;
+  p.N = I;
+  p.Kdim = H;
+  p.n_tiles = (int)ceil_div(I, C::BN);
+  p.out0 = (uint16_t*)dz;
+  p.out0_stride = 2 * I;
+  p.out1 = (uint16_t*)y1s;
+  p.out1_stride = I;
+  p.zin = (const uint16_t*)z;
+  p.zin_stride = 2 * I;
+  p.scores = scores;
+  p.sidx = sidx;
+  p.ds_partial = ds_partial;
+  p.ds_cols = smoe_dz_partial_cols(I);
+  return launch_varlen_m<C, ROLE_DZ>(p, TK, E, st);
+}
+
+int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
+              const int32_t* off, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st) {
+  using C = CfgMN;
+  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
+  int rc = launch_build_tile_map(off, E, C::BM, tm, st);
+  if (rc) return rc;
+  VarlenMParams p = {};
+  p.P = (const uint16_t*)dz;
+  p.p_stride = 2 * I;
+  p.Q = (const uint16_t*)w1;  // W1[e] is (2I, H): k = j rows, n = h contiguous
+  p.q_stride_e = w1_stride_e;
+  p.q_stride_row = w1_stride_row;
+  p.off = off;
+  p.tm = tm;
+  p.N = H;
+  p.Kdim = 2 * I;
+  p.n_tiles = (int)ceil_div(H, C::BN);
+  p.out0 = (uint16_t*)dx_expanded;
+  p.out0_stride = H;
+  return launch_varlen_m<C, ROLE_PLAIN>(p, TK, E, st);
+}
+
+}  // namespace smoe

@@ -1,0 +1,297 @@
+"""Autograd layer of the MoE hot path (public entry points of sonicmoe/functional/__init__.py).
+
+    moe_TC_softmax_topk_layer      router GEMM -> top-K softmax -> routing metadata -> experts -> combine
+    moe_general_routing_inputs     same expert path for caller-supplied (score, token, expert) triples
+
+What is kept for the backward pass is x, z (the pre-activation) and the routing metadata; the gathered inputs, y1, y2
+and dx_expanded are transient.  y1 is rebuilt from z inside the dz kernel and the token rows are gathered again
+inside the weight-gradient kernels.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+from .. import _lib
+from ..count_cumsum import count_cumsum
+from ..enums import LIBRARY_NAME, ActivationType, is_glu
+from .backward import _down_projection_backward, _softmax_topk_bwd, _token_broadcast_backward, _up_projection_backward
+from .forward import _down_projection_forward, _router_forward, _softmax_topk_fwd, _up_projection_forward
+from .utils import enable_quack_gemm, is_using_quack_gemm
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# routing metadata (one stable counting sort on the device instead of argsort + bincount + index arithmetic)
+# ---------------------------------------------------------------------------------------------------------------
+
+
+@torch.library.custom_op(
+    f"{LIBRARY_NAME}::_routing_metadata",
+    mutates_args={"freq", "off", "x_gather_idx", "s_scatter_idx", "s_reverse_scatter_idx", "tok_off"},
+)
+def _routing_metadata(
+    expert_idx: torch.Tensor,
+    token_idx: torch.Tensor | None,
+    T: int,
+    K: int,
+    freq: torch.Tensor,
+    off: torch.Tensor,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    s_reverse_scatter_idx: torch.Tensor,
+    tok_off: torch.Tensor,
+) -> None:
+    _lib.require_device(expert_idx, token_idx, freq, off, x_gather_idx, s_scatter_idx, s_reverse_scatter_idx, tok_off)
+    assert expert_idx.dtype == torch.int32 and expert_idx.is_contiguous()
+    assert token_idx is None or (token_idx.dtype == torch.int32 and token_idx.is_contiguous())
+    TK, E = expert_idx.numel(), freq.numel()
+    L = _lib.lib()
+    ws_bytes = L.smoe_routing_metadata_workspace_bytes(TK, E)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=expert_idx.device)
+    rc = L.smoe_routing_metadata(
+        _lib.ptr(expert_idx),
+        _lib.ptr(token_idx),
+        TK,
+        T,
+        E,
+        K,
+        _lib.ptr(freq),
+        _lib.ptr(off),
+        _lib.ptr(x_gather_idx),
+        _lib.ptr(s_scatter_idx),
+        _lib.ptr(s_reverse_scatter_idx),
+        _lib.ptr(tok_off),
+        _lib.ptr(ws),
+        ws.numel(),
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_routing_metadata")
+
+
+@torch.no_grad()
+def _build_metadata(expert_idx: torch.Tensor, token_idx: torch.Tensor | None, T: int, E: int, K: int):
+    dev = expert_idx.device
+    TK = expert_idx.numel()
+    i32 = dict(dtype=torch.int32, device=dev)
+    freq = torch.empty(E, **i32)
+    off = torch.empty(E + 1, **i32)
+    gidx = torch.empty(TK, **i32)
+    sidx = torch.empty(TK, **i32)
+    ridx = torch.empty(TK, **i32)
+    tok_off = torch.empty(T + 1, **i32)
+    expert_idx = expert_idx.contiguous().to(torch.int32)
+    if token_idx is not None:
+        token_idx = token_idx.contiguous().to(torch.int32)
+    _routing_metadata(expert_idx, token_idx, T, K, freq, off, gidx, sidx, ridx, tok_off)
+    return freq, off, gidx, sidx, ridx, tok_off
+
+
+def TC_topk_router_metadata(topk_router_indices: torch.Tensor, expert_frequency_offset: torch.Tensor, K: int):
+    """Token-choice top-K metadata (interface of sonicmoe/functional/__init__.py:19-46).  `expert_frequency_offset` is
+    the (E,) inclusive cumsum the reference passes in; only its length is used, the offsets are recomputed together
+    with the sort.  Returns (expert_frequency_offset (E+1,), x_gather_idx, s_scatter_idx, s_reverse_scatter_idx,
+    num_activated_expert_per_token_offset); the order inside an expert is ascending flat slot (stable)."""
+    T = topk_router_indices.size(0)
+    E = expert_frequency_offset.numel()
+    _, off, gidx, sidx, ridx, tok_off = _build_metadata(topk_router_indices.reshape(-1), None, T, E, K)
+    return off, gidx, sidx, ridx, tok_off
+
+
+def general_routing_router_metadata(
+    router_scores_selected: torch.Tensor, sorted_selected_T: torch.Tensor, selected_E: torch.Tensor, T: int, E: int
+):
+    """Metadata for arbitrary (token, expert) pairs with tokens sorted ascending (interface of
+    sonicmoe/functional/__init__.py:49-82).  Returns (expert_frequency, expert_frequency_offset, x_gather_idx,
+    s_scatter_idx, s_reverse_scatter_idx, num_activated_expert_per_token_offset)."""
+    freq, off, gidx, sidx, ridx, tok_off = _build_metadata(selected_E, sorted_selected_T, T, E, 1)
+    return freq, off, gidx, sidx, ridx, tok_off
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# autograd functions
+# ---------------------------------------------------------------------------------------------------------------
+
+
+class TC_Softmax_Topk_Router_Function(torch.autograd.Function):
+    """(scores fp32 (T, K), indices int32 (T, K)) = softmax(top-K(logits)); backward scatters into a zero (T, E)."""
+
+    @staticmethod
+    def forward(ctx, router_logits: torch.Tensor, E: int, K: int):
+        T = router_logits.size(0)
+        scores = torch.empty(T, K, dtype=torch.float32, device=router_logits.device)
+        indices = torch.empty(T, K, dtype=torch.int32, device=router_logits.device)
+        _softmax_topk_fwd(router_logits, scores, indices, E, K)
+        ctx.save_for_backward(scores, indices)
+        ctx.E, ctx.K, ctx.logits_dtype = E, K, router_logits.dtype
+        ctx.mark_non_differentiable(indices)
+        return scores, indices
+
+    @staticmethod
+    def backward(ctx, dscores: torch.Tensor, _unused):
+        scores, indices = ctx.saved_tensors
+        dlogits = torch.zeros(scores.size(0), ctx.E, dtype=ctx.logits_dtype, device=scores.device)
+        _softmax_topk_bwd(dlogits, None, dscores, scores, indices, ctx.K)
+        return dlogits, None, None
+
+
+class _ExpertsFunction(torch.autograd.Function):
+    """o = combine(down(act(up(gather(x))))) over the routed (token, expert) pairs.
+
+    Differentiable inputs: x (T, H), w1 (2I, H, E) view, w2 (H, I, E) view, scores (flat, fp32).
+    """
+
+    @staticmethod
+    def forward(
+        ctx,
+        x,
+        w1,
+        w2,
+        scores_flat,
+        off,
+        gidx,
+        sidx,
+        ridx,
+        tok_off,
+        K_or_maxK: int,
+        is_varlen_K: bool,
+        activation_type: ActivationType,
+        stream_id: int,
+        inference: bool,
+    ):
+        T, H = x.shape
+        N1, _, E = w1.shape
+        glu = is_glu(activation_type)
+        I = N1 // 2 if glu else N1
+        TK = gidx.numel()
+        x = x.contiguous()
+        scores_flat = scores_flat.contiguous()
+
+        z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
+        y1 = torch.empty(TK, I, dtype=x.dtype, device=x.device)
+        _up_projection_forward(
+            x, w1, z, y1, None, off, None, gidx, stream_id, activation_type.value, glu, inference
+        )
+        y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
+        _down_projection_forward(w2, y1, y2, None, off, None, gidx, stream_id)
+        del y1
+        o = torch.empty(T, H, dtype=x.dtype, device=x.device)
+        _router_forward(y2, o, scores_flat, ridx, tok_off, K_or_maxK, H, is_varlen_K)
+        del y2
+
+        if not inference:
+            ctx.save_for_backward(x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
+        ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference)
+        return o
+
+    @staticmethod
+    def backward(ctx, dout):
+        K_or_maxK, is_varlen_K, activation_type, stream_id, inference = ctx.cfg
+        if inference:
+            raise RuntimeError("backward through an inference-mode MoE forward: z was not stored")
+        x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
+        T, H = x.shape
+        TK = gidx.numel()
+        glu = is_glu(activation_type)
+        dout = dout.contiguous()
+
+        dw2 = torch.empty_like(w2)  # keeps the (E, H, I)-contiguous layout of the parameter view
+        dz = torch.empty_like(z)
+        ds = torch.empty(TK, dtype=torch.float32, device=x.device)
+        _down_projection_backward(
+            dout, z, w2, dw2, dz, ds, None, None, scores_flat, off, None, gidx, sidx, stream_id, glu,
+            activation_type.value,
+        )
+        dw1 = torch.empty_like(w1)
+        dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
+        _up_projection_backward(x, w1, dx_expanded, dw1, dz, None, off, None, gidx, sidx, glu, stream_id)
+        del dz
+        dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
+        _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
+        return dx, dw1, dw2, ds, None, None, None, None, None, None, None, None, None, None
+
+
+def _check_bias(b1, b2):
+    assert (b1 is None) == (b2 is None), "b1 and b2 has to be None or not None at the same time!"
+    if b1 is not None:
+        raise NotImplementedError("expert biases are not implemented in the HIP backend")
+
+
+def _as_activation(activation_type) -> ActivationType:
+    return ActivationType(activation_type) if isinstance(activation_type, str) else activation_type
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# layer entry points
+# ---------------------------------------------------------------------------------------------------------------
+
+
+def moe_TC_softmax_topk_layer(
+    x: torch.Tensor,
+    router_w: torch.Tensor,
+    w1: torch.Tensor,
+    b1: torch.Tensor | None,
+    w2: torch.Tensor,
+    b2: torch.Tensor | None,
+    K: int,
+    stream_id: int,
+    activation_type: ActivationType | str = ActivationType.SWIGLU,
+    is_inference_mode_enabled: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Token-choice top-K MoE layer (interface of sonicmoe/functional/__init__.py:423-490).
+
+    x (T, H); router_w (E, H); w1 (2I, H, E) and w2 (H, I, E) are permuted views of the (E, out, in) parameters.
+    Returns (o (T, H), router_logits (T, E), expert_frequency (E,) int32).
+    """
+    _check_bias(b1, b2)
+    activation_type = _as_activation(activation_type)
+    T, E = x.size(0), router_w.size(0)
+    router_logits = F.linear(x, router_w)
+    topk_scores, topk_indices = TC_Softmax_Topk_Router_Function.apply(router_logits, E, K)
+    freq, off, gidx, sidx, ridx, tok_off = _build_metadata(topk_indices.view(-1), None, T, E, K)
+    o = _ExpertsFunction.apply(
+        x, w1, w2, topk_scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id,
+        is_inference_mode_enabled,
+    )
+    return o, router_logits, freq
+
+
+def moe_general_routing_inputs(
+    x: torch.Tensor,
+    router_scores: torch.Tensor,
+    token_indices: torch.Tensor,
+    expert_indices: torch.Tensor,
+    w1: torch.Tensor,
+    b1: torch.Tensor | None,
+    w2: torch.Tensor,
+    b2: torch.Tensor | None,
+    E: int,
+    stream_id: int,
+    activation_type: ActivationType,
+    is_inference_mode_enabled: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """MoE layer for arbitrary routing (interface of sonicmoe/functional/__init__.py:497-562): pair j sends token
+    token_indices[j] (SORTED ascending) to expert expert_indices[j] with weight router_scores[j].
+    Returns (o (T, H), expert_frequency (E,) int32); d(router_scores) comes back in the pairs' order."""
+    _check_bias(b1, b2)
+    activation_type = _as_activation(activation_type)
+    T = x.size(0)
+    E = w2.size(-1)
+    freq, off, gidx, sidx, ridx, tok_off = _build_metadata(expert_indices, token_indices, T, E, 1)
+    o = _ExpertsFunction.apply(
+        x, w1, w2, router_scores.float(), off, gidx, sidx, ridx, tok_off, E, True, activation_type, stream_id,
+        is_inference_mode_enabled,
+    )
+    return o, freq
+
+
+__all__ = [
+    "TC_Softmax_Topk_Router_Function",
+    "TC_topk_router_metadata",
+    "general_routing_router_metadata",
+    "count_cumsum",
+    "enable_quack_gemm",
+    "is_using_quack_gemm",
+    "moe_TC_softmax_topk_layer",
+    "moe_general_routing_inputs",
+]

@@ -1,0 +1,191 @@
+"""Backward operators `sonicmoe::*` (names, arguments and mutation contracts of sonicmoe/functional/backward.py)."""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
+from ..utils import expert_major_strides
+from .forward import _check_bf16, _gather_sum, _gemm_workspace
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_backward", mutates_args={"dw1", "dx_expanded", "db1"})
+def _up_projection_backward(
+    x: torch.Tensor,
+    w1: torch.Tensor,
+    dx_expanded: torch.Tensor,
+    dw1: torch.Tensor,
+    dz: torch.Tensor,
+    db1: torch.Tensor | None,
+    expert_frequency_offset: torch.Tensor,
+    expert_schedule_order: torch.Tensor | None,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    is_glu_activation: bool,
+    stream_id: int,
+) -> None:
+    """dw1[e] = sum_m dz[m]^T x[t_m] (zeros for empty experts), dx_expanded = dz W1[e]."""
+    if db1 is not None:
+        raise NotImplementedError("_up_projection_backward: bias is not implemented in the HIP path")
+    if expert_schedule_order is not None:
+        raise NotImplementedError("_up_projection_backward: expert_schedule_order is not supported")
+    if not is_glu_activation:
+        raise NotImplementedError("_up_projection_backward: only GLU activations are implemented in the HIP path")
+    _lib.require_device(x, w1, dx_expanded, dw1, dz, expert_frequency_offset, x_gather_idx)
+    _check_bf16(("x", x), ("w1", w1), ("dx_expanded", dx_expanded), ("dw1", dw1), ("dz", dz))
+    N1, H, E = w1.shape
+    I = N1 // 2
+    T, TK = x.size(0), dz.size(0)
+    assert x.is_contiguous() and dz.is_contiguous() and dx_expanded.is_contiguous()
+    w_se, w_sr = expert_major_strides(w1, "w1")
+    d_se, d_sr = expert_major_strides(dw1, "dw1")
+    ws = _gemm_workspace(TK, E, x.device)
+    rc = _lib.lib().smoe_up_projection_backward(
+        _lib.ptr(x),
+        _lib.ptr(w1),
+        w_se,
+        w_sr,
+        _lib.ptr(dz),
+        _lib.ptr(dw1),
+        d_se,
+        d_sr,
+        _lib.ptr(dx_expanded),
+        _lib.ptr(expert_frequency_offset),
+        _lib.ptr(x_gather_idx),
+        T,
+        TK,
+        H,
+        I,
+        E,
+        ACTIVATION_CODE[ActivationType.SWIGLU],
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_up_projection_backward")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_down_projection_backward", mutates_args={"dw2", "dz", "ds", "db2"})
+def _down_projection_backward(
+    dout: torch.Tensor,
+    z: torch.Tensor,
+    w2: torch.Tensor,
+    dw2: torch.Tensor,
+    dz: torch.Tensor,
+    ds: torch.Tensor,
+    b2: torch.Tensor | None,
+    db2: torch.Tensor | None,
+    topk_scores: torch.Tensor,
+    expert_frequency_offset: torch.Tensor,
+    expert_schedule_order: torch.Tensor | None,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    stream_id: int,
+    is_glu_activation: bool,
+    activation_type: str,
+) -> None:
+    """dz, ds (flat routing-slot order) and dw2 of the down projection + weighted combine; y1 is recomputed from z and
+    the dout rows are re-gathered, nothing of size (TK, H) is kept from the forward."""
+    if b2 is not None or db2 is not None:
+        raise NotImplementedError("_down_projection_backward: bias is not implemented in the HIP path")
+    if expert_schedule_order is not None:
+        raise NotImplementedError("_down_projection_backward: expert_schedule_order is not supported")
+    _lib.require_device(dout, z, w2, dw2, dz, ds, topk_scores, expert_frequency_offset, x_gather_idx, s_scatter_idx)
+    _check_bf16(("dout", dout), ("z", z), ("w2", w2), ("dw2", dw2), ("dz", dz))
+    H, I, E = w2.shape
+    T, TK = dout.size(0), x_gather_idx.size(0)
+    dout = dout.contiguous()
+    assert z.is_contiguous() and dz.is_contiguous() and ds.is_contiguous() and ds.dtype == torch.float32
+    assert topk_scores.dtype == torch.float32 and topk_scores.is_contiguous()
+    w_se, w_sr = expert_major_strides(w2, "w2")
+    d_se, d_sr = expert_major_strides(dw2, "dw2")
+    y1s = torch.empty(TK, I, dtype=z.dtype, device=z.device)
+    ncols = _lib.lib().smoe_dz_partial_cols(I)
+    ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
+    ws = _gemm_workspace(TK, E, z.device)
+    rc = _lib.lib().smoe_down_projection_backward(
+        _lib.ptr(dout),
+        _lib.ptr(z),
+        _lib.ptr(w2),
+        w_se,
+        w_sr,
+        _lib.ptr(dw2),
+        d_se,
+        d_sr,
+        _lib.ptr(dz),
+        _lib.ptr(y1s),
+        _lib.ptr(ds),
+        _lib.ptr(ds_partial),
+        _lib.ptr(topk_scores),
+        _lib.ptr(expert_frequency_offset),
+        _lib.ptr(x_gather_idx),
+        _lib.ptr(s_scatter_idx),
+        T,
+        TK,
+        H,
+        I,
+        E,
+        ACTIVATION_CODE[ActivationType(activation_type)],
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_down_projection_backward")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_token_broadcast_backward", mutates_args={"dx_reduced"})
+def _token_broadcast_backward(
+    dx_reduced: torch.Tensor,
+    dx_expanded: torch.Tensor,
+    s_reverse_scatter_idx: torch.Tensor,
+    num_activated_expert_per_token_offset: torch.Tensor,
+    varlen_K_max: int,
+    H: int,
+    is_varlen_K: bool,
+) -> None:
+    """dx_reduced[t] = sum over the token's routing slots j of dx_expanded[s_reverse_scatter_idx[j]]."""
+    _gather_sum(
+        dx_expanded,
+        dx_reduced,
+        None,
+        s_reverse_scatter_idx,
+        num_activated_expert_per_token_offset,
+        varlen_K_max,
+        H,
+        is_varlen_K,
+        "_token_broadcast_backward",
+    )
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_softmax_topk_bwd", mutates_args={"dlogits_full"})
+def _softmax_topk_bwd(
+    dlogits_full: torch.Tensor,
+    dlogits: Optional[torch.Tensor],
+    dtopk_score: torch.Tensor,
+    topk_router_score: torch.Tensor,
+    topk_router_indices: torch.Tensor,
+    K: int,
+) -> None:
+    """dlogits_full[t, idx[t,k]] = s_k (ds_k - sum_j ds_j s_j); the caller zero-fills dlogits_full."""
+    if dlogits is not None:
+        raise NotImplementedError("_softmax_topk_bwd: accumulating into an existing dlogits is not supported")
+    _lib.require_device(dlogits_full, dtopk_score, topk_router_score, topk_router_indices)
+    if dlogits_full.dtype not in _lib.DT_CODE:
+        raise NotImplementedError(f"_softmax_topk_bwd: unsupported dtype {dlogits_full.dtype}")
+    dtopk_score = dtopk_score.contiguous().float()
+    assert topk_router_score.is_contiguous() and topk_router_indices.is_contiguous() and dlogits_full.stride(1) == 1
+    rc = _lib.lib().smoe_softmax_topk_bwd(
+        _lib.ptr(dlogits_full),
+        _lib.DT_CODE[dlogits_full.dtype],
+        dlogits_full.stride(0),
+        _lib.ptr(dtopk_score),
+        _lib.ptr(topk_router_score),
+        _lib.ptr(topk_router_indices),
+        dtopk_score.size(0),
+        K,
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_softmax_topk_bwd")

@@ -1,0 +1,195 @@
+"""Forward operators `sonicmoe::*` (names, arguments and mutation contracts of sonicmoe/functional/forward.py).
+
+Every operator is an out-variant: the caller allocates the outputs, the operator fills them through the C ABI of
+libsonicmoe_hip.so on the given stream and returns None.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
+from ..utils import expert_major_strides
+
+
+def _gemm_workspace(TK: int, E: int, device) -> torch.Tensor:
+    n = _lib.lib().smoe_gemm_workspace_bytes(TK, E)
+    return torch.empty(max(n, 16), dtype=torch.uint8, device=device)
+
+
+def _check_bf16(*named):
+    for name, t in named:
+        if t is not None and t.dtype != torch.bfloat16:
+            raise NotImplementedError(f"{name}: the HIP grouped GEMMs take bfloat16 tensors, got {t.dtype}")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_topk_fwd", mutates_args={"values", "indices"})
+def _topk_fwd(
+    x: torch.Tensor, k: int, values: torch.Tensor, indices: torch.Tensor, require_softmax_fusion: bool = True
+) -> None:
+    """Row-wise top-k of x (M, N) -> values (M, k) fp32 (softmax over the winners if requested), indices (M, k) int32."""
+    _lib.require_device(x, values, indices)
+    if x.dtype not in _lib.DT_CODE:
+        raise NotImplementedError(f"_topk_fwd: unsupported logits dtype {x.dtype}")
+    assert values.dtype == torch.float32 and indices.dtype == torch.int32
+    assert values.is_contiguous() and indices.is_contiguous() and x.stride(1) == 1
+    M, N = x.shape
+    rc = _lib.lib().smoe_topk_softmax_fwd(
+        _lib.ptr(x),
+        _lib.DT_CODE[x.dtype],
+        M,
+        N,
+        k,
+        x.stride(0),
+        _lib.ptr(values),
+        _lib.ptr(indices),
+        1 if require_softmax_fusion else 0,
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_topk_fwd")
+
+
+@torch.library.custom_op(
+    f"{LIBRARY_NAME}::_softmax_topk_fwd", mutates_args={"topk_router_score", "topk_router_indices"}
+)
+def _softmax_topk_fwd(
+    router_logits: torch.Tensor, topk_router_score: torch.Tensor, topk_router_indices: torch.Tensor, E: int, K: int
+) -> None:
+    _topk_fwd(router_logits, K, topk_router_score, topk_router_indices, True)
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_forward", mutates_args={"z", "y1"})
+def _up_projection_forward(
+    x: torch.Tensor,
+    w1: torch.Tensor,
+    z: torch.Tensor | None,
+    y1: torch.Tensor,
+    b1: torch.Tensor | None,
+    expert_frequency_offset: torch.Tensor,
+    expert_schedule_order: torch.Tensor | None,
+    x_gather_idx: torch.Tensor,
+    stream_id: int,
+    activation_type: str,
+    is_glu_activation: bool,
+    is_inference_mode_enabled: bool = False,
+) -> None:
+    """z = gather(x) W1^T, y1 = act(z); w1 is the (2I, H, E) view of the (E, 2I, H) parameter."""
+    if b1 is not None:
+        raise NotImplementedError("_up_projection_forward: bias is not implemented in the HIP path")
+    if expert_schedule_order is not None:
+        raise NotImplementedError("_up_projection_forward: expert_schedule_order is not supported")
+    _lib.require_device(x, w1, y1, expert_frequency_offset, x_gather_idx)
+    _check_bf16(("x", x), ("w1", w1), ("z", z), ("y1", y1))
+    N1, H, E = w1.shape
+    I = N1 // 2 if is_glu_activation else N1
+    T, TK = x.size(0), y1.size(0)
+    assert x.is_contiguous() and y1.is_contiguous() and (z is None or z.is_contiguous())
+    s_e, s_row = expert_major_strides(w1, "w1")
+    ws = _gemm_workspace(TK, E, x.device)
+    rc = _lib.lib().smoe_up_projection_forward(
+        _lib.ptr(x),
+        _lib.ptr(w1),
+        s_e,
+        s_row,
+        None if is_inference_mode_enabled else _lib.ptr(z),
+        _lib.ptr(y1),
+        _lib.ptr(expert_frequency_offset),
+        _lib.ptr(x_gather_idx),
+        T,
+        TK,
+        H,
+        I,
+        E,
+        ACTIVATION_CODE[ActivationType(activation_type)],
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_up_projection_forward")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_down_projection_forward", mutates_args={"y2"})
+def _down_projection_forward(
+    w2: torch.Tensor,
+    y1: torch.Tensor,
+    y2: torch.Tensor,
+    b2: torch.Tensor | None,
+    expert_frequency_offset: torch.Tensor,
+    expert_schedule_order: torch.Tensor | None,
+    x_gather_idx: torch.Tensor,
+    stream_id: int,
+) -> None:
+    """y2 = y1 W2^T per expert; w2 is the (H, I, E) view of the (E, H, I) parameter."""
+    if b2 is not None:
+        raise NotImplementedError("_down_projection_forward: bias is not implemented in the HIP path")
+    if expert_schedule_order is not None:
+        raise NotImplementedError("_down_projection_forward: expert_schedule_order is not supported")
+    _lib.require_device(w2, y1, y2, expert_frequency_offset)
+    _check_bf16(("w2", w2), ("y1", y1), ("y2", y2))
+    H, I, E = w2.shape
+    TK = y1.size(0)
+    assert y1.is_contiguous() and y2.is_contiguous()
+    s_e, s_row = expert_major_strides(w2, "w2")
+    ws = _gemm_workspace(TK, E, y1.device)
+    rc = _lib.lib().smoe_down_projection_forward(
+        _lib.ptr(y1),
+        _lib.ptr(w2),
+        s_e,
+        s_row,
+        _lib.ptr(y2),
+        _lib.ptr(expert_frequency_offset),
+        TK,
+        H,
+        I,
+        E,
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_down_projection_forward")
+
+
+def _gather_sum(src, out, weights, ridx, tok_off, K, H, is_varlen_K, what):
+    _lib.require_device(src, out, weights, ridx, tok_off)
+    _check_bf16((what + ".src", src), (what + ".out", out))
+    assert src.is_contiguous() and out.is_contiguous() and ridx.dtype == torch.int32
+    if weights is not None:
+        assert weights.dtype == torch.float32 and weights.is_contiguous()
+    rc = _lib.lib().smoe_gather_sum(
+        _lib.ptr(src),
+        _lib.ptr(out),
+        _lib.ptr(weights),
+        _lib.ptr(ridx),
+        _lib.ptr(tok_off) if is_varlen_K else None,
+        out.size(0),
+        K,
+        H,
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, what)
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_router_forward", mutates_args={"o"})
+def _router_forward(
+    y2: torch.Tensor,
+    o: torch.Tensor,
+    topk_scores: torch.Tensor,
+    s_reverse_scatter_idx: torch.Tensor,
+    num_activated_expert_per_token_offset: torch.Tensor,
+    varlen_K_max: int,
+    H: int,
+    is_varlen_K: bool,
+) -> None:
+    """o[t] = sum over the token's routing slots j of topk_scores[j] * y2[s_reverse_scatter_idx[j]]."""
+    _gather_sum(
+        y2,
+        o,
+        topk_scores,
+        s_reverse_scatter_idx,
+        num_activated_expert_per_token_offset,
+        varlen_K_max,
+        H,
+        is_varlen_K,
+        "_router_forward",
+    )

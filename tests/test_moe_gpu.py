@@ -1,0 +1,129 @@
+"""GPU parity of the whole layer (module API, forward + all gradients) against the restated torch backend.
+
+The oracle is evaluated in fp32 on the same bf16-rounded inputs and parameters (what the reference's own test does
+under autocast(float32), tests/moe_test.py:87-118) and is driven with the HIP path's expert choice, because
+torch.topk's order among tied logits is unspecified.  Bar: relative L2 <= 1e-2 for the output and every gradient.
+"""
+
+import pytest
+import torch
+
+from helpers import rel_l2
+from oracle import moe_math as M
+from oracle import routing as R
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _build(dev, T, H, I, E, K, seed=42, x_scale=1.0):
+    from sonicmoe import MoE
+    from sonicmoe.enums import ActivationType
+
+    torch.manual_seed(seed)
+    moe = MoE(E, K, H, I, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():
+        moe.router.weight.normal_(0, 0.02)
+    x = (x_scale * torch.randn(T, H, device=dev)).to(torch.bfloat16).requires_grad_()
+    dy = (x_scale * torch.randn(T, H, device=dev)).to(torch.bfloat16)
+    return moe, x, dy
+
+
+@pytest.mark.parametrize(
+    "T,H,I,E,K",
+    [
+        (1024, 512, 256, 8, 2),     # C1 shape
+        (2048, 768, 256, 128, 8),   # reference test shapes (tests/moe_test.py:26-37) at T=2048
+        (2048, 1536, 512, 64, 4),
+        (2048, 4096, 1024, 32, 2),
+        (1024, 4096, 256, 256, 16),
+        (8192, 4096, 1024, 128, 8), # reference test shape at full T
+    ],
+)
+def test_moe_forward_backward(dev, T, H, I, E, K):
+    from sonicmoe import KernelBackendMoE
+
+    moe, x, dy = _build(dev, T, H, I, E, K)
+    out, aux = moe(x, kernel_backend_moe=KernelBackendMoE.sonicmoe)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_proj.weight]
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+
+    # routing: bit-exact against the oracle on the very logits the layer saw
+    with torch.no_grad():
+        logits = torch.nn.functional.linear(x, moe.router.weight)
+    s_ref, i_ref = R.topk_softmax(logits.float().cpu().numpy(), K)
+    sel = torch.from_numpy(i_ref).to(dev)
+
+    xr = x.detach().clone().requires_grad_()
+    pr = [p.detach().clone().requires_grad_() for p in params]
+    out_ref, logits_ref, freq_ref = M.moe_torch_backend(xr, pr[0], pr[1], pr[2], K, selected_experts=sel)
+    grads_ref = torch.autograd.grad(out_ref, [xr] + pr, grad_outputs=dy.float())
+
+    assert rel_l2(out, out_ref) < TOL
+    names = ["dx", "d_router_w", "d_w1", "d_w2"]
+    for n, g, gr in zip(names, grads, grads_ref):
+        assert g.shape == gr.shape
+        assert rel_l2(g, gr) < TOL, n
+    aux_ref = M.switch_aux_loss(logits, freq_ref)
+    assert abs(float(aux) - float(aux_ref)) < 1e-3 * abs(float(aux_ref))
+
+
+def test_inference_mode_matches_training_forward(dev):
+    from sonicmoe import KernelBackendMoE
+
+    moe, x, _ = _build(dev, 1024, 512, 256, 8, 2)
+    out_train, _ = moe(x, kernel_backend_moe=KernelBackendMoE.sonicmoe)
+    with torch.no_grad():
+        out_inf, _ = moe(x, kernel_backend_moe=KernelBackendMoE.sonicmoe, is_inference_mode=True)
+    assert torch.equal(out_train, out_inf)
+
+
+def test_torch_backend_of_module_matches_oracle(dev):
+    """The module's own torch backend (the CPU-runnable configuration) against the oracle restatement, fp32 on GPU."""
+    from sonicmoe import KernelBackendMoE, MoE
+    from sonicmoe.enums import ActivationType
+
+    torch.manual_seed(0)
+    moe = MoE(8, 2, 512, 256, ActivationType.SWIGLU, False, 0.02).to(dev)
+    x = torch.randn(1024, 512, device=dev)
+    out, _ = moe(x, kernel_backend_moe=KernelBackendMoE.torch)
+    out_ref, _, _ = M.moe_torch_backend(x, moe.router.weight, moe.c_fc.weight, moe.c_proj.weight, 2)
+    assert rel_l2(out, out_ref) < 1e-5
+
+
+def test_general_routing_layer(dev):
+    """moe_general_routing_inputs against the per-expert masked loop of the reference's benchmark."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import moe_general_routing_inputs
+    from helpers import make_weights
+
+    T, H, I, E = 1024, 512, 256, 16
+    _, w1, w2 = make_weights(E, H, I, dev, seed=3)
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    # ragged: token t gets (t % 5) experts, so some tokens get none
+    tok, exp = [], []
+    for t in range(T):
+        k = t % 5
+        if k:
+            tok += [t] * k
+            exp += torch.randperm(E, generator=g)[:k].tolist()
+    tok = torch.tensor(tok, dtype=torch.int32, device=dev)
+    exp = torch.tensor(exp, dtype=torch.int32, device=dev)
+    scores = torch.rand(tok.numel(), generator=g).to(dev).requires_grad_()
+    w1p, w2p = w1.requires_grad_(), w2.requires_grad_()
+    o, freq = moe_general_routing_inputs(x, scores, tok, exp, w1p.permute(1, 2, 0), None, w2p.permute(1, 2, 0), None, E,
+                                         torch.cuda.current_stream().cuda_stream, ActivationType.SWIGLU, False)
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    grads = torch.autograd.grad(o, [x, scores, w1p, w2p], grad_outputs=dy)
+
+    xr, sr = x.detach().clone().requires_grad_(), scores.detach().clone().requires_grad_()
+    w1r, w2r = w1.detach().clone().requires_grad_(), w2.detach().clone().requires_grad_()
+    o_ref = M.general_routing_reference(xr, sr, tok, exp, w1r, w2r, E)
+    grads_ref = torch.autograd.grad(o_ref, [xr, sr, w1r, w2r], grad_outputs=dy.float())
+    assert torch.equal(freq.cpu(), torch.bincount(exp.long().cpu(), minlength=E).int())
+    assert rel_l2(o, o_ref) < TOL
+    for n, a, b in zip(["dx", "dscores", "dw1", "dw2"], grads, grads_ref):
+        assert rel_l2(a, b) < TOL, n
+    # tokens without any expert get exactly zero
+    assert bool((o[::5] == 0).all())
