@@ -1,0 +1,281 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE-layer hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config C2|C3] [--no-cpu-baseline]
+
+One "step" is one forward + backward pass of the whole layer (router GEMM, top-K softmax, routing metadata, the two
+forward grouped GEMMs, combine, the four backward grouped GEMMs, dx reduction, router backward) on seeded synthetic
+inputs that are resident in HBM before the timed region.  FLOPs are counted as the reference's benchmark does
+(benchmarks/moe-cute.py:231-232, :297-298): 18 * T*K * I * H for forward + backward with a gated activation; the
+router GEMM and the routing kernels are in the time but not in the FLOPs.
+
+Prints ONE JSON line on stdout; a per-kernel breakdown goes to stderr.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT / "sonic-moe_amd"))
+sys.path.insert(0, str(ROOT))
+
+import torch  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+CONFIGS = {
+    "C2": dict(T=32768, H=4096, I=1024, E=128, K=8, zipf=False),
+    "C3": dict(T=32768, H=4096, I=1536, E=128, K=8, zipf=True),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_inputs(cfg, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    T, H, I, E = cfg["T"], cfg["H"], cfg["I"], cfg["E"]
+    bf = torch.bfloat16
+    x = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(bf).requires_grad_()
+    wr = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(bf).requires_grad_()
+    w1 = (0.02 * torch.randn(E, 2 * I, H, generator=g, device=dev)).to(bf).requires_grad_()
+    w2 = (0.02 * torch.randn(E, H, I, generator=g, device=dev)).to(bf).requires_grad_()
+    dout = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(bf)
+    return x, wr, w1, w2, dout
+
+
+def time_region(fn, steps, warmup):
+    """ms per call: `warmup` untimed calls, then `steps` calls between two events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return e0.elapsed_time(e1) / steps, wall
+
+
+def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps):
+    """Time every operator of the path on its own (events on the launch stream) and return a list of dicts with
+    algorithmic FLOPs / bytes.  The grouped GEMM ops launch a tile-map builder (~5 us) next to the GEMM kernel."""
+    from sonicmoe.functional import _build_metadata, backward, forward
+
+    T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    TK = T * K
+    dev = x.device
+    bf = torch.bfloat16
+    stream = torch.cuda.current_stream().cuda_stream
+    with torch.no_grad():
+        logits = torch.nn.functional.linear(x, wr)
+        if cfg["zipf"]:
+            logits = logits + zipf_bias(E, dev).to(logits.dtype)
+        scores = torch.empty(T, K, dtype=torch.float32, device=dev)
+        idx = torch.empty(T, K, dtype=torch.int32, device=dev)
+        forward._topk_fwd(logits, K, scores, idx, True)
+        freq, off, gidx, sidx, ridx, tok_off = _build_metadata(idx.view(-1), None, T, E, K)
+        z = torch.empty(TK, 2 * I, dtype=bf, device=dev)
+        y1 = torch.empty(TK, I, dtype=bf, device=dev)
+        y2 = torch.empty(TK, H, dtype=bf, device=dev)
+        o = torch.empty(T, H, dtype=bf, device=dev)
+        dz = torch.empty_like(z)
+        ds = torch.empty(TK, dtype=torch.float32, device=dev)
+        dw1 = torch.empty_like(w1).permute(1, 2, 0)
+        dw2 = torch.empty_like(w2).permute(1, 2, 0)
+        dxe = torch.empty(TK, H, dtype=bf, device=dev)
+        dx = torch.empty(T, H, dtype=bf, device=dev)
+        dlog = torch.zeros(T, E, dtype=bf, device=dev)
+        w1v, w2v = w1.detach().permute(1, 2, 0), w2.detach().permute(1, 2, 0)
+        xd = x.detach()
+        sflat = scores.view(-1)
+        gemm = 2.0 * TK * I * H
+        ops = [
+            ("router_gemm(hipBLASLt)", lambda: torch.nn.functional.linear(xd, wr.detach()), 2.0 * T * H * E, None),
+            ("topk_softmax", lambda: forward._topk_fwd(logits, K, scores, idx, True), None, T * E * 2 + T * K * 8),
+            ("routing_metadata", lambda: _build_metadata(idx.view(-1), None, T, E, K), None, TK * 4 * 4),
+            ("up_projection_forward", lambda: forward._up_projection_forward(xd, w1v, z, y1, None, off, None, gidx, stream, "swiglu", True, False), 2 * gemm, None),
+            ("down_projection_forward", lambda: forward._down_projection_forward(w2v, y1, y2, None, off, None, gidx, stream), gemm, None),
+            ("router_forward(combine)", lambda: forward._router_forward(y2, o, sflat, ridx, tok_off, K, H, False), None, TK * H * 2 + T * H * 2 + TK * 8),
+            ("down_projection_backward(dz+dW2)", lambda: backward._down_projection_backward(dout, z, w2v, dw2, dz, ds, None, None, sflat, off, None, gidx, sidx, stream, True, "swiglu"), 2 * gemm, None),
+            ("up_projection_backward(dW1+dx)", lambda: backward._up_projection_backward(xd, w1v, dxe, dw1, dz, None, off, None, gidx, sidx, True, stream), 4 * gemm, None),
+            ("token_broadcast_backward", lambda: backward._token_broadcast_backward(dx, dxe, ridx, tok_off, K, H, False), None, TK * H * 2 + T * H * 2 + TK * 4),
+            ("softmax_topk_bwd", lambda: backward._softmax_topk_bwd(dlog, None, ds.view(T, K), scores, idx, K), None, T * K * 12 + T * E * 2),
+        ]
+        rows = []
+        for name, fn, flops, nbytes in ops:
+            ms, _ = time_region(fn, steps, 2)
+            row = dict(op=name, ms=round(ms, 4))
+            if flops:
+                row["tflops"] = round(flops / ms / 1e9, 1)
+                row["frac_mfma_peak"] = round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)
+                row["flops"] = flops
+            if nbytes:
+                row["gbs"] = round(nbytes / ms / 1e6, 1)
+                row["frac_hbm_peak"] = round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)
+            rows.append(row)
+            log(f"  {name:36s} {ms:9.4f} ms" + (f"  {row['tflops']:8.1f} TFLOP/s ({100*row['frac_mfma_peak']:.1f}% peak)" if flops else "")
+                + (f"  {row['gbs']:8.1f} GB/s ({100*row['frac_hbm_peak']:.1f}% HBM)" if nbytes else ""))
+    return rows
+
+
+def zipf_bias(E, dev):
+    e = torch.arange(E, device=dev, dtype=torch.float32)
+    return 2.0 * torch.log(1.0 / (e + 1.0))
+
+
+def cpu_baseline(cfg, budget_s=20.0):
+    """The oracle's restated torch backend (fp32, torch.autograd backward) on the host cores, on a bounded sample of the
+    same workload: same H, I, E, K, tokens scaled down so that one forward+backward pass takes seconds."""
+    from oracle import moe_math as M
+
+    H, I, E, K = cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    T = 2048
+    torch.manual_seed(0)
+    x = torch.randn(T, H, requires_grad=True)
+    wr = (0.02 * torch.randn(E, H)).requires_grad_()
+    w1 = (0.02 * torch.randn(E, 2 * I, H)).requires_grad_()
+    w2 = (0.02 * torch.randn(E, H, I)).requires_grad_()
+    dout = torch.randn(T, H)
+    flops = 18.0 * T * K * I * H
+
+    def step():
+        out, _, _ = M.moe_torch_backend(x, wr, w1, w2, K)
+        torch.autograd.grad(out, [x, wr, w1, w2], grad_outputs=dout)
+
+    step()  # warm-up (thread pool, allocator)
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < 5 and (time.perf_counter() - t_start) < budget_s:
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    best = sorted(times)[len(times) // 2]
+    return dict(
+        value=round(flops / best / 1e12, 4),
+        unit="TFLOP/s",
+        cores=torch.get_num_threads(),
+        kind="port",
+        sample=f"oracle.moe_torch_backend fp32 fwd+bwd, T={T} tokens (1/{cfg['T'] // T} of the workload's tokens), "
+        f"H={H} I={I} E={E} K={K}; median of {len(times)} passes, {best * 1e3:.0f} ms per pass",
+    )
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-breakdown", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import (
+        TC_Softmax_Topk_Router_Function,
+        _build_metadata,
+        _ExpertsFunction,
+        moe_TC_softmax_topk_layer,
+    )
+
+    cfg = CONFIGS[a.config]
+    dev = torch.device("cuda:0")
+    T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    x, wr, w1, w2, dout = make_inputs(cfg, dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    w1v, w2v = w1.permute(1, 2, 0), w2.permute(1, 2, 0)
+    bias = zipf_bias(E, dev).to(torch.bfloat16) if cfg["zipf"] else None
+
+    def layer():
+        if bias is None:
+            o, _, _ = moe_TC_softmax_topk_layer(x, wr, w1v, None, w2v, None, K, stream, ActivationType.SWIGLU, False)
+            return o
+        logits = torch.nn.functional.linear(x, wr) + bias
+        s, i = TC_Softmax_Topk_Router_Function.apply(logits, E, K)
+        _, off, gidx, sidx, ridx, tok_off = _build_metadata(i.view(-1), None, T, E, K)
+        return _ExpertsFunction.apply(x, w1v, w2v, s.view(-1), off, gidx, sidx, ridx, tok_off, K, False,
+                                      ActivationType.SWIGLU, stream, False)
+
+    def fwd_only():
+        with torch.no_grad():
+            layer()
+
+    def fwd_bwd():
+        o = layer()
+        torch.autograd.grad(o, [x, wr, w1, w2], grad_outputs=dout)
+
+    TK = T * K
+    flops_fwd, flops_all = 6.0 * TK * I * H, 18.0 * TK * I * H
+    fwd_ms, _ = time_region(fwd_only, a.steps, a.warmup)
+    ms, wall_ms = time_region(fwd_bwd, a.steps, a.warmup)
+    tflops = flops_all / ms / 1e9
+    log(f"{a.config}: fwd {fwd_ms:.3f} ms ({flops_fwd / fwd_ms / 1e9:.1f} TFLOP/s), fwd+bwd {ms:.3f} ms "
+        f"({tflops:.1f} TFLOP/s = {100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak), host wall {wall_ms:.3f} ms/step")
+
+    rows = [] if a.no_breakdown else kernel_breakdown(cfg, x, wr, w1, w2, dout, max(5, a.steps // 2))
+    gemm_rows = [r for r in rows if "flops" in r]
+    roofline = None
+    if gemm_rows:
+        dom = max(gemm_rows, key=lambda r: r["ms"])
+        roofline = dict(
+            bound="mfma",
+            kernel=dom["op"],
+            achieved=dom["tflops"],
+            peak=PEAK_BF16_TFLOPS,
+            unit="TFLOP/s",
+            frac=dom["frac_mfma_peak"],
+            traffic=None,
+        )
+
+    out = dict(
+        metric="MoE fwd+bwd TFLOP/s (% bf16 MFMA peak), T=32768 H=4096 I=1024 E=128 K=8",
+        value=round(tflops, 2),
+        unit="TFLOP/s",
+        n_gpus=1,
+        steps=a.steps,
+        warmup=a.warmup,
+        ms_per_step=round(ms, 4),
+        higher_is_better=True,
+        scaling="weak",
+        vs_baseline=None,
+        dtype="bf16",
+        data="synthetic",
+        config=dict(
+            workload=f"{a.config}: MoE layer fwd+bwd, T={T} H={H} I={I} E={E} K={K}, SwiGLU, no bias, token-choice softmax "
+            f"top-k router{' with Zipf logit bias' if cfg['zipf'] else ''}; x,dout~N(0,1), weights~N(0,0.02), seed 0",
+            flops_per_step=flops_all,
+        ),
+        frac_of_peak=round(tflops / PEAK_BF16_TFLOPS, 4),
+        fwd_ms=round(fwd_ms, 4),
+        fwd_tflops=round(flops_fwd / fwd_ms / 1e9, 2),
+        roofline=roofline,
+        kernels=[{k: v for k, v in r.items() if k != "flops"} for r in rows],
+    )
+    if not a.no_cpu_baseline:
+        del x, wr, w1, w2, dout
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(cfg)
+        log("cpu baseline:", out["cpu_baseline"])
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
