@@ -141,7 +141,7 @@ def cpu_baseline(cfg, budget_s=20.0):
     from oracle import moe_math as M
 
     H, I, E, K = cfg["H"], cfg["I"], cfg["E"], cfg["K"]
-    T = 2048
+    T = 1024
     torch.manual_seed(0)
     x = torch.randn(T, H, requires_grad=True)
     wr = (0.02 * torch.randn(E, H)).requires_grad_()

@@ -72,7 +72,8 @@ def moe_torch_backend(
     fan_in = sorted_scattered // K  # moe.py:342
     batch_gates = gates.flatten()[sorted_scattered]  # moe.py:345-346
     xs = xm[fan_in].split(freq.tolist(), dim=0)  # moe.py:348, :141
-    w1m, w2m = w1.to(math_dtype), w2.to(math_dtype)
+    # unbind (not w[e]) so that autograd stacks the per-expert weight gradients instead of adding E full-size tensors
+    w1m, w2m = w1.to(math_dtype).unbind(0), w2.to(math_dtype).unbind(0)
     outs = []
     for e in range(E):  # moe.py:145-148, :354-355
         h = F.linear(xs[e], w1m[e], None if b1 is None else b1[e].to(math_dtype))

@@ -1,14 +1,14 @@
 // Building blocks shared by the grouped GEMM kernels (gfx950, wave64, bf16 MFMA 32x32x16, fp32 accumulate).
 //
 // Vocabulary.  A GEMM tile multiplies a "P" operand (token side) with a "Q" operand (weight side) over a
-// contraction index k.  Both live in LDS as BK = 64 deep stages, filled by direct-to-LDS loads
+// contraction index k.  Both live in LDS as a ring of NSTAGE stages, BK = 32 deep each, filled by direct-to-LDS loads
 // (global_load_lds_dwordx4: every lane names its own 16 global bytes, the wavefront's 64 pieces land in 1024
 // consecutive LDS bytes), so the LDS position of a piece is fixed by (wave, instruction, lane) and swizzling is
 // done by choosing WHICH global piece a lane fetches.
 //
-//   K-major stage : [rows][64 k]   row = 128 B = 8 pieces; piece c of row r sits at c ^ kswz(r).
+//   K-major stage : [rows][32 k]   row = 64 B = 4 pieces; piece c of row r sits at c ^ kswz(r).
 //                   MFMA operand fragment = one ds_read_b128 per lane (row l%32, pieces 2*ks + l/32).
-//   MN-major stage: [64 k][cols]   row = cols*2 B; 32-byte group g of k-row k sits at g ^ (k & 15) (mod groups).
+//   MN-major stage: [32 k][cols]   row = cols*2 B; 32-byte group g of k-row k sits at g ^ (k & 15) (mod groups).
 //                   MFMA operand fragment = two ds_read_b64_tr_b16 per lane (the transpose load hands lane i of a
 //                   16-lane group column i of a 4 x 16 block whose rows are named by the lanes' addresses).
 //
@@ -22,16 +22,28 @@
 
 namespace smoe {
 
-constexpr int BK = 64;  // contraction depth of one LDS stage
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
-SMOE_DEV void load16_to_lds(const void* g, void* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
+// byte address inside the workgroup's LDS allocation of a generic pointer into __shared__ memory
+SMOE_DEV uint32_t lds_address(const void* p) { return (uint32_t)(uintptr_t)(lds_ptr_t)p; }
+
+// Direct-to-LDS load: every lane fetches its own 16 global bytes; the 64 pieces of the wavefront land in the 1024
+// LDS bytes starting at the wave-uniform address lds_wave_base (M0).  Issued through inline assembly on purpose:
+// when the compiler knows an instruction writes LDS from memory it protects every later LDS read with
+// s_waitcnt vmcnt(0), which would allow only one stage in flight.  The kernels wait by hand (wait_vmem_upto) for
+// exactly the stage they are about to read.
+SMOE_DEV void load16_to_lds(const void* g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(lds_wave_base) : "memory");
 }
 
-SMOE_DEV int kswz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+// piece swizzle of a K-major stage with BK_ of the contraction per row (BK_*2/16 pieces): chosen so that the 16 lanes
+// of a ds_read_b128 quarter-wave (16 consecutive rows, same piece) hit 16 different 16-byte bank groups
+template <int BK_>
+SMOE_DEV int kswz(int row) {
+  if constexpr (BK_ == 32) return (row >> 2) & 3;
+  else return (row & 7) ^ ((row >> 3) & 1);
+}
 
 SMOE_DEV bf16x8 lds_read_b128(const char* p) { return *(const bf16x8*)p; }
 
@@ -57,7 +69,132 @@ SMOE_DEV void static_for(F&& f) {
   static_for_impl<0, N>(f);
 }
 
-SMOE_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+// -DSMOE_PROBE_NO_MFMA / -DSMOE_PROBE_NO_REFILL build timing probes (wrong results) that remove the matrix
+// instructions resp. the steady-state global loads, to tell which side of the pipeline bounds a kernel.
+SMOE_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+#ifdef SMOE_PROBE_NO_MFMA
+  c[0] += (float)a[0] * (float)b[0];
+  return c;
+#else
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+#endif
+}
+
+// s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wave's vector-memory operations (oldest first) may still be
+// outstanding, and all of its LDS operations have completed
+template <int N>
+SMOE_DEV void wait_vmem_upto() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
+}
+SMOE_DEV void wait_vmem_all() { wait_vmem_upto<0>(); }
+
+// Workgroup barrier WITHOUT the memory fence of __syncthreads(): a fence would wait for every outstanding
+// direct-to-LDS load (vmcnt(0)) and collapse the ring to one stage in flight.  The waits that make LDS contents
+// visible are placed by hand (wait_vmem_upto before the barrier); the empty asm statements keep the compiler from
+// moving LDS accesses across the barrier.
+SMOE_DEV void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+// ---- software-pipelined main loop ------------------------------------------------------------------------------
+// LDS holds a ring of NSTAGE stages; a stage covers SLICES MFMA k-slices (16 each) of the contraction.  One stage is
+// consumed while up to NSTAGE-1 are in flight from L2/HBM.  Per stage:
+//   slices 0..SLICES-2: read the fragments of the next slice from LDS while the MFMAs of the current slice run;
+//   last slice: wait until this wave's pieces of the NEXT stage have landed (vmcnt leaves the younger stages in
+//            flight), workgroup barrier (everyone's pieces landed; everyone drained the current stage), refill the
+//            current stage's slot with stage s+NSTAGE, read slice 0 of the next stage while the last MFMAs run.
+//   issue(buf, s)                 start this wave's LPS direct-to-LDS loads of stage s into ring slot buf
+//   load(buf, s, ks, qf, pf)      read the fragments of slice ks of stage s from ring slot buf
+template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Issue, class Load>
+SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, Load&& load) {
+  if (S <= 0) return;
+  static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
+  static_assert(SLICES % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 6, "unsupported pipeline shape");
+  bf16x8 qf[2][NQ], pf[2][NP];
+  const int pre = S < NSTAGE ? S : NSTAGE;
+  for (int s = 0; s < pre; s++) issue(s, s);
+
+  auto wait_next_stage = [&](int younger) {  // `younger` stages were issued after the one we need
+    if constexpr (NSTAGE >= 6) if (younger >= 4) { wait_vmem_upto<4 * LPS>(); return; }
+    if constexpr (NSTAGE >= 5) if (younger == 3) { wait_vmem_upto<3 * LPS>(); return; }
+    if constexpr (NSTAGE >= 4) if (younger == 2) { wait_vmem_upto<2 * LPS>(); return; }
+    if constexpr (NSTAGE >= 3) if (younger == 1) { wait_vmem_upto<LPS>(); return; }
+    wait_vmem_all();
+  };
+  // the MFMAs of one slice; the LDS reads issued just before them (for the NEXT slice) are slotted in one per MFMA,
+  // starting after the first MFMA so that the wait in front of it covers only reads of the previous slice
+  auto slice_mfma = [&](auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+#pragma unroll
+    for (int q = 0; q < NQ; q++)
+#pragma unroll
+      for (int pp = 0; pp < NP; pp++) acc[q][pp] = mfma32(qf[cur][q], pf[cur][pp], acc[q][pp]);
+    constexpr int NM = NQ * NP, NR = NREADS < NM ? NREADS : NM - 1;
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  };
+  auto inner_slices = [&](int buf, int s) {
+    static_for<SLICES - 1>([&](auto ks_c) {
+      constexpr int ks = decltype(ks_c)::value;
+      load(buf, s, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
+      slice_mfma(std::integral_constant<int, (ks & 1)>{});
+    });
+  };
+
+  wait_next_stage(pre - 1);
+  lds_barrier();
+  load(0, 0, 0, qf[0], pf[0]);
+  int buf = 0;
+  for (int s = 0; s < S - 1; s++) {
+    inner_slices(buf, s);
+    const int younger = S - 2 - s < NSTAGE - 2 ? S - 2 - s : NSTAGE - 2;
+    wait_next_stage(younger);
+    lds_barrier();
+#ifndef SMOE_PROBE_NO_REFILL
+    if (s + NSTAGE < S) issue(buf, s + NSTAGE);
+#endif
+    buf = buf + 1 == NSTAGE ? 0 : buf + 1;
+    load(buf, s + 1, 0, qf[0], pf[0]);
+    slice_mfma(std::integral_constant<int, 1>{});
+  }
+  inner_slices(buf, S - 1);
+  slice_mfma(std::integral_constant<int, 1>{});
+}
+
+// ---- epilogue through LDS ----------------------------------------------------------------------------------------
+// A wavefront parks its TR x TC accumulator tile (lane = tile row l%32, register quad = 4 consecutive columns) as
+// bf16 in its own LDS region with padded rows, then reads it back row-contiguous and writes 16 bytes per lane.
+template <int TC>
+struct EpiLayout {
+  static constexpr int ROW_BYTES = TC * 2 + 16;  // +16: quads of different rows fall into different banks
+  static constexpr int LANES_PER_ROW = TC * 2 / 16;
+  static constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+};
+
+// store rows [0, TR) of the parked tile: global row = row_base + r (valid below row_limit), col = col_base + c
+template <int TR, int TC>
+SMOE_DEV void epilogue_flush(const char* region, int lane, uint16_t* out, int64_t out_stride, int row_base,
+                             int row_limit, int col_base, int col_limit) {
+  using L = EpiLayout<TC>;
+  const int rr = lane / L::LANES_PER_ROW, cc = lane % L::LANES_PER_ROW;
+#pragma unroll
+  for (int it = 0; it < TR / L::ROWS_PER_PASS; it++) {
+    const int r = it * L::ROWS_PER_PASS + rr;
+    const u32x4 v = *(const u32x4*)(region + r * L::ROW_BYTES + cc * 16);
+    const int row = row_base + r, col = col_base + cc * 8;
+    if (row < row_limit && col < col_limit) *(u32x4*)(out + (int64_t)row * out_stride + col) = v;
+  }
+}
+
+// 256 zero bytes: clamped (out-of-range) token rows of the weight-gradient GEMMs are fetched from here
+static __device__ __attribute__((aligned(256))) const uint32_t smoe_zero_page[64] = {};
 
 // ---- tile map ------------------------------------------------------------------------------------------------
 // Built on the device from the expert offsets; header[0] = number of token tiles.  Entry i = (expert, first row).

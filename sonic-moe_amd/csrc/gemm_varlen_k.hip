@@ -6,6 +6,8 @@
 // materialised gathered copy.  Experts without tokens still get their zeros written.
 //   dW1[e] (2I, H): R = dz rows,              S = x rows gathered
 //   dW2[e] (H, I) : R = dout rows gathered,   S = y1s rows
+#include <stdlib.h>
+
 #include "gemm_common.h"
 
 namespace smoe {
@@ -24,28 +26,31 @@ struct VarlenKParams {
   int E;
 };
 
-template <int BA_, int BB_, int WA_, int WB_, bool R_GATHER_, bool S_GATHER_>
+template <int BA_, int BB_, int WA_, int WB_, bool R_GATHER_, bool S_GATHER_, int BK_, int NSTAGE_>
 struct KCfg {
-  static constexpr int BA = BA_, BB = BB_, WA = WA_, WB = WB_;
+  static constexpr int BA = BA_, BB = BB_, WA = WA_, WB = WB_, BK = BK_, NSTAGE = NSTAGE_;
   static constexpr bool R_GATHER = R_GATHER_, S_GATHER = S_GATHER_;
   static constexpr int NW = WA * WB, NT = NW * 64;
   static constexpr int TA = BA / WA, TB = BB / WB;
   static constexpr int FA = TA / 32, FB = TB / 32;
   static constexpr int R_STAGE = BA * BK * 2, S_STAGE = BB * BK * 2;
   static constexpr int STAGE = R_STAGE + S_STAGE;
-  static constexpr int SMEM = 2 * STAGE;
+  static constexpr int EPI = NW * TA * (TB * 2 + 16);
+  static constexpr int SMEM = NSTAGE * STAGE > EPI ? NSTAGE * STAGE : EPI;
   static constexpr int R_ROWB = BA * 2, S_ROWB = BB * 2;
   static constexpr int R_LPR = R_ROWB / 16, S_LPR = S_ROWB / 16;
   static constexpr int R_RPI = 64 / R_LPR, S_RPI = 64 / S_LPR;
   static constexpr int R_INSTR = R_STAGE / 1024 / NW, S_INSTR = S_STAGE / 1024 / NW;
   static constexpr int R_SWM = (R_ROWB / 32 < 16 ? R_ROWB / 32 : 16) - 1;
   static constexpr int S_SWM = (S_ROWB / 32 < 16 ? S_ROWB / 32 : 16) - 1;
+  static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
 template <class C>
 __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int FA = C::FA, FB = C::FB;
+  constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
+  const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave % C::WA, wb = wave / C::WA;
@@ -59,10 +64,10 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   const int a0 = ta * C::BA, b0 = tb * C::BB;
   const int row_begin = p.off[e], row_end = p.off[e + 1];
   const int cnt = row_end - row_begin;
-  const int KT = (cnt + BK - 1) / BK;
+  const int S = (cnt + BK - 1) / BK;
 
-  // per-instruction k-row inside a stage and column offset (elements) of this lane's 16-byte piece
-  int r_kl[C::R_INSTR], r_col[C::R_INSTR], s_kl[C::S_INSTR], s_col[C::S_INSTR];
+  // per-instruction token row inside a stage and column offset (elements) of this lane's 16-byte piece
+  int r_col[C::R_INSTR], s_col[C::S_INSTR];
 #pragma unroll
   for (int i = 0; i < C::R_INSTR; i++) {
     const int kl = (wave * C::R_INSTR + i) * C::R_RPI + lane / C::R_LPR;
@@ -70,7 +75,6 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     const int log32 = (phys16 >> 1) ^ (kl & C::R_SWM);
     int a = a0 + ((log32 << 1) | (phys16 & 1)) * 8;
     a = a <= p.NA - 8 ? a : p.NA - 8;
-    r_kl[i] = kl;
     r_col[i] = a;
   }
 #pragma unroll
@@ -80,7 +84,6 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     const int log32 = (phys16 >> 1) ^ (kl & C::S_SWM);
     int b = b0 + ((log32 << 1) | (phys16 & 1)) * 8;
     b = b <= p.NB - 8 ? b : p.NB - 8;
-    s_kl[i] = kl;
     s_col[i] = b;
   }
 
@@ -117,102 +120,90 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[fb][fa][r] = 0.f;
 
-  // source row of token (row_begin + kt*64 + kl), clamped to the expert's last token
-  auto token_row = [&](int kt, int kl, bool gather) -> int64_t {
-    int m = row_begin + kt * BK + kl;
-    m = m < row_end ? m : row_end - 1;
-    return gather ? (int64_t)p.gidx[m] : (int64_t)m;
-  };
-
-  int64_t r_row[C::R_INSTR], s_row[C::S_INSTR];
-  auto fetch_rows = [&](int kt) {
+  // Token rows of a stage: wave w feeds rows [w*RPW, (w+1)*RPW) of each operand's stage, R_RPI resp. S_RPI rows per
+  // load instruction.  The gather indices of those rows are wave-uniform, so they are fetched with SCALAR loads:
+  // vector loads would share the in-order vmcnt counter with the direct-to-LDS loads and serialise the ring.
+  static_assert(C::R_INSTR * C::R_RPI == C::S_INSTR * C::S_RPI, "both operands cover the same token rows per wave");
+  constexpr int RPW = C::R_INSTR * C::R_RPI;  // token rows per wave and stage
+  const uint16_t* zero = (const uint16_t*)smoe_zero_page;
+  // constant address space: a uniform address then becomes a scalar load (the indices are read-only here)
+  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+  const const_i32_ptr gidx = (const_i32_ptr)p.gidx;
+  int tok[RPW];  // source row of token (stage base + wave*RPW + j); -1 past the expert's end
+  auto fetch = [&](int s) {
+    const int m0 = row_begin + s * BK + wave * RPW;
 #pragma unroll
-    for (int i = 0; i < C::R_INSTR; i++) r_row[i] = token_row(kt, r_kl[i], C::R_GATHER);
-#pragma unroll
-    for (int i = 0; i < C::S_INSTR; i++) s_row[i] = token_row(kt, s_kl[i], C::S_GATHER);
+    for (int j = 0; j < RPW; j++) {
+      const int m = m0 + j;
+      const int mc = m < row_end ? m : row_end - 1;
+      const int g = (C::R_GATHER || C::S_GATHER) ? gidx[mc] : mc;
+      tok[j] = m < row_end ? g : -1;
+    }
   };
-  auto issue = [&](int stage) {
-    char* base = smem + stage * C::STAGE;
+  // branch-free: pick this lane's token row among the RPI rows of instruction i, then its global address
+  auto piece = [&](const uint16_t* base, int64_t stride, bool gather, int rpi, int lpr, int s, int i, int col) {
+    const int sel = lane / lpr;
+    int t = tok[i * rpi];
+#pragma unroll
+    for (int j = 1; j < rpi; j++) t = sel == j ? tok[i * rpi + j] : t;
+    const int64_t row = gather ? (int64_t)t : (int64_t)(row_begin + s * BK + wave * RPW + i * rpi + sel);
+    const uint16_t* src = base + row * stride + col;
+    return t < 0 ? zero : src;
+  };
+  auto issue = [&](int buf, int s) {
+    const uint32_t base = smem_base + buf * C::STAGE;
 #pragma unroll
     for (int i = 0; i < C::R_INSTR; i++)
-      load16_to_lds(p.R + r_row[i] * p.r_stride + r_col[i], base + (wave * C::R_INSTR + i) * 1024);
+      load16_to_lds(piece(p.R, p.r_stride, C::R_GATHER, C::R_RPI, C::R_LPR, s, i, r_col[i]),
+                    base + (wave * C::R_INSTR + i) * 1024);
 #pragma unroll
     for (int i = 0; i < C::S_INSTR; i++)
-      load16_to_lds(p.S + s_row[i] * p.s_stride + s_col[i], base + C::R_STAGE + (wave * C::S_INSTR + i) * 1024);
+      load16_to_lds(piece(p.S, p.s_stride, C::S_GATHER, C::S_RPI, C::S_LPR, s, i, s_col[i]),
+                    base + C::R_STAGE + (wave * C::S_INSTR + i) * 1024);
+    if (s + 1 < S) fetch(s + 1);  // stages are issued in order: have the next one's rows ready
   };
+  auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
+    const char* st = smem + buf * C::STAGE;
+#pragma unroll
+    for (int f = 0; f < FA; f++)
+      rf[f] = lds_read_tr2(st + r_off[f * 2] + ks * 16 * C::R_ROWB, st + r_off[f * 2 + 1] + ks * 16 * C::R_ROWB);
+#pragma unroll
+    for (int f = 0; f < FB; f++)
+      sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
+  };
+  if (S > 0) fetch(0);
+  // MFMA as D[b][a] += S[b][k] R[k][a]: lane owns output row a = l%32, register quads hold 4 consecutive columns b
+  gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE>(S, acc, issue, load);
 
-  if (KT > 0) {
-    fetch_rows(0);
-    issue(0);
-    if (KT > 1) fetch_rows(1);
-  }
-  for (int kt = 0; kt < KT; kt++) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-    if (kt + 1 < KT) {
-      issue((kt + 1) & 1);
-      if (kt + 2 < KT) fetch_rows(kt + 2);
-    }
-    const char* st = smem + (kt & 1) * C::STAGE;
-    const int kvalid = cnt - kt * BK;  // tokens of this stage that exist (>= 64: all)
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      bf16x8 rf[FA], sf[FB];
-#pragma unroll
-      for (int f = 0; f < FA; f++)
-        rf[f] = lds_read_tr2(st + r_off[f * 2] + ks * 16 * C::R_ROWB, st + r_off[f * 2 + 1] + ks * 16 * C::R_ROWB);
-#pragma unroll
-      for (int f = 0; f < FB; f++)
-        sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
-      if (kvalid < BK) {  // ragged end of the expert: rows past it were clamped copies, remove them from one side
-        const int kbase = ks * 16 + 8 * (lane >> 5);
-#pragma unroll
-        for (int f = 0; f < FB; f++) {
-          u32x4 w = __builtin_bit_cast(u32x4, sf[f]);
-#pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const uint32_t keep = (kbase + 2 * q < kvalid ? 0x0000ffffu : 0u) | (kbase + 2 * q + 1 < kvalid ? 0xffff0000u : 0u);
-            w[q] &= keep;
-          }
-          sf[f] = __builtin_bit_cast(bf16x8, w);
-        }
-      }
-#pragma unroll
-      for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-        for (int fa = 0; fa < FA; fa++) acc[fb][fa] = mfma32(sf[fb], rf[fa], acc[fb][fa]);
-    }
-  }
-
-  // epilogue: lane owns output row a = l%32, four consecutive columns b per register quad
-  uint16_t* oe = p.out + (int64_t)e * p.out_stride_e;
-#pragma unroll
-  for (int fa = 0; fa < FA; fa++) {
-    const int a = a0 + wa * C::TA + fa * 32 + (lane & 31);
-    if (a >= p.NA) continue;
-#pragma unroll
-    for (int fb = 0; fb < FB; fb++) {
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        const int b = b0 + wb * C::TB + fb * 32 + 8 * rg + 4 * (lane >> 5);
-        if (b < p.NB) {
-          u32x2 v = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
-                     pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
-          *(u32x2*)(oe + (int64_t)a * p.out_stride_row + b) = v;
-        }
-      }
-    }
-  }
+  // epilogue through LDS (also writes the zeros of experts without tokens)
+  using L = EpiLayout<C::TB>;
+  char* region = smem + wave * (C::TA * L::ROW_BYTES);
+  wait_vmem_all();
+  lds_barrier();
+  static_for<FA>([&](auto fa_c) {
+    constexpr int fa = decltype(fa_c)::value;
+    static_for<FB * 4>([&](auto q_c) {
+      constexpr int fb = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+      u32x2 v = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
+                 pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
+      *(u32x2*)(region + (fa * 32 + (lane & 31)) * L::ROW_BYTES + (fb * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+    });
+  });
+  epilogue_flush<C::TA, C::TB>(region, lane, p.out + (int64_t)e * p.out_stride_e, p.out_stride_row, a0 + wa * C::TA,
+                               p.NA, b0 + wb * C::TB, p.NB);
 }
 
 template <class C>
-static int launch_varlen_k(const VarlenKParams& p, hipStream_t st) {
+static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   static bool attr_set = false;
   auto kern = varlen_k_kernel<C>;
   if (!attr_set) {
     SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
     attr_set = true;
   }
+  VarlenKParams p = pin;
+  p.tiles_a = (int)ceil_div(p.NA, C::BA);
+  p.tiles_b = (int)ceil_div(p.NB, C::BB);
   const int64_t total = (int64_t)p.tiles_a * p.tiles_b * p.E;
   const int64_t grid = ((total + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "weight-grad gemm: too many tiles");
@@ -221,8 +212,26 @@ static int launch_varlen_k(const VarlenKParams& p, hipStream_t st) {
   return SMOE_OK;
 }
 
-using KCfgDW1 = KCfg<256, 256, 2, 2, false, true>;
-using KCfgDW2 = KCfg<256, 256, 2, 2, true, false>;
+// SMOE_GEMM_VARIANT_K (environment, read once) picks the tile configuration of the varlen-K kernels; 3 = default.
+int gemm_variant_k() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("SMOE_GEMM_VARIANT_K");
+    v = e ? atoi(e) : 3;
+    if (v < 0 || v > 3) v = 3;
+  }
+  return v;
+}
+
+template <bool RG, bool SG>
+static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st) {
+  switch (gemm_variant_k()) {
+    case 0: return launch_varlen_k<KCfg<256, 256, 2, 2, RG, SG, 32, 5>>(p, st);   // 4 waves, BK 32, ring
+    case 1: return launch_varlen_k<KCfg<256, 256, 2, 2, RG, SG, 64, 2>>(p, st);   // 4 waves, BK 64, double buffer
+    case 2: return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 32, 5>>(p, st);   // 8 waves, BK 32, ring
+    default: return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 64, 2>>(p, st);  // 8 waves, BK 64, double buffer
+  }
+}
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
               void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
@@ -266,7 +275,6 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
     rc = launch_ds_finalize(ds_partial, smoe_dz_partial_cols(I), s_scatter_idx, ds, TK, st);
     if (rc) return rc;
   }
-  using C = KCfgDW2;
   VarlenKParams p = {};
   p.R = (const uint16_t*)dout;
   p.r_stride = H;
@@ -279,10 +287,8 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
   p.out_stride_row = dw2_stride_row;
   p.NA = H;
   p.NB = I;
-  p.tiles_a = (int)ceil_div(H, C::BA);
-  p.tiles_b = (int)ceil_div(I, C::BB);
   p.E = E;
-  return launch_varlen_k<C>(p, st);
+  return launch_varlen_k_variant<true, false>(p, st);
 }
 
 extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
@@ -300,7 +306,6 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
   (void)T;
   hipStream_t st = (hipStream_t)stream;
   {
-    using C = KCfgDW1;
     VarlenKParams p = {};
     p.R = (const uint16_t*)dz;
     p.r_stride = 2 * I;
@@ -313,10 +318,8 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     p.out_stride_row = dw1_stride_row;
     p.NA = 2 * I;
     p.NB = H;
-    p.tiles_a = (int)ceil_div(2 * I, C::BA);
-    p.tiles_b = (int)ceil_div(H, C::BB);
     p.E = E;
-    rc = launch_varlen_k<C>(p, st);
+    rc = launch_varlen_k_variant<false, true>(p, st);
     if (rc) return rc;
   }
   if (TK > 0) {

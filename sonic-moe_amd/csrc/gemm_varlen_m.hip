@@ -5,6 +5,8 @@
 //   down-projection forward  P = y1 rows,                          Q = W2[e] (K-major)   -> y2
 //   down-proj activation grad P = dout rows gathered,              Q = W2[e] (MN-major)  -> dz, y1s, ds partials
 //   up-proj activation grad  P = dz rows,                          Q = W1[e] (MN-major)  -> dx_expanded
+#include <stdlib.h>
+
 #include "gemm_common.h"
 
 namespace smoe {
@@ -32,32 +34,47 @@ struct VarlenMParams {
   int ds_cols;
 };
 
-template <int BM_, int BN_, int WM_, int WN_, bool QMN_>
+template <int BM_, int BN_, int WM_, int WN_, bool QMN_, int BK_, int NSTAGE_>
 struct Cfg {
-  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_;
+  static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, NSTAGE = NSTAGE_;
   static constexpr bool QMN = QMN_;
   static constexpr int NW = WM * WN, NT = NW * 64;
   static constexpr int TM = BM / WM, TN = BN / WN;
   static constexpr int FM = TM / 32, FN = TN / 32;
-  static constexpr int P_STAGE = BM * BK * 2, Q_STAGE = BN * BK * 2;
+  static constexpr int P_STAGE = BM * BK * 2, Q_STAGE = BN * BK * 2;  // bytes
   static constexpr int STAGE = P_STAGE + Q_STAGE;
-  static constexpr int P_INSTR = P_STAGE / 1024 / NW;
+  static constexpr int P_INSTR = P_STAGE / 1024 / NW;  // direct-to-LDS loads per wave and stage
   static constexpr int Q_INSTR = Q_STAGE / 1024 / NW;
-  static constexpr int SMEM = 2 * STAGE;
+  static constexpr int KROW = BK * 2;                   // bytes per row of a K-major stage
+  static constexpr int EPI = NW * TM * (TN * 2 + 16);   // per-wave parking regions of the LDS epilogue
+  static constexpr int SMEM = NSTAGE * STAGE > EPI ? NSTAGE * STAGE : EPI;
   // MN-major Q stage geometry
   static constexpr int ROWB = BN * 2;     // bytes per k-row
   static constexpr int LPR = ROWB / 16;   // lanes (16-byte pieces) per k-row
   static constexpr int RPI = 64 / LPR;    // k-rows per load instruction
+  static constexpr int KPR = KROW / 16;   // 16-byte pieces per row of a K-major stage
+  static constexpr int KRPI = 64 / KPR;   // rows per load instruction of a K-major stage
   static constexpr int NG = ROWB / 32;    // 32-byte groups per k-row
   static constexpr int SWM = (NG < 16 ? NG : 16) - 1;
   static_assert(P_INSTR >= 1 && Q_INSTR >= 1, "tile too small for the wave count");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA");
+  static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
+
+#ifdef SMOE_PROBE_TIMING
+// probe build only: per-tile shader-clock timestamps (start, pipeline primed, main loop done, end) of the first tiles
+__device__ unsigned long long g_probe_times[4096 * 4];
+#define SMOE_STAMP(i) \
+  if (lin < 4096 && tid == 0) g_probe_times[lin * 4 + (i)] = __builtin_amdgcn_s_memtime();
+#else
+#define SMOE_STAMP(i)
+#endif
 
 template <class C, int ROLE>
 __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int BN = C::BN, FM = C::FM, FN = C::FN;
+  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
+  const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % C::WM, wn = wave / C::WM;
@@ -71,6 +88,11 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   const int group = (int)(lin / per_group);
   const int first_m = group * GM;
   const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
+  SMOE_STAMP(0)
+#ifdef SMOE_PROBE_TIMING
+  if (lin < 4096 && tid == 0)
+    g_probe_times[lin * 4 + 1] = ((unsigned long long)__builtin_amdgcn_s_getreg(63508) << 32) | __builtin_amdgcn_s_getreg(63492);
+#endif
   const int within = (int)(lin - (int64_t)group * per_group);
   const int mt = first_m + within % gm;
   const int nt = within / gm;
@@ -83,11 +105,11 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   const uint16_t* p_src[C::P_INSTR];
 #pragma unroll
   for (int i = 0; i < C::P_INSTR; i++) {
-    const int r = (wave * C::P_INSTR + i) * 8 + (lane >> 3);
+    const int r = (wave * C::P_INSTR + i) * C::KRPI + lane / C::KPR;
     int m = row0 + r;
     m = m < row_end ? m : row_end - 1;
     const int64_t src_row = p.gidx ? (int64_t)p.gidx[m] : (int64_t)m;
-    p_src[i] = p.P + src_row * p.p_stride + (((lane & 7) ^ kswz(r)) << 3);
+    p_src[i] = p.P + src_row * p.p_stride + (((lane % C::KPR) ^ kswz<BK>(r)) << 3);
   }
   const uint16_t* q_src[C::Q_INSTR];
   const uint16_t* qe = p.Q + (int64_t)e * p.q_stride_e;
@@ -95,10 +117,10 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   if constexpr (!C::QMN) {
 #pragma unroll
     for (int i = 0; i < C::Q_INSTR; i++) {
-      const int r = (wave * C::Q_INSTR + i) * 8 + (lane >> 3);
+      const int r = (wave * C::Q_INSTR + i) * C::KRPI + lane / C::KPR;
       int n = n0 + r;
       n = n < p.N ? n : p.N - 1;
-      q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane & 7) ^ kswz(r)) << 3);
+      q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane % C::KPR) ^ kswz<BK>(r)) << 3);
     }
     q_step = BK;
   } else {
@@ -115,19 +137,19 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   }
 
   // ---- per-lane LDS fragment offsets (bytes inside a stage) ----
-  int p_off[4];
+  int p_off[SLICES];
   {
     const int row = wm * C::TM + (lane & 31);
-    const int sw = kswz(row);
+    const int sw = kswz<BK>(row);
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) p_off[ks] = row * 128 + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+    for (int ks = 0; ks < SLICES; ks++) p_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
   }
-  int q_off[C::QMN ? 2 * FN : 4];
+  int q_off[C::QMN ? 2 * FN : SLICES];
   if constexpr (!C::QMN) {
     const int row = wn * C::TN + (lane & 31);
-    const int sw = kswz(row);
+    const int sw = kswz<BK>(row);
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) q_off[ks] = C::P_STAGE + row * 128 + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = C::P_STAGE + row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
   } else {
     const int grp = lane >> 4, i16 = lane & 15;
     const int kk = 8 * (grp >> 1) + (i16 >> 2);
@@ -150,8 +172,8 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
 
-  auto issue = [&](int stage) {
-    char* base = smem + stage * C::STAGE;
+  auto issue = [&](int buf, int /*s*/) {
+    const uint32_t base = smem_base + buf * C::STAGE;
 #pragma unroll
     for (int i = 0; i < C::P_INSTR; i++) {
       load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
@@ -163,95 +185,107 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       q_src[i] += q_step;
     }
   };
-
-  const int KT = p.Kdim / BK;
-  issue(0);
-  for (int kt = 0; kt < KT; kt++) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces of stage kt have landed
-    __syncthreads();                     // everyone's pieces have landed; everyone is done reading the other stage
-    if (kt + 1 < KT) issue((kt + 1) & 1);
-    const char* st = smem + (kt & 1) * C::STAGE;
+  auto load = [&](int buf, int /*s*/, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
+#ifdef SMOE_PROBE_NO_LDSREAD
+    return;
+#endif
+    const char* st = smem + buf * C::STAGE;
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) {
-      bf16x8 pf[FM], qf[FN];
+    for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(st + p_off[ks] + fm * 32 * C::KROW);
 #pragma unroll
-      for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(st + p_off[ks] + fm * 32 * 128);
-#pragma unroll
-      for (int fn = 0; fn < FN; fn++) {
-        if constexpr (!C::QMN) {
-          qf[fn] = lds_read_b128(st + q_off[ks] + fn * 32 * 128);
-        } else {
-          qf[fn] = lds_read_tr2(st + q_off[fn * 2] + ks * 16 * C::ROWB, st + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
-        }
+    for (int fn = 0; fn < FN; fn++) {
+      if constexpr (!C::QMN) {
+        qf[fn] = lds_read_b128(st + q_off[ks] + fn * 32 * C::KROW);
+      } else {
+        qf[fn] = lds_read_tr2(st + q_off[fn * 2] + ks * 16 * C::ROWB, st + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
       }
-#pragma unroll
-      for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-        for (int fm = 0; fm < FM; fm++) acc[fn][fm] = mfma32(qf[fn], pf[fm], acc[fn][fm]);
     }
-  }
+  };
+  gemm_mainloop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR + C::Q_INSTR, SLICES, NSTAGE>(p.Kdim / BK, acc, issue,
+                                                                                            load);
 
-  // ---- epilogue: lane owns token column m = l%32 and 4 consecutive features per register quad ----
-  static_for<FM>([&](auto fm_c) {
-    constexpr int fm = decltype(fm_c)::value;
-    const int m = row0 + wm * C::TM + fm * 32 + (lane & 31);
-    const bool mvalid = m < row_end;
-    float s = 0.f, dsum = 0.f;
-    if constexpr (ROLE == ROLE_DZ) {
-      if (mvalid) s = p.scores[p.sidx[m]];
+  SMOE_STAMP(2)
+  const int m_base = row0 + wm * C::TM, n_base = n0 + wn * C::TN;
+#ifdef SMOE_PROBE_NO_EPILOGUE
+  if (acc[0][0][0] != 12345.f) return;
+#endif
+
+  if constexpr (ROLE == ROLE_PLAIN || ROLE == ROLE_UP_FWD) {
+    // ---- epilogue through LDS: every wave parks its tile in its own region, then stores 16 B per lane ----
+    using LZ = EpiLayout<C::TN>;
+    using LY = EpiLayout<C::TN / 2>;
+    char* region = smem + wave * (C::TM * LZ::ROW_BYTES);
+    wait_vmem_all();
+    lds_barrier();  // all waves are done reading the last stage
+    if (ROLE == ROLE_PLAIN || p.out0 != nullptr) {
+      static_for<FM>([&](auto fm_c) {
+        constexpr int fm = decltype(fm_c)::value;
+        static_for<FN * 4>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+          u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
+                     pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
+          *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+        });
+      });
+      epilogue_flush<C::TM, C::TN>(region, lane, p.out0, p.out0_stride, m_base, row_end, n_base, p.N);
     }
-    static_for<FN * 4>([&](auto q_c) {
-      constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-      const int n = n0 + wn * C::TN + fn * 32 + 8 * rg + 4 * (lane >> 5);
-      const bool ok = mvalid && n < p.N;
-      const float a0 = acc[fn][fm][4 * rg + 0], a1 = acc[fn][fm][4 * rg + 1], a2 = acc[fn][fm][4 * rg + 2],
-                  a3 = acc[fn][fm][4 * rg + 3];
-      if constexpr (ROLE == ROLE_PLAIN) {
-        if (ok) {
-          u32x2 v = {pack_bf16x2(a0, a1), pack_bf16x2(a2, a3)};
-          *(u32x2*)(p.out0 + (int64_t)m * p.out0_stride + n) = v;
-        }
-      } else if constexpr (ROLE == ROLE_UP_FWD) {
-        if (ok) {
-          if (p.out0) {
-            u32x2 v = {pack_bf16x2(a0, a1), pack_bf16x2(a2, a3)};
-            *(u32x2*)(p.out0 + (int64_t)m * p.out0_stride + n) = v;
-          }
-          const float y0 = a0 * fast_sigmoid(a0) * a1;
-          const float y1v = a2 * fast_sigmoid(a2) * a3;
-          *(uint32_t*)(p.out1 + (int64_t)m * p.out1_stride + (n >> 1)) = pack_bf16x2(y0, y1v);
-        }
-      } else {  // ROLE_DZ: n indexes the intermediate feature i; z holds (gate, up) pairs
-        if (ok) {
+    if constexpr (ROLE == ROLE_UP_FWD) {
+      static_for<FM>([&](auto fm_c) {
+        constexpr int fm = decltype(fm_c)::value;
+        static_for<FN * 4>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+          const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
+          const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
+          const uint32_t v = pack_bf16x2(g0 * fast_sigmoid(g0) * u0, g1 * fast_sigmoid(g1) * u1);
+          *(uint32_t*)(region + (fm * 32 + (lane & 31)) * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * (lane >> 5)) * 2) = v;
+        });
+      });
+      epilogue_flush<C::TM, C::TN / 2>(region, lane, p.out1, p.out1_stride, m_base, row_end, n_base / 2, p.N / 2);
+    }
+  } else {
+    // ---- dz epilogue: lane owns token column m = l%32 and 4 consecutive intermediate features per register quad ----
+    static_for<FM>([&](auto fm_c) {
+      constexpr int fm = decltype(fm_c)::value;
+      const int m = m_base + fm * 32 + (lane & 31);
+      const bool mvalid = m < row_end;
+      float s = 0.f, dsum = 0.f;
+      if (mvalid) s = p.scores[p.sidx[m]];
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        const int n = n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
+        if (mvalid && n < p.N) {
           const u32x4 zz = *(const u32x4*)(p.zin + (int64_t)m * p.zin_stride + 2 * n);
-          const float dy0[4] = {a0, a1, a2, a3};
           u32x4 dzv;
           float ys[4];
 #pragma unroll
           for (int q = 0; q < 4; q++) {
+            const float dy = acc[fn][fm][4 * rg + q];
             const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
             const float sig = fast_sigmoid(g);
             const float silu = g * sig;
             const float y1v = silu * u;
-            dsum += dy0[q] * y1v;
-            const float sd = s * dy0[q];
-            const float dg = sd * u * (silu * (1.f - sig) + sig);
-            const float du = sd * silu;
-            dzv[q] = pack_bf16x2(dg, du);
+            dsum += dy * y1v;
+            const float sd = s * dy;
+            dzv[q] = pack_bf16x2(sd * u * (silu * (1.f - sig) + sig), sd * silu);
             ys[q] = s * y1v;
           }
           *(u32x4*)(p.out0 + (int64_t)m * p.out0_stride + 2 * n) = dzv;
           u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
           *(u32x2*)(p.out1 + (int64_t)m * p.out1_stride + n) = yv;
         }
-      }
-    });
-    if constexpr (ROLE == ROLE_DZ) {
+      });
       dsum += __shfl_xor(dsum, 32, 64);
       if (mvalid && lane < 32) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
-    }
-  });
+    });
+  }
+  SMOE_STAMP(3)
 }
+
+#ifdef SMOE_PROBE_TIMING
+extern "C" int smoe_probe_read(void* dst, size_t bytes) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_probe_times), bytes);
+}
+#endif
 
 template <class C, int ROLE>
 static int launch_varlen_m(const VarlenMParams& p, int64_t TK, int E, hipStream_t st) {
@@ -270,8 +304,55 @@ static int launch_varlen_m(const VarlenMParams& p, int64_t TK, int E, hipStream_
 }
 
 // tile configurations ------------------------------------------------------------------------------------------
-using CfgKM = Cfg<256, 256, 2, 2, false>;   // K-major weights (forward GEMMs)
-using CfgMN = Cfg<256, 256, 2, 2, true>;    // MN-major weights (activation-gradient GEMMs)
+// SMOE_GEMM_VARIANT (environment, read once) picks the tile configuration of the varlen-M kernels; 3 is the default.
+template <bool QMN>
+using CfgV0 = Cfg<256, 256, 2, 2, QMN, 32, 5>;  // 4 waves, BK 32, 5-stage ring
+template <bool QMN>
+using CfgV1 = Cfg<256, 256, 2, 2, QMN, 64, 2>;  // 4 waves, BK 64, double buffer
+template <bool QMN>
+using CfgV2 = Cfg<256, 256, 2, 4, QMN, 32, 5>;  // 8 waves (2 per SIMD), BK 32, 5-stage ring
+template <bool QMN>
+using CfgV3 = Cfg<256, 256, 2, 4, QMN, 64, 2>;  // 8 waves, BK 64, double buffer
+template <bool QMN>
+using CfgV4 = Cfg<256, 256, 4, 2, QMN, 64, 2>;  // 8 waves, 4 along tokens
+
+int gemm_variant() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("SMOE_GEMM_VARIANT");
+    v = e ? atoi(e) : 3;
+    if (v < 0 || v > 4) v = 3;
+  }
+  return v;
+}
+
+template <bool QMN, int ROLE>
+static int launch_varlen_m_variant(VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E,
+                                   hipStream_t st) {
+  auto go = [&](auto cfg) {
+    using C = decltype(cfg);
+    p.tm = carve_tile_map(workspace, TK, E, C::BM);
+    int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
+    if (rc) return rc;
+    p.n_tiles = (int)ceil_div(p.N, C::BN);
+    if (ROLE == ROLE_DZ) p.ds_cols = p.n_tiles * C::WN;
+    return launch_varlen_m<C, ROLE>(p, TK, E, st);
+  };
+  switch (gemm_variant()) {
+    case 0: return go(CfgV0<QMN>{});
+    case 1: return go(CfgV1<QMN>{});
+    case 2: return go(CfgV2<QMN>{});
+    case 4: return go(CfgV4<QMN>{});
+    default: return go(CfgV3<QMN>{});
+  }
+}
+
+int dz_wave_cols() {
+  switch (gemm_variant()) {
+    case 0: case 1: case 4: return 2;
+    default: return 4;
+  }
+}
 
 }  // namespace smoe
 
@@ -292,7 +373,7 @@ extern "C" size_t smoe_gemm_workspace_bytes(int64_t TK, int E) {
   return tile_map_bytes(TK, E);
 }
 
-extern "C" int smoe_dz_partial_cols(int I) { return (int)ceil_div(I, CfgMN::BN) * CfgMN::WN; }
+extern "C" int smoe_dz_partial_cols(int I) { return (int)ceil_div(I, 256) * dz_wave_cols(); }
 
 extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
                                           void* z, void* y1, const int32_t* off, const int32_t* x_gather_idx,
@@ -306,10 +387,6 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
   SMOE_REQUIRE(x && w1 && y1 && off && x_gather_idx, SMOE_ERR_INVALID, "up_projection_forward: null pointer");
   SMOE_REQUIRE(T > 0, SMOE_ERR_INVALID, "up_projection_forward: T must be positive");
   hipStream_t st = (hipStream_t)stream;
-  using C = CfgKM;
-  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
-  rc = launch_build_tile_map(off, E, C::BM, tm, st);
-  if (rc) return rc;
   VarlenMParams p = {};
   p.P = (const uint16_t*)x;
   p.p_stride = H;
@@ -318,15 +395,13 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
   p.off = off;
-  p.tm = tm;
   p.N = 2 * I;
   p.Kdim = H;
-  p.n_tiles = (int)ceil_div(2 * I, C::BN);
   p.out0 = (uint16_t*)z;
   p.out0_stride = 2 * I;
   p.out1 = (uint16_t*)y1;
   p.out1_stride = I;
-  return launch_varlen_m<C, ROLE_UP_FWD>(p, TK, E, st);
+  return launch_varlen_m_variant<false, ROLE_UP_FWD>(p, off, workspace, TK, E, st);
 }
 
 extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
@@ -337,10 +412,6 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
   if (TK == 0) return SMOE_OK;
   SMOE_REQUIRE(y1 && w2 && y2 && off, SMOE_ERR_INVALID, "down_projection_forward: null pointer");
   hipStream_t st = (hipStream_t)stream;
-  using C = CfgKM;
-  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
-  rc = launch_build_tile_map(off, E, C::BM, tm, st);
-  if (rc) return rc;
   VarlenMParams p = {};
   p.P = (const uint16_t*)y1;
   p.p_stride = I;
@@ -348,13 +419,11 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
   p.q_stride_e = w2_stride_e;
   p.q_stride_row = w2_stride_row;
   p.off = off;
-  p.tm = tm;
   p.N = H;
   p.Kdim = I;
-  p.n_tiles = (int)ceil_div(H, C::BN);
   p.out0 = (uint16_t*)y2;
   p.out0_stride = H;
-  return launch_varlen_m<C, ROLE_PLAIN>(p, TK, E, st);
+  return launch_varlen_m_variant<false, ROLE_PLAIN>(p, off, workspace, TK, E, st);
 }
 
 // activation-gradient halves of the two backward operators; the weight-gradient halves live in gemm_varlen_k.hip
@@ -363,10 +432,6 @@ namespace smoe {
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
               void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
               const int32_t* sidx, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st) {
-  using C = CfgMN;
-  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
-  int rc = launch_build_tile_map(off, E, C::BM, tm, st);
-  if (rc) return rc;
   VarlenMParams p = {};
   p.P = (const uint16_t*)dout;
   p.p_stride = H;
@@ -375,10 +440,8 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.q_stride_e = w2_stride_e;
   p.q_stride_row = w2_stride_row;
   p.off = off;
-  p.tm = tm;
   p.N = I;
   p.Kdim = H;
-  p.n_tiles = (int)ceil_div(I, C::BN);
   p.out0 = (uint16_t*)dz;
   p.out0_stride = 2 * I;
   p.out1 = (uint16_t*)y1s;
@@ -388,16 +451,11 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.scores = scores;
   p.sidx = sidx;
   p.ds_partial = ds_partial;
-  p.ds_cols = smoe_dz_partial_cols(I);
-  return launch_varlen_m<C, ROLE_DZ>(p, TK, E, st);
+  return launch_varlen_m_variant<true, ROLE_DZ>(p, off, workspace, TK, E, st);
 }
 
 int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
               const int32_t* off, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st) {
-  using C = CfgMN;
-  TileMap tm = carve_tile_map(workspace, TK, E, C::BM);
-  int rc = launch_build_tile_map(off, E, C::BM, tm, st);
-  if (rc) return rc;
   VarlenMParams p = {};
   p.P = (const uint16_t*)dz;
   p.p_stride = 2 * I;
@@ -405,13 +463,11 @@ int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_st
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
   p.off = off;
-  p.tm = tm;
   p.N = H;
   p.Kdim = 2 * I;
-  p.n_tiles = (int)ceil_div(H, C::BN);
   p.out0 = (uint16_t*)dx_expanded;
   p.out0_stride = H;
-  return launch_varlen_m<C, ROLE_PLAIN>(p, TK, E, st);
+  return launch_varlen_m_variant<true, ROLE_PLAIN>(p, off, workspace, TK, E, st);
 }
 
 }  // namespace smoe

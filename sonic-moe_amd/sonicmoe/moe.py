@@ -64,9 +64,9 @@ class Experts(nn.Module):
 
     def torch_forward(self, chunks: list[torch.Tensor]) -> list[torch.Tensor]:
         """chunks[e] (n_e, in) -> (n_e, out) with expert e's map."""
-        return [
-            F.linear(c, self.weight[e], None if self.bias is None else self.bias[e]) for e, c in enumerate(chunks)
-        ]
+        weights = self.weight.unbind(0)  # one autograd node for all experts' weight gradients
+        biases = [None] * self.num_experts if self.bias is None else self.bias.unbind(0)
+        return [F.linear(c, w, b) for c, w, b in zip(chunks, weights, biases)]
 
     def extra_repr(self) -> str:
         return f"num_experts={self.num_experts}, in_features={self.in_features}, out_features={self.out_features}"
