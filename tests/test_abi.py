@@ -1,0 +1,74 @@
+"""The C-ABI library loads and exports every entry point that include/sonicmoe_hip.h declares; argument checks
+that happen before any GPU work report the documented status codes.  No compute is launched here."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "sonicmoe_hip.h"
+
+
+def declared_functions() -> list[str]:
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(smoe_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from sonicmoe import _lib
+
+    if not _lib.library_path().exists():
+        import __graft_entry__
+
+        __graft_entry__.build()
+    return _lib.lib()
+
+
+def test_header_and_binding_agree(lib):
+    from sonicmoe import _lib
+
+    names = declared_functions()
+    assert len(names) >= 14
+    assert sorted(_lib.exported_symbols()) == names
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_version_and_error_text(lib):
+    assert lib.smoe_version() >= 100
+    assert isinstance(lib.smoe_last_error(), bytes)
+
+
+def test_argument_checks_return_status_codes(lib):
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # E out of range -> SMOE_ERR_UNSUPPORTED (2), before anything is launched
+    assert lib.smoe_count_cumsum(p, 0, 4, 0, p, p, None) == 2
+    assert b"E=0" in lib.smoe_last_error()
+    # null output -> SMOE_ERR_INVALID (1)
+    assert lib.smoe_count_cumsum(p, 0, 4, 8, None, None, None) == 1
+    # K > E
+    assert lib.smoe_topk_softmax_fwd(p, 0, 4, 8, 9, 8, p, p, 1, None) == 2
+    # H not a multiple of 64
+    assert lib.smoe_up_projection_forward(p, p, 0, 0, p, p, p, p, 4, 8, 96, 64, 2, 0, p, 1 << 20, None) == 2
+    assert b"multiple of 64" in lib.smoe_last_error()
+    # workspace too small
+    assert lib.smoe_down_projection_forward(p, p, 0, 0, p, p, 1 << 20, 64, 64, 2, p, 8, None) == 4
+    # unsupported activation
+    assert lib.smoe_up_projection_forward(p, p, 0, 0, p, p, p, p, 4, 8, 64, 64, 2, 5, p, 1 << 20, None) == 2
+    # workspace size queries are pure host functions
+    assert lib.smoe_gemm_workspace_bytes(262144, 128) > 0
+    assert lib.smoe_routing_metadata_workspace_bytes(262144, 128) == 2 * 128 * 256 * 4
+    assert lib.smoe_dz_partial_cols(1024) >= 4
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from sonicmoe import _lib
+
+    monkeypatch.setenv("SONICMOE_HIP_LIB", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_lib, "_LIB", None)
+    with pytest.raises(RuntimeError, match="not found"):
+        _lib.lib()
