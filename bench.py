@@ -68,7 +68,7 @@ def time_region(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps, wall
 
 
-def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps):
+def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
     """Time every operator of the path on its own (events on the launch stream) and return a list of dicts with
     algorithmic FLOPs / bytes.  The grouped GEMM ops launch a tile-map builder (~5 us) next to the GEMM kernel."""
     from sonicmoe.functional import _build_metadata, backward, forward
@@ -108,13 +108,17 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps):
             ("up_projection_forward", lambda: forward._up_projection_forward(xd, w1v, z, y1, None, off, None, gidx, stream, "swiglu", True, False), 2 * gemm, None),
             ("down_projection_forward", lambda: forward._down_projection_forward(w2v, y1, y2, None, off, None, gidx, stream), gemm, None),
             ("router_forward(combine)", lambda: forward._router_forward(y2, o, sflat, ridx, tok_off, K, H, False), None, TK * H * 2 + T * H * 2 + TK * 8),
+            ("down_projection_backward(dz only)", lambda: backward._down_projection_backward(dout, z, w2v, None, dz, ds, None, None, sflat, off, None, gidx, sidx, stream, True, "swiglu"), gemm, None),
             ("down_projection_backward(dz+dW2)", lambda: backward._down_projection_backward(dout, z, w2v, dw2, dz, ds, None, None, sflat, off, None, gidx, sidx, stream, True, "swiglu"), 2 * gemm, None),
-            ("up_projection_backward(dW1+dx)", lambda: backward._up_projection_backward(xd, w1v, dxe, dw1, dz, None, off, None, gidx, sidx, True, stream), 4 * gemm, None),
+            ("up_projection_backward(dW1 only)", lambda: backward._up_projection_backward(xd, w1v, None, dw1, dz, None, off, None, gidx, sidx, True, stream), 2 * gemm, None),
+            ("up_projection_backward(dx only)", lambda: backward._up_projection_backward(xd, w1v, dxe, None, dz, None, off, None, gidx, sidx, True, stream), 2 * gemm, None),
             ("token_broadcast_backward", lambda: backward._token_broadcast_backward(dx, dxe, ridx, tok_off, K, H, False), None, TK * H * 2 + T * H * 2 + TK * 4),
             ("softmax_topk_bwd", lambda: backward._softmax_topk_bwd(dlog, None, ds.view(T, K), scores, idx, K), None, T * K * 12 + T * E * 2),
         ]
         rows = []
         for name, fn, flops, nbytes in ops:
+            if only is not None and name != only:
+                continue
             ms, _ = time_region(fn, steps, 2)
             row = dict(op=name, ms=round(ms, 4))
             if flops:
@@ -128,6 +132,44 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps):
             log(f"  {name:36s} {ms:9.4f} ms" + (f"  {row['tflops']:8.1f} TFLOP/s ({100*row['frac_mfma_peak']:.1f}% peak)" if flops else "")
                 + (f"  {row['gbs']:8.1f} GB/s ({100*row['frac_hbm_peak']:.1f}% HBM)" if nbytes else ""))
     return rows
+
+
+# operators that are one grouped-GEMM kernel launch (plus a ~5 us tile-map builder), and the kernel they launch
+SINGLE_KERNEL_OPS = {
+    "up_projection_forward": "varlen_m_kernel<up-projection forward>",
+    "down_projection_forward": "varlen_m_kernel<down-projection forward>",
+    "down_projection_backward(dz only)": "varlen_m_kernel<dz>",
+    "up_projection_backward(dW1 only)": "varlen_k_kernel<dW1>",
+    "up_projection_backward(dx only)": "varlen_m_kernel<dx_expanded>",
+}
+
+
+def recorded_traffic(kernel: str, config: str):
+    """HBM bytes per launch of `kernel`, measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE and calibrated against
+    a copy of known size; recorded in profiles/hbm_traffic.json (None if that kernel has no record)."""
+    f = ROOT / "profiles" / "hbm_traffic.json"
+    if not f.exists():
+        return None
+    try:
+        return json.loads(f.read_text()).get(config, {}).get(kernel)
+    except (ValueError, OSError):
+        return None
+
+
+def pmc_target(cfg, op_name, dev):
+    """Workload for the counter passes: 3 launches of one operator's kernel and one 1 GiB device-to-device copy whose
+    FETCH_SIZE / WRITE_SIZE readings calibrate the counters."""
+    x, wr, w1, w2, dout = make_inputs(cfg, dev)
+    a = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
+    b = torch.empty_like(a)
+    b.copy_(a)
+    torch.cuda.synchronize()
+    import contextlib, io
+
+    with contextlib.redirect_stderr(io.StringIO()):
+        rows = kernel_breakdown(cfg, x, wr, w1, w2, dout, 1, only=op_name)
+    torch.cuda.synchronize()
+    print(json.dumps(dict(pmc_target=op_name, copy_bytes=a.numel() * 4, rows=rows)))
 
 
 def zipf_bias(E, dev):
@@ -180,6 +222,8 @@ def main():
     ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--pmc-target", default=None, choices=sorted(SINGLE_KERNEL_OPS),
+                    help="run only this operator (3 launches) and a 1 GiB copy: the workload of the rocprofv3 --pmc passes")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -198,6 +242,9 @@ def main():
 
     cfg = CONFIGS[a.config]
     dev = torch.device("cuda:0")
+    if a.pmc_target:
+        pmc_target(cfg, a.pmc_target, dev)
+        return
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     x, wr, w1, w2, dout = make_inputs(cfg, dev)
     stream = torch.cuda.current_stream().cuda_stream
@@ -231,18 +278,21 @@ def main():
         f"({tflops:.1f} TFLOP/s = {100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak), host wall {wall_ms:.3f} ms/step")
 
     rows = [] if a.no_breakdown else kernel_breakdown(cfg, x, wr, w1, w2, dout, max(5, a.steps // 2))
-    gemm_rows = [r for r in rows if "flops" in r]
+    # dominant kernel = the single grouped-GEMM launch with the largest average duration
+    single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS]
     roofline = None
-    if gemm_rows:
-        dom = max(gemm_rows, key=lambda r: r["ms"])
+    if single:
+        dom = max(single, key=lambda r: r["ms"])
         roofline = dict(
             bound="mfma",
-            kernel=dom["op"],
+            kernel=SINGLE_KERNEL_OPS[dom["op"]],
+            op=dom["op"],
+            avg_launch_ms=dom["ms"],
             achieved=dom["tflops"],
             peak=PEAK_BF16_TFLOPS,
             unit="TFLOP/s",
             frac=dom["frac_mfma_peak"],
-            traffic=None,
+            traffic=recorded_traffic(SINGLE_KERNEL_OPS[dom["op"]], a.config),
         )
 
     out = dict(

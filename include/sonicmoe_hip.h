@@ -127,7 +127,9 @@ int smoe_gather_sum(const void* src, void* out, const float* w, const int32_t* r
  *   dy1 = dout[x_gather_idx] W2[e] (never stored); with (g,u) = z pairs and s = scores[s_scatter_idx[m]]:
  *   dz (TK, 2I), y1s = s*silu(g)*u (TK, I), ds[s_scatter_idx[m]] = sum_i dy1*y1 (fp32, flat-slot order),
  *   dw2 (E, H, I) = sum_m dout[t_m]^T (x) y1s[m]  (zeros for empty experts).
- *   ds_partial: fp32 scratch of TK * smoe_dz_partial_cols(I) elements. */
+ *   ds_partial: fp32 scratch of TK * smoe_dz_partial_cols(I) elements.
+ *   dw2 == NULL skips the weight gradient; dz == NULL skips the activation gradient (y1s must then hold the values a
+ *   previous call produced). */
 int smoe_dz_partial_cols(int I);
 int smoe_down_projection_backward(const void* dout, const void* z, const void* w2, int64_t w2_stride_e,
                                   int64_t w2_stride_row, void* dw2, int64_t dw2_stride_e, int64_t dw2_stride_row,
@@ -137,7 +139,8 @@ int smoe_down_projection_backward(const void* dout, const void* z, const void* w
                                   size_t workspace_bytes, void* stream);
 
 /* dW1[e] = sum_m dz[m]^T (x) x[t_m];  dx_expanded[m] = dz[m] W1[e].
- * Replaces sonicmoe::_up_projection_backward (sonicmoe/functional/backward.py:195-283). */
+ * Replaces sonicmoe::_up_projection_backward (sonicmoe/functional/backward.py:195-283).
+ *   dw1 == NULL or dx_expanded == NULL skips that output (frozen weights / no input gradient). */
 int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
                                 const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row,
                                 void* dx_expanded, const int32_t* off, const int32_t* x_gather_idx, int64_t T,

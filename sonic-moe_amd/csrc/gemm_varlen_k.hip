@@ -263,18 +263,21 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
   if (rc) return rc;
   SMOE_REQUIRE(activation == SMOE_ACT_SWIGLU, SMOE_ERR_UNSUPPORTED,
                "down_projection_backward: only SwiGLU is implemented (activation=%d)", activation);
-  SMOE_REQUIRE(dw2 && off, SMOE_ERR_INVALID, "down_projection_backward: null pointer");
-  SMOE_REQUIRE(TK == 0 || (dout && z && w2 && dz && y1s && ds && ds_partial && scores && x_gather_idx && s_scatter_idx),
-               SMOE_ERR_INVALID, "down_projection_backward: null pointer");
+  SMOE_REQUIRE(off, SMOE_ERR_INVALID, "down_projection_backward: null pointer");
+  SMOE_REQUIRE(dz || dw2, SMOE_ERR_INVALID, "down_projection_backward: nothing to compute (dz and dw2 are both null)");
+  SMOE_REQUIRE(TK == 0 || (dout && y1s && x_gather_idx), SMOE_ERR_INVALID, "down_projection_backward: null pointer");
+  SMOE_REQUIRE(TK == 0 || !dz || (z && w2 && ds && ds_partial && scores && s_scatter_idx), SMOE_ERR_INVALID,
+               "down_projection_backward: null pointer");
   (void)T;
   hipStream_t st = (hipStream_t)stream;
-  if (TK > 0) {
+  if (TK > 0 && dz) {
     rc = launch_dz(dout, z, w2, w2_stride_e, w2_stride_row, dz, y1s, ds_partial, scores, off, x_gather_idx,
                    s_scatter_idx, TK, H, I, E, workspace, st);
     if (rc) return rc;
     rc = launch_ds_finalize(ds_partial, smoe_dz_partial_cols(I), s_scatter_idx, ds, TK, st);
     if (rc) return rc;
   }
+  if (!dw2) return SMOE_OK;
   VarlenKParams p = {};
   p.R = (const uint16_t*)dout;
   p.r_stride = H;
@@ -300,12 +303,14 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
   if (rc) return rc;
   SMOE_REQUIRE(activation == SMOE_ACT_SWIGLU, SMOE_ERR_UNSUPPORTED,
                "up_projection_backward: only SwiGLU is implemented (activation=%d)", activation);
-  SMOE_REQUIRE(dw1 && off, SMOE_ERR_INVALID, "up_projection_backward: null pointer");
-  SMOE_REQUIRE(TK == 0 || (x && w1 && dz && dx_expanded && x_gather_idx), SMOE_ERR_INVALID,
+  SMOE_REQUIRE(off, SMOE_ERR_INVALID, "up_projection_backward: null pointer");
+  SMOE_REQUIRE(dw1 || dx_expanded, SMOE_ERR_INVALID,
+               "up_projection_backward: nothing to compute (dw1 and dx_expanded are both null)");
+  SMOE_REQUIRE(TK == 0 || (dz && x_gather_idx && (!dw1 || x) && (!dx_expanded || w1)), SMOE_ERR_INVALID,
                "up_projection_backward: null pointer");
   (void)T;
   hipStream_t st = (hipStream_t)stream;
-  {
+  if (dw1) {
     VarlenKParams p = {};
     p.R = (const uint16_t*)dz;
     p.r_stride = 2 * I;
@@ -322,7 +327,7 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     rc = launch_varlen_k_variant<false, true>(p, st);
     if (rc) return rc;
   }
-  if (TK > 0) {
+  if (TK > 0 && dx_expanded) {
     rc = launch_dx(dz, w1, w1_stride_e, w1_stride_row, dx_expanded, off, TK, H, I, E, workspace, st);
     if (rc) return rc;
   }

@@ -136,6 +136,8 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     q_step = (int64_t)BK * p.q_stride_row;
   }
 
+  const int S_total = p.Kdim / BK;
+
   // ---- per-lane LDS fragment offsets (bytes inside a stage) ----
   int p_off[SLICES];
   {
@@ -201,8 +203,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       }
     }
   };
-  gemm_mainloop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR + C::Q_INSTR, SLICES, NSTAGE>(p.Kdim / BK, acc, issue,
-                                                                                            load);
+  gemm_mainloop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR + C::Q_INSTR, SLICES, NSTAGE>(S_total, acc, issue, load);
 
   SMOE_STAMP(2)
   const int m_base = row0 + wm * C::TM, n_base = n0 + wn * C::TN;

@@ -16,8 +16,8 @@ from .forward import _check_bf16, _gather_sum, _gemm_workspace
 def _up_projection_backward(
     x: torch.Tensor,
     w1: torch.Tensor,
-    dx_expanded: torch.Tensor,
-    dw1: torch.Tensor,
+    dx_expanded: torch.Tensor | None,
+    dw1: torch.Tensor | None,
     dz: torch.Tensor,
     db1: torch.Tensor | None,
     expert_frequency_offset: torch.Tensor,
@@ -27,7 +27,8 @@ def _up_projection_backward(
     is_glu_activation: bool,
     stream_id: int,
 ) -> None:
-    """dw1[e] = sum_m dz[m]^T x[t_m] (zeros for empty experts), dx_expanded = dz W1[e]."""
+    """dw1[e] = sum_m dz[m]^T x[t_m] (zeros for empty experts), dx_expanded = dz W1[e]; either output may be None
+    to skip it."""
     if db1 is not None:
         raise NotImplementedError("_up_projection_backward: bias is not implemented in the HIP path")
     if expert_schedule_order is not None:
@@ -39,9 +40,9 @@ def _up_projection_backward(
     N1, H, E = w1.shape
     I = N1 // 2
     T, TK = x.size(0), dz.size(0)
-    assert x.is_contiguous() and dz.is_contiguous() and dx_expanded.is_contiguous()
+    assert x.is_contiguous() and dz.is_contiguous() and (dx_expanded is None or dx_expanded.is_contiguous())
     w_se, w_sr = expert_major_strides(w1, "w1")
-    d_se, d_sr = expert_major_strides(dw1, "dw1")
+    d_se, d_sr = expert_major_strides(dw1, "dw1") if dw1 is not None else (0, 0)
     ws = _gemm_workspace(TK, E, x.device)
     rc = _lib.lib().smoe_up_projection_backward(
         _lib.ptr(x),
@@ -73,7 +74,7 @@ def _down_projection_backward(
     dout: torch.Tensor,
     z: torch.Tensor,
     w2: torch.Tensor,
-    dw2: torch.Tensor,
+    dw2: torch.Tensor | None,
     dz: torch.Tensor,
     ds: torch.Tensor,
     b2: torch.Tensor | None,
@@ -101,7 +102,7 @@ def _down_projection_backward(
     assert z.is_contiguous() and dz.is_contiguous() and ds.is_contiguous() and ds.dtype == torch.float32
     assert topk_scores.dtype == torch.float32 and topk_scores.is_contiguous()
     w_se, w_sr = expert_major_strides(w2, "w2")
-    d_se, d_sr = expert_major_strides(dw2, "dw2")
+    d_se, d_sr = expert_major_strides(dw2, "dw2") if dw2 is not None else (0, 0)
     y1s = torch.empty(TK, I, dtype=z.dtype, device=z.device)
     ncols = _lib.lib().smoe_dz_partial_cols(I)
     ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
