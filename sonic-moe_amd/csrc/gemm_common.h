@@ -6,9 +6,9 @@
 // consecutive LDS bytes), so the LDS position of a piece is fixed by (wave, instruction, lane) and swizzling is
 // done by choosing WHICH global piece a lane fetches.
 //
-//   K-major stage : [rows][32 k]   row = 64 B = 4 pieces; piece c of row r sits at c ^ kswz(r).
+//   K-major stage : [rows][BK k]   row = BK*2 B = BK/8 pieces; piece c of row r sits at c ^ kswz(r).
 //                   MFMA operand fragment = one ds_read_b128 per lane (row l%32, pieces 2*ks + l/32).
-//   MN-major stage: [32 k][cols]   row = cols*2 B; 32-byte group g of k-row k sits at g ^ (k & 15) (mod groups).
+//   MN-major stage: [BK k][cols]   row = cols*2 B; 32-byte group g of k-row k sits at g ^ mnswz(k).
 //                   MFMA operand fragment = two ds_read_b64_tr_b16 per lane (the transpose load hands lane i of a
 //                   16-lane group column i of a 4 x 16 block whose rows are named by the lanes' addresses).
 //
@@ -44,6 +44,12 @@ SMOE_DEV int kswz(int row) {
   if constexpr (BK_ == 32) return (row >> 2) & 3;
   else return (row & 7) ^ ((row >> 3) & 1);
 }
+
+// 32-byte-group swizzle of an MN-major stage: group g of contraction row k sits at g ^ mnswz(k).  A transpose load
+// makes the 32 lanes of a half-wave read 4 consecutive k-rows x 2 neighbouring groups; (k & 3) << 1 moves the four rows
+// to four different even offsets and leaves bit 0 to tell the two groups apart, so the eight 32-byte pieces fall into
+// the eight different 32-byte bank groups of the 64 banks.
+SMOE_DEV int mnswz(int k) { return (k & 3) << 1; }
 
 SMOE_DEV bf16x8 lds_read_b128(const char* p) { return *(const bf16x8*)p; }
 

@@ -41,8 +41,6 @@ struct KCfg {
   static constexpr int R_LPR = R_ROWB / 16, S_LPR = S_ROWB / 16;
   static constexpr int R_RPI = 64 / R_LPR, S_RPI = 64 / S_LPR;
   static constexpr int R_INSTR = R_STAGE / 1024 / NW, S_INSTR = S_STAGE / 1024 / NW;
-  static constexpr int R_SWM = (R_ROWB / 32 < 16 ? R_ROWB / 32 : 16) - 1;
-  static constexpr int S_SWM = (S_ROWB / 32 < 16 ? S_ROWB / 32 : 16) - 1;
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
@@ -72,7 +70,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   for (int i = 0; i < C::R_INSTR; i++) {
     const int kl = (wave * C::R_INSTR + i) * C::R_RPI + lane / C::R_LPR;
     const int phys16 = lane % C::R_LPR;
-    const int log32 = (phys16 >> 1) ^ (kl & C::R_SWM);
+    const int log32 = (phys16 >> 1) ^ mnswz(kl);
     int a = a0 + ((log32 << 1) | (phys16 & 1)) * 8;
     a = a <= p.NA - 8 ? a : p.NA - 8;
     r_col[i] = a;
@@ -81,7 +79,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   for (int i = 0; i < C::S_INSTR; i++) {
     const int kl = (wave * C::S_INSTR + i) * C::S_RPI + lane / C::S_LPR;
     const int phys16 = lane % C::S_LPR;
-    const int log32 = (phys16 >> 1) ^ (kl & C::S_SWM);
+    const int log32 = (phys16 >> 1) ^ mnswz(kl);
     int b = b0 + ((log32 << 1) | (phys16 & 1)) * 8;
     b = b <= p.NB - 8 ? b : p.NB - 8;
     s_col[i] = b;
@@ -98,7 +96,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        r_off[f * 2 + h] = k * C::R_ROWB + ((c32 ^ (k & C::R_SWM)) << 5) + ((i16 & 3) << 3);
+        r_off[f * 2 + h] = k * C::R_ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
 #pragma unroll
@@ -107,7 +105,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c32 ^ (k & C::S_SWM)) << 5) + ((i16 & 3) << 3);
+        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
   }

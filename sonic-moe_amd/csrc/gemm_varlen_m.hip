@@ -55,7 +55,6 @@ struct Cfg {
   static constexpr int KPR = KROW / 16;   // 16-byte pieces per row of a K-major stage
   static constexpr int KRPI = 64 / KPR;   // rows per load instruction of a K-major stage
   static constexpr int NG = ROWB / 32;    // 32-byte groups per k-row
-  static constexpr int SWM = (NG < 16 ? NG : 16) - 1;
   static_assert(P_INSTR >= 1 && Q_INSTR >= 1, "tile too small for the wave count");
   static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA");
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
@@ -128,7 +127,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     for (int i = 0; i < C::Q_INSTR; i++) {
       const int kl = (wave * C::Q_INSTR + i) * C::RPI + lane / C::LPR;
       const int phys16 = lane % C::LPR;
-      const int log32 = (phys16 >> 1) ^ (kl & C::SWM);
+      const int log32 = (phys16 >> 1) ^ mnswz(kl);
       int n = n0 + ((log32 << 1) | (phys16 & 1)) * 8;
       n = n <= p.N - 8 ? n : p.N - 8;
       q_src[i] = qe + (int64_t)kl * p.q_stride_row + n;
@@ -161,7 +160,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        q_off[fn * 2 + h] = C::P_STAGE + k * C::ROWB + ((c32 ^ (k & C::SWM)) << 5) + ((i16 & 3) << 3);
+        q_off[fn * 2 + h] = C::P_STAGE + k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
   }
