@@ -33,6 +33,7 @@ PEAK_HBM_GBS = 8000.0
 CONFIGS = {
     "C2": dict(T=32768, H=4096, I=1024, E=128, K=8, zipf=False),
     "C3": dict(T=32768, H=4096, I=1536, E=128, K=8, zipf=True),
+    "C4": dict(T=16384, H=4096, I=1024, E=256, K=8, zipf=False, rounding="nr", tile=128),
 }
 
 
@@ -251,7 +252,20 @@ def main():
     w1v, w2v = w1.permute(1, 2, 0), w2.permute(1, 2, 0)
     bias = zipf_bias(E, dev).to(torch.bfloat16) if cfg["zipf"] else None
 
+    rounding = cfg.get("rounding")
+    if rounding:
+        from sonicmoe.functional import moe_general_routing_inputs
+        from sonicmoe.routing import token_choice_rounding
+
+        with torch.no_grad():  # the rounding router is host-side torch and outside the timed region, as in the reference
+            r_scores, r_tok, r_exp = token_choice_rounding(torch.nn.functional.linear(x, wr), K, cfg["tile"], rounding)
+        r_scores = r_scores.float().requires_grad_()
+
     def layer():
+        if rounding:
+            o, _ = moe_general_routing_inputs(x, r_scores, r_tok, r_exp, w1v, None, w2v, None, E, stream,
+                                              ActivationType.SWIGLU, False)
+            return o
         if bias is None:
             o, _, _ = moe_TC_softmax_topk_layer(x, wr, w1v, None, w2v, None, K, stream, ActivationType.SWIGLU, False)
             return o
@@ -267,9 +281,9 @@ def main():
 
     def fwd_bwd():
         o = layer()
-        torch.autograd.grad(o, [x, wr, w1, w2], grad_outputs=dout)
+        torch.autograd.grad(o, [x, r_scores, w1, w2] if rounding else [x, wr, w1, w2], grad_outputs=dout)
 
-    TK = T * K
+    TK = r_tok.numel() if rounding else T * K
     flops_fwd, flops_all = 6.0 * TK * I * H, 18.0 * TK * I * H
     fwd_ms, _ = time_region(fwd_only, a.steps, a.warmup)
     ms, wall_ms = time_region(fwd_bwd, a.steps, a.warmup)
@@ -277,7 +291,7 @@ def main():
     log(f"{a.config}: fwd {fwd_ms:.3f} ms ({flops_fwd / fwd_ms / 1e9:.1f} TFLOP/s), fwd+bwd {ms:.3f} ms "
         f"({tflops:.1f} TFLOP/s = {100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak), host wall {wall_ms:.3f} ms/step")
 
-    rows = [] if a.no_breakdown else kernel_breakdown(cfg, x, wr, w1, w2, dout, max(5, a.steps // 2))
+    rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, x, wr, w1, w2, dout, max(5, a.steps // 2))
     # dominant kernel = the single grouped-GEMM launch with the largest average duration
     single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS]
     roofline = None
@@ -296,7 +310,7 @@ def main():
         )
 
     out = dict(
-        metric="MoE fwd+bwd TFLOP/s (% bf16 MFMA peak), T=32768 H=4096 I=1024 E=128 K=8",
+        metric=f"MoE fwd+bwd TFLOP/s (% bf16 MFMA peak), T={T} H={H} I={I} E={E} K={K}",
         value=round(tflops, 2),
         unit="TFLOP/s",
         n_gpus=1,
@@ -310,7 +324,9 @@ def main():
         data="synthetic",
         config=dict(
             workload=f"{a.config}: MoE layer fwd+bwd, T={T} H={H} I={I} E={E} K={K}, SwiGLU, no bias, token-choice softmax "
-            f"top-k router{' with Zipf logit bias' if cfg['zipf'] else ''}; x,dout~N(0,1), weights~N(0,0.02), seed 0",
+            f"top-k router{' with Zipf logit bias' if cfg['zipf'] else ''}"
+            f"{' then token rounding (' + rounding + ', tile 128), ' + str(TK) + ' routed pairs, general-routing entry' if rounding else ''}"
+            f"; x,dout~N(0,1), weights~N(0,0.02), seed 0",
             flops_per_step=flops_all,
         ),
         frac_of_peak=round(tflops / PEAK_BF16_TFLOPS, 4),

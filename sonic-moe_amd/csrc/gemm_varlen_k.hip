@@ -24,6 +24,7 @@ struct VarlenKParams {
   int NA, NB;  // output rows / cols
   int tiles_a, tiles_b;
   int E;
+  int xcd_chunked;  // 1: contiguous tile range per XCD (probe), 0: round-robin
 };
 
 template <int BA_, int BB_, int WA_, int WB_, bool R_GATHER_, bool S_GATHER_, int BK_, int NSTAGE_>
@@ -53,8 +54,11 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave % C::WA, wb = wave / C::WA;
 
+  // Tiles of one expert are dealt round-robin over the XCDs (workgroup b runs on XCD b % 8): an expert's cost is its
+  // token count, so giving every XCD a slice of every expert balances skewed loads, and the tiles an XCD gets from one
+  // expert (every 8th) still share their S-operand columns in its L2.
   const int64_t per_e = (int64_t)p.tiles_a * p.tiles_b;
-  const int64_t lin = xcd_linear_tile(per_e * p.E);
+  const int64_t lin = p.xcd_chunked ? xcd_linear_tile(per_e * p.E) : (blockIdx.x < per_e * p.E ? (int64_t)blockIdx.x : -1);
   if (lin < 0) return;
   const int e = (int)(lin / per_e);
   const int within = (int)(lin - (int64_t)e * per_e);
@@ -202,6 +206,10 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   VarlenKParams p = pin;
   p.tiles_a = (int)ceil_div(p.NA, C::BA);
   p.tiles_b = (int)ceil_div(p.NB, C::BB);
+  {
+    static const int chunked = getenv("SMOE_VARLEN_K_XCD_CHUNKED") ? atoi(getenv("SMOE_VARLEN_K_XCD_CHUNKED")) : 0;
+    p.xcd_chunked = chunked;
+  }
   const int64_t total = (int64_t)p.tiles_a * p.tiles_b * p.E;
   const int64_t grid = ((total + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "weight-grad gemm: too many tiles");

@@ -1,0 +1,147 @@
+"""GPU parity at the remaining BASELINE configurations: Zipf-skewed load with empty experts (config 3, reduced T so
+that the fp32 oracle finishes in seconds), token-rounding routing through moe_general_routing_inputs (config 4), and
+size-independent properties at the full size of config 2."""
+
+import pytest
+import torch
+
+from helpers import make_weights, rel_l2
+from oracle import moe_math as M
+from oracle import routing as R
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _zipf_bias(E, dev):
+    e = torch.arange(E, device=dev, dtype=torch.float32)
+    return 2.0 * torch.log(1.0 / (e + 1.0))
+
+
+def test_zipf_skewed_load_with_empty_experts(dev):
+    """Config 3 semantics: logits + 2*log(1/(e+1)); the tail experts receive no token, the head ones thousands."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import TC_Softmax_Topk_Router_Function, _build_metadata, _ExpertsFunction
+
+    T, H, I, E, K = 4096, 1024, 384, 128, 8
+    wr, w1, w2 = make_weights(E, H, I, dev, seed=21)
+    g = torch.Generator().manual_seed(22)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    w1.requires_grad_(); w2.requires_grad_(); wr.requires_grad_()
+    logits = torch.nn.functional.linear(x, wr) + _zipf_bias(E, dev).to(torch.bfloat16)
+    s, i = TC_Softmax_Topk_Router_Function.apply(logits, E, K)
+    freq, off, gidx, sidx, ridx, tok_off = _build_metadata(i.view(-1), None, T, E, K)
+    assert int((freq == 0).sum()) > 0, "the skew should leave some experts empty"
+    assert int(freq.max()) > 4 * T * K // E
+    o = _ExpertsFunction.apply(x, w1.permute(1, 2, 0), w2.permute(1, 2, 0), s.view(-1), off, gidx, sidx, ridx, tok_off,
+                               K, False, ActivationType.SWIGLU, torch.cuda.current_stream().cuda_stream, False)
+    grads = torch.autograd.grad(o, [x, wr, w1, w2], grad_outputs=dy)
+
+    # routing bit-exact against the oracle on the same logits
+    s_ref, i_ref = R.topk_softmax(logits.detach().float().cpu().numpy(), K)
+    assert torch.equal(i.cpu(), torch.from_numpy(i_ref))
+    meta = R.tc_topk_router_metadata(i_ref, E)
+    for name, t in zip(["expert_frequency", "expert_frequency_offset", "x_gather_idx", "s_scatter_idx",
+                        "s_reverse_scatter_idx"], [freq, off, gidx, sidx, ridx]):
+        assert torch.equal(t.cpu(), torch.from_numpy(meta[name])), name
+
+    # float parity: the same function in fp32 torch (logit bias added by hand, so restate the few lines here)
+    xr, wrr, w1r, w2r = (t.detach().clone().float().requires_grad_() for t in (x, wr, w1, w2))
+    lin = torch.nn.functional.linear(xr, wrr)
+    # value: the bf16-rounded biased logits the layer saw; gradient: that of the linear map
+    lg = (lin.detach().to(torch.bfloat16) + _zipf_bias(E, dev).to(torch.bfloat16)).float() + (lin - lin.detach())
+    gates = torch.softmax(lg.gather(1, i.long()), dim=-1)
+    tok = torch.arange(T, device=dev).repeat_interleave(K)
+    o_ref = M.general_routing_reference(xr, gates.reshape(-1), tok, i.reshape(-1), w1r, w2r, E)
+    grads_ref = torch.autograd.grad(o_ref, [xr, wrr, w1r, w2r], grad_outputs=dy.float())
+    assert rel_l2(o, o_ref) < TOL
+    for n, a, b in zip(["dx", "d_router", "dw1", "dw2"], grads, grads_ref):
+        assert rel_l2(a, b) < TOL, (n, rel_l2(a, b))
+    empty = (freq == 0).nonzero().flatten().tolist()
+    assert bool((grads[2][empty] == 0).all()) and bool((grads[3][empty] == 0).all())
+
+
+@pytest.mark.parametrize("routing", ["nr", "up", "down"])
+def test_token_rounding_general_routing(dev, routing):
+    """Config 4 semantics at T=4096: expert counts rounded to multiples of the 128-token tile, general-routing entry."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import moe_general_routing_inputs
+    from sonicmoe.routing import token_choice_rounding
+
+    T, H, I, E, K, tile = 4096, 1024, 256, 64, 4, 128
+    wr, w1, w2 = make_weights(E, H, I, dev, seed=31)
+    g = torch.Generator().manual_seed(32)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    with torch.no_grad():
+        logits = torch.nn.functional.linear(x, wr)
+        scores, tok, exp = token_choice_rounding(logits, K, tile, routing)
+    scores = scores.float().requires_grad_()
+    w1.requires_grad_(); w2.requires_grad_()
+    o, freq = moe_general_routing_inputs(x, scores, tok, exp, w1.permute(1, 2, 0), None, w2.permute(1, 2, 0), None, E,
+                                         torch.cuda.current_stream().cuda_stream, ActivationType.SWIGLU, False)
+    assert bool((freq % tile == 0).all()) and int(freq.sum()) == tok.numel()
+    grads = torch.autograd.grad(o, [x, scores, w1, w2], grad_outputs=dy)
+    xr, sr, w1r, w2r = (t.detach().clone().float().requires_grad_() for t in (x, scores, w1, w2))
+    o_ref = M.general_routing_reference(xr, sr, tok, exp, w1r, w2r, E)
+    grads_ref = torch.autograd.grad(o_ref, [xr, sr, w1r, w2r], grad_outputs=dy.float())
+    assert rel_l2(o, o_ref) < TOL
+    for n, a, b in zip(["dx", "dscores", "dw1", "dw2"], grads, grads_ref):
+        assert rel_l2(a, b) < TOL, n
+
+
+def test_full_size_properties(dev):
+    """Config 2 at full size (T=32768,H=4096,I=1024,E=128,K=8): properties that need no second implementation.
+    (1) the routing metadata is a stable sort of the router's choice; (2) two runs are bit-identical; (3) the layer is
+    linear in the upstream gradient: grads(2*dout) == 2*grads(dout) exactly in bf16 (power-of-two scaling);
+    (4) 64 sampled tokens agree with a dense fp32 evaluation of just those tokens."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import _build_metadata, moe_TC_softmax_topk_layer
+
+    T, H, I, E, K = 32768, 4096, 1024, 128, 8
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16).requires_grad_()
+    wr = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    w1 = (0.02 * torch.randn(E, 2 * I, H, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    w2 = (0.02 * torch.randn(E, H, I, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    dout = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(dy):
+        o, logits, freq = moe_TC_softmax_topk_layer(x, wr, w1.permute(1, 2, 0), None, w2.permute(1, 2, 0), None, K, st,
+                                                    ActivationType.SWIGLU, False)
+        return o, logits, freq, torch.autograd.grad(o, [x, wr, w1, w2], grad_outputs=dy)
+
+    o1, logits, freq, g1 = run(dout)
+    o2, _, _, g2 = run(dout)
+    assert torch.equal(o1, o2) and all(torch.equal(a, b) for a, b in zip(g1, g2)), "not deterministic"
+    _, _, _, g3 = run(dout * 2)
+    for a, b in zip(g1[2:], g3[2:]):  # weight gradients: exactly linear (scores' path does not enter them twice)
+        assert torch.equal(a * 2, b)
+
+    # metadata invariants on the real routing
+    with torch.no_grad():
+        from sonicmoe.functional import forward
+
+        scores = torch.empty(T, K, dtype=torch.float32, device=dev)
+        idx = torch.empty(T, K, dtype=torch.int32, device=dev)
+        forward._topk_fwd(logits, K, scores, idx, True)
+        f, off, gidx, sidx, ridx, tok_off = _build_metadata(idx.view(-1), None, T, E, K)
+    flat = idx.view(-1).long()
+    assert torch.equal(f, freq) and int(f.sum()) == T * K and int(off[-1]) == T * K
+    assert torch.equal(sidx.long(), torch.sort(flat, stable=True).indices)
+    assert torch.equal(ridx[sidx.long()].long(), torch.arange(T * K, device=dev))
+    assert torch.equal(gidx, sidx // K)
+    assert bool((idx[:, :-1] != idx[:, 1:]).all()) and bool((scores[:, :-1] >= scores[:, 1:]).all())
+
+    # sampled tokens against a dense fp32 evaluation
+    sample = torch.randperm(T, generator=torch.Generator().manual_seed(1))[:64].to(dev)
+    xs = x.detach()[sample].float()
+    ref = torch.zeros(64, H, device=dev)
+    for j in range(K):
+        e = idx[sample, j].long()
+        h = torch.einsum("th,tnh->tn", xs, w1.detach()[e].float())
+        y = torch.nn.functional.silu(h[:, 0::2]) * h[:, 1::2]
+        ref += scores[sample, j, None] * torch.einsum("ti,thi->th", y, w2.detach()[e].float())
+    assert rel_l2(o1.detach()[sample], ref) < TOL
