@@ -60,15 +60,6 @@ struct Cfg {
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
-#ifdef SMOE_PROBE_TIMING
-// probe build only: per-tile shader-clock timestamps (start, pipeline primed, main loop done, end) of the first tiles
-__device__ unsigned long long g_probe_times[4096 * 4];
-#define SMOE_STAMP(i) \
-  if (lin < 4096 && tid == 0) g_probe_times[lin * 4 + (i)] = __builtin_amdgcn_s_memtime();
-#else
-#define SMOE_STAMP(i)
-#endif
-
 template <class C, int ROLE>
 __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -87,11 +78,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   const int group = (int)(lin / per_group);
   const int first_m = group * GM;
   const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
-  SMOE_STAMP(0)
-#ifdef SMOE_PROBE_TIMING
-  if (lin < 4096 && tid == 0)
-    g_probe_times[lin * 4 + 1] = ((unsigned long long)__builtin_amdgcn_s_getreg(63508) << 32) | __builtin_amdgcn_s_getreg(63492);
-#endif
   const int within = (int)(lin - (int64_t)group * per_group);
   const int mt = first_m + within % gm;
   const int nt = within / gm;
@@ -204,7 +190,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   };
   gemm_mainloop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR + C::Q_INSTR, SLICES, NSTAGE>(S_total, acc, issue, load);
 
-  SMOE_STAMP(2)
   const int m_base = row0 + wm * C::TM, n_base = n0 + wn * C::TN;
 #ifdef SMOE_PROBE_NO_EPILOGUE
   if (acc[0][0][0] != 12345.f) return;
@@ -278,14 +263,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       if (mvalid && lane < 32) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
     });
   }
-  SMOE_STAMP(3)
 }
-
-#ifdef SMOE_PROBE_TIMING
-extern "C" int smoe_probe_read(void* dst, size_t bytes) {
-  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_probe_times), bytes);
-}
-#endif
 
 template <class C, int ROLE>
 static int launch_varlen_m(const VarlenMParams& p, int64_t TK, int E, hipStream_t st) {

@@ -127,3 +127,20 @@ def test_general_routing_layer(dev):
         assert rel_l2(a, b) < TOL, n
     # tokens without any expert get exactly zero
     assert bool((o[::5] == 0).all())
+
+
+def test_torch_compile_fullgraph(dev):
+    """The operators are registered custom ops with declared mutations, so the module compiles with fullgraph=True
+    (the reference tests the same: tests/moe_test.py:80-81); results must match eager."""
+    from sonicmoe import KernelBackendMoE
+
+    moe, x, dy = _build(dev, 1024, 512, 256, 8, 2)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_proj.weight]
+    out, _ = moe(x, kernel_backend_moe=KernelBackendMoE.sonicmoe)
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+    compiled = torch.compile(moe, fullgraph=True)
+    out_c, _ = compiled(x)
+    grads_c = torch.autograd.grad(out_c, [x] + params, grad_outputs=dy)
+    assert torch.equal(out, out_c)
+    for a, b in zip(grads, grads_c):
+        assert rel_l2(a, b) < 1e-3  # dx: the compiled graph fuses the two dx contributions before the bf16 rounding
