@@ -94,6 +94,8 @@ SMOE_DEV void wait_vmem_upto() {
   __builtin_amdgcn_s_waitcnt(0x0070 | (N & 15) | ((N >> 4) << 14));
 }
 SMOE_DEV void wait_vmem_all() { wait_vmem_upto<0>(); }
+// s_waitcnt lgkmcnt(0) only: all of this wave's LDS operations have completed, vector memory untouched
+SMOE_DEV void wait_lds_all() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 
 // Workgroup barrier WITHOUT the memory fence of __syncthreads(): a fence would wait for every outstanding
 // direct-to-LDS load (vmcnt(0)) and collapse the ring to one stage in flight.  The waits that make LDS contents
@@ -201,6 +203,14 @@ SMOE_DEV void epilogue_flush(const char* region, int lane, uint16_t* out, int64_
 
 // 256 zero bytes: clamped (out-of-range) token rows of the weight-gradient GEMMs are fetched from here
 static __device__ __attribute__((aligned(256))) const uint32_t smoe_zero_page[64] = {};
+
+// park a few bytes of row `row` of an unpadded [32][RB-byte] LDS area; 16-byte chunk c sits at c ^ ((row >> 1) & 7)
+template <int RB, class V>
+SMOE_DEV void epi_park_y(char* area, int row, int col_bytes, V v) {
+  constexpr int CH = RB / 16;
+  const int chunk = (col_bytes >> 4) ^ ((row >> 1) & (CH < 8 ? CH - 1 : 7));
+  *(V*)(area + row * RB + (chunk << 4) + (col_bytes & 15)) = v;
+}
 
 // ---- tile map ------------------------------------------------------------------------------------------------
 // Built on the device from the expert offsets; header[0] = number of token tiles.  Entry i = (expert, first row).

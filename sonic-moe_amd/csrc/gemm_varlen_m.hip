@@ -228,39 +228,85 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       epilogue_flush<C::TM, C::TN / 2>(region, lane, p.out1, p.out1_stride, m_base, row_end, n_base / 2, p.N / 2);
     }
   } else {
-    // ---- dz epilogue: lane owns token column m = l%32 and 4 consecutive intermediate features per register quad ----
+    // ---- dz epilogue ----
+    // acc = dy1[i][m].  Per 32-row fragment row the wavefront stages its z sub-tile (32 x 2*TN bf16) through LDS:
+    // row-contiguous 16-byte global loads (two fragment rows in flight in registers) -> LDS -> each lane picks the
+    // four (gate, up) pairs of its token row, computes dz in place and y1s into a second area -> both are written back
+    // row-contiguous.  All global traffic of the epilogue is full 128-byte lines.
+    constexpr int ZB = C::TN * 4, YB = C::TN * 2;            // bytes per staged z/dz row, y1s row
+    constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
+    constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
+    static_assert(C::NW * 32 * (ZB + YB) <= NSTAGE * C::STAGE, "dz staging must fit into the idle ring");
+    char* zbuf = smem + wave * (32 * (ZB + YB));
+    char* ybuf = zbuf + 32 * ZB;
+    const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
+    const int zcol = 2 * n_base + zc * 8;  // first z column of this lane's 16-byte chunk
+    const int zcol_c = zcol <= 2 * p.N - 8 ? zcol : 2 * p.N - 8;
+    u32x4 zreg[2][ZN];
+    auto fetch_z = [&](int fm, u32x4(&dst)[ZN]) {
+#pragma unroll
+      for (int it = 0; it < ZN; it++) {
+        int m = m_base + fm * 32 + it * ZR + zr;
+        m = m < row_end ? m : row_end - 1;
+        dst[it] = *(const u32x4*)(p.zin + (int64_t)m * p.zin_stride + zcol_c);
+      }
+    };
+    fetch_z(0, zreg[0]);
+    if constexpr (FM > 1) fetch_z(1, zreg[1]);
+    wait_lds_all();
+    lds_barrier();  // every wave has finished reading the ring
     static_for<FM>([&](auto fm_c) {
       constexpr int fm = decltype(fm_c)::value;
-      const int m = m_base + fm * 32 + (lane & 31);
+#pragma unroll
+      for (int it = 0; it < ZN; it++) {
+        const int r = it * ZR + zr;
+        *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & 15)) << 4)) = zreg[fm & 1][it];
+      }
+      if constexpr (fm + 2 < FM) fetch_z(fm + 2, zreg[fm & 1]);
+      const int mrow = lane & 31;
+      const int m = m_base + fm * 32 + mrow;
       const bool mvalid = m < row_end;
-      float s = 0.f, dsum = 0.f;
-      if (mvalid) s = p.scores[p.sidx[m]];
+      float sc = 0.f, dsum = 0.f;
+      if (mvalid) sc = p.scores[p.sidx[m]];
       static_for<FN * 4>([&](auto q_c) {
         constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        const int n = n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
-        if (mvalid && n < p.N) {
-          const u32x4 zz = *(const u32x4*)(p.zin + (int64_t)m * p.zin_stride + 2 * n);
-          u32x4 dzv;
-          float ys[4];
+        const int il = fn * 32 + 8 * rg + 4 * (lane >> 5);  // first of this lane's 4 intermediate features (wave-local)
+        char* zaddr = zbuf + mrow * ZB + ((((il * 4) >> 4) ^ (mrow & 15)) << 4);
+        const u32x4 zz = *(const u32x4*)zaddr;
+        u32x4 dzv;
+        float ys[4];
 #pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const float dy = acc[fn][fm][4 * rg + q];
-            const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
-            const float sig = fast_sigmoid(g);
-            const float silu = g * sig;
-            const float y1v = silu * u;
-            dsum += dy * y1v;
-            const float sd = s * dy;
-            dzv[q] = pack_bf16x2(sd * u * (silu * (1.f - sig) + sig), sd * silu);
-            ys[q] = s * y1v;
-          }
-          *(u32x4*)(p.out0 + (int64_t)m * p.out0_stride + 2 * n) = dzv;
-          u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
-          *(u32x2*)(p.out1 + (int64_t)m * p.out1_stride + n) = yv;
+        for (int q = 0; q < 4; q++) {
+          const float dy = acc[fn][fm][4 * rg + q];
+          const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
+          const float sig = fast_sigmoid(g);
+          const float silu = g * sig;
+          const float y1v = silu * u;
+          if (n_base + il + q < p.N) dsum += dy * y1v;
+          const float sd = sc * dy;
+          dzv[q] = pack_bf16x2(sd * u * (silu * (1.f - sig) + sig), sd * silu);
+          ys[q] = sc * y1v;
         }
+        *(u32x4*)zaddr = dzv;
+        u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
+        epi_park_y<YB>(ybuf, mrow, il * 2, yv);
       });
       dsum += __shfl_xor(dsum, 32, 64);
       if (mvalid && lane < 32) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
+#pragma unroll
+      for (int it = 0; it < ZN; it++) {
+        const int r = it * ZR + zr;
+        const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & 15)) << 4));
+        const int mm = m_base + fm * 32 + r;
+        if (mm < row_end && zcol < 2 * p.N) *(u32x4*)(p.out0 + (int64_t)mm * p.out0_stride + zcol) = v;
+      }
+#pragma unroll
+      for (int it = 0; it < YN; it++) {
+        const int r = it * YR + yr;
+        const u32x4 v = *(const u32x4*)(ybuf + r * YB + ((yc ^ ((r >> 1) & (YL < 8 ? YL - 1 : 7))) << 4));
+        const int mm = m_base + fm * 32 + r, col = n_base + yc * 8;
+        if (mm < row_end && col < p.N) *(u32x4*)(p.out1 + (int64_t)mm * p.out1_stride + col) = v;
+      }
     });
   }
 }
@@ -291,15 +337,13 @@ template <bool QMN>
 using CfgV2 = Cfg<256, 256, 2, 4, QMN, 32, 5>;  // 8 waves (2 per SIMD), BK 32, 5-stage ring
 template <bool QMN>
 using CfgV3 = Cfg<256, 256, 2, 4, QMN, 64, 2>;  // 8 waves, BK 64, double buffer
-template <bool QMN>
-using CfgV4 = Cfg<256, 256, 4, 2, QMN, 64, 2>;  // 8 waves, 4 along tokens
 
 int gemm_variant() {
   static int v = -1;
   if (v < 0) {
     const char* e = getenv("SMOE_GEMM_VARIANT");
     v = e ? atoi(e) : 3;
-    if (v < 0 || v > 4) v = 3;
+    if (v < 0 || v > 3) v = 3;
   }
   return v;
 }
@@ -320,14 +364,13 @@ static int launch_varlen_m_variant(VarlenMParams& p, const int32_t* off, void* w
     case 0: return go(CfgV0<QMN>{});
     case 1: return go(CfgV1<QMN>{});
     case 2: return go(CfgV2<QMN>{});
-    case 4: return go(CfgV4<QMN>{});
     default: return go(CfgV3<QMN>{});
   }
 }
 
 int dz_wave_cols() {
   switch (gemm_variant()) {
-    case 0: case 1: case 4: return 2;
+    case 0: case 1: return 2;
     default: return 4;
   }
 }
