@@ -272,7 +272,7 @@ def main():
         logits = torch.nn.functional.linear(x, wr) + bias
         s, i = TC_Softmax_Topk_Router_Function.apply(logits, E, K)
         _, off, gidx, sidx, ridx, tok_off = _build_metadata(i.view(-1), None, T, E, K)
-        return _ExpertsFunction.apply(x, w1v, w2v, s.view(-1), off, gidx, sidx, ridx, tok_off, K, False,
+        return _ExpertsFunction.apply(x, w1v, None, w2v, None, s.view(-1), off, gidx, sidx, ridx, tok_off, K, False,
                                       ActivationType.SWIGLU, stream, False)
 
     def fwd_only():

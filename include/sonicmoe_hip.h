@@ -100,20 +100,24 @@ int smoe_routing_metadata(const int32_t* expert_idx, const int32_t* token_idx, i
 /* Workspace needed by every grouped GEMM below (tile map built from `off` on the device). */
 size_t smoe_gemm_workspace_bytes(int64_t TK, int E);
 
-/* z[m] = x[x_gather_idx[m]] W1[e]^T ; y1[m] = act(z_even) * z_odd (GLU, gate = even columns) or act(z).
- * Replaces sonicmoe::_up_projection_forward (sonicmoe/functional/forward.py:53-129).
- *   x (T, H); w1 (E, N1, H) with N1 = 2I (GLU) or I; z (TK, N1) or NULL (inference: not stored); y1 (TK, I)
- * Limits: H % 64 == 0, I % 64 == 0, SwiGLU only in this version, no bias. */
-int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* z,
-                               void* y1, const int32_t* off, const int32_t* x_gather_idx, int64_t T, int64_t TK,
-                               int H, int I, int E, int activation, void* workspace, size_t workspace_bytes,
-                               void* stream);
+/* z[m] = x[x_gather_idx[m]] W1[e]^T (+ b1[e]);  y1[m] = f(z_even) * z_odd for the gated activations (gate = even
+ * columns), f(z) otherwise; f = silu / gelu (erf form) / relu / relu^2 as the activation code says.
+ * Replaces sonicmoe::_up_projection_forward (sonicmoe/functional/forward.py:53-129; activation epilogue
+ * sonicmoe/functional/grouped_gemm.py:423-439, :1273-1357).
+ *   x (T, H); w1 (E, N1, H) with N1 = 2I (gated) or I; b1 (E, N1) contiguous or NULL; z (TK, N1) or NULL
+ *   (inference: not stored); y1 (TK, I)
+ * Limits: H % 64 == 0, I % 64 == 0. */
+int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
+                               const void* b1, void* z, void* y1, const int32_t* off, const int32_t* x_gather_idx,
+                               int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
+                               size_t workspace_bytes, void* stream);
 
-/* y2[m] = y1[m] W2[e]^T.  Replaces sonicmoe::_down_projection_forward (sonicmoe/functional/forward.py:132-178).
- *   y1 (TK, I); w2 (E, H, I); y2 (TK, H) */
+/* y2[m] = y1[m] W2[e]^T (+ b2[e]).  Replaces sonicmoe::_down_projection_forward
+ * (sonicmoe/functional/forward.py:132-178).
+ *   y1 (TK, I); w2 (E, H, I); b2 (E, H) contiguous or NULL; y2 (TK, H) */
 int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
-                                 void* y2, const int32_t* off, int64_t TK, int H, int I, int E, void* workspace,
-                                 size_t workspace_bytes, void* stream);
+                                 const void* b2, void* y2, const int32_t* off, int64_t TK, int H, int I, int E,
+                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /* out[t] = sum_{j in [tok_off[t], tok_off[t+1])} w[j] * src[ridx[j]]  (w == NULL: unweighted), fp32 accumulate.
  * Replaces sonicmoe::_router_forward and sonicmoe::_token_broadcast_backward
@@ -123,26 +127,31 @@ int smoe_gather_sum(const void* src, void* out, const float* w, const int32_t* r
                     int64_t T, int K, int H, void* stream);
 
 /* Backward of down projection + combine.  Replaces sonicmoe::_down_projection_backward
- * (sonicmoe/functional/backward.py:286-461).
- *   dy1 = dout[x_gather_idx] W2[e] (never stored); with (g,u) = z pairs and s = scores[s_scatter_idx[m]]:
- *   dz (TK, 2I), y1s = s*silu(g)*u (TK, I), ds[s_scatter_idx[m]] = sum_i dy1*y1 (fp32, flat-slot order),
- *   dw2 (E, H, I) = sum_m dout[t_m]^T (x) y1s[m]  (zeros for empty experts).
+ * (sonicmoe/functional/backward.py:286-461; bias part backward.py:31-107; epilogue math
+ * sonicmoe/functional/grouped_gemm.py:1154-1271, :1311-1333, :2536-2561).
+ *   dy1 = dout[x_gather_idx] W2[e] (never stored); with s = scores[s_scatter_idx[m]] and y1 = act(z) recomputed:
+ *   dz (TK, N1) = s * dy1 * d(act)/dz, y1s = s*y1 (TK, I),
+ *   ds[s_scatter_idx[m]] = sum_i dy1*y1 (+ <dout[t_m], b2[e]> when b2 is given) (fp32, flat-slot order),
+ *   dw2 (E, H, I) = sum_m dout[t_m]^T (x) y1s[m]  (zeros for empty experts),
+ *   db2 (E, H) contiguous = sum_m s * dout[t_m]  (bf16, zeros for empty experts).
  *   ds_partial: fp32 scratch of TK * smoe_dz_partial_cols(I) elements.
- *   dw2 == NULL skips the weight gradient; dz == NULL skips the activation gradient (y1s must then hold the values a
- *   previous call produced). */
+ *   dw2 == NULL / db2 == NULL skip those gradients; dz == NULL skips the activation gradient (y1s must then hold
+ *   the values a previous call produced). */
 int smoe_dz_partial_cols(int I);
 int smoe_down_projection_backward(const void* dout, const void* z, const void* w2, int64_t w2_stride_e,
-                                  int64_t w2_stride_row, void* dw2, int64_t dw2_stride_e, int64_t dw2_stride_row,
-                                  void* dz, void* y1s, float* ds, float* ds_partial, const float* scores,
-                                  const int32_t* off, const int32_t* x_gather_idx, const int32_t* s_scatter_idx,
-                                  int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
-                                  size_t workspace_bytes, void* stream);
+                                  int64_t w2_stride_row, const void* b2, void* dw2, int64_t dw2_stride_e,
+                                  int64_t dw2_stride_row, void* db2, void* dz, void* y1s, float* ds,
+                                  float* ds_partial, const float* scores, const int32_t* off,
+                                  const int32_t* x_gather_idx, const int32_t* s_scatter_idx, int64_t T, int64_t TK,
+                                  int H, int I, int E, int activation, void* workspace, size_t workspace_bytes,
+                                  void* stream);
 
-/* dW1[e] = sum_m dz[m]^T (x) x[t_m];  dx_expanded[m] = dz[m] W1[e].
- * Replaces sonicmoe::_up_projection_backward (sonicmoe/functional/backward.py:195-283).
- *   dw1 == NULL or dx_expanded == NULL skips that output (frozen weights / no input gradient). */
+/* dW1[e] = sum_m dz[m]^T (x) x[t_m];  db1[e] = sum_m dz[m];  dx_expanded[m] = dz[m] W1[e].
+ * Replaces sonicmoe::_up_projection_backward (sonicmoe/functional/backward.py:195-283; db1 backward.py:109-168).
+ *   dz (TK, N1) with N1 = 2I for gated activations, I otherwise; db1 (E, N1) contiguous, bf16
+ *   dw1 == NULL, db1 == NULL or dx_expanded == NULL skips that output (frozen weights / no input gradient). */
 int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
-                                const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row,
+                                const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row, void* db1,
                                 void* dx_expanded, const int32_t* off, const int32_t* x_gather_idx, int64_t T,
                                 int64_t TK, int H, int I, int E, int activation, void* workspace,
                                 size_t workspace_bytes, void* stream);

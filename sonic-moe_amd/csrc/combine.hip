@@ -1,6 +1,6 @@
-// Weighted gather-sum over a token's routed rows (forward combine, backward dx reduction) and the ds finalise.
-// HBM-bound: each grouped row is read exactly once in 16-byte pieces, each output row written once.
-#include "common.h"
+// Weighted gather-sum over a token's routed rows (forward combine, backward dx reduction), the ds finalise and the
+// bias-gradient reductions.  HBM-bound: each row is read exactly once in 16-byte pieces, each output row written once.
+#include "gemm_common.h"
 
 namespace smoe {
 
@@ -70,6 +70,107 @@ int launch_ds_finalize(const float* ds_partial, int ncols, const int32_t* sidx, 
   if (TK == 0) return SMOE_OK;
   hipLaunchKernelGGL(ds_finalize_kernel, dim3((unsigned)ceil_div(TK, 256)), dim3(256), 0, st, ds_partial, ncols, sidx,
                      ds, TK);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+// Per-expert weighted column sums.  Workgroup (e, column block of 512): its four wavefronts walk the expert's rows
+// four apart, every lane keeps 8 columns in fp32; the four partial sums meet in LDS and are rounded once.
+__global__ __launch_bounds__(256) void expert_colsum_kernel(const uint16_t* __restrict__ src, int64_t src_stride,
+                                                            int ncols, const int32_t* __restrict__ gidx,
+                                                            const float* __restrict__ scores,
+                                                            const int32_t* __restrict__ sidx,
+                                                            const int32_t* __restrict__ off,
+                                                            uint16_t* __restrict__ out) {
+  __shared__ float part[4][64][8];
+  const int e = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = (blockIdx.y * 64 + lane) * 8;
+  const bool active = col < ncols;
+  const int begin = off[e], end = off[e + 1];
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++) acc[i] = 0.f;
+  constexpr int UNROLL = 4;
+  for (int m0 = begin + wave; m0 < end; m0 += 4 * UNROLL) {
+    u32x4 v[UNROLL];
+    float w[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+      const int m = m0 + 4 * u;
+      v[u] = u32x4{0, 0, 0, 0};
+      w[u] = 0.f;
+      if (m < end && active) {
+        const int64_t row = gidx ? (int64_t)gidx[m] : (int64_t)m;
+        w[u] = scores ? scores[sidx[m]] : 1.f;
+        v[u] = *(const u32x4*)(src + row * src_stride + col);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        acc[2 * q] += w[u] * bf16_lo(v[u][q]);
+        acc[2 * q + 1] += w[u] * bf16_hi(v[u][q]);
+      }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; i++) part[wave][lane][i] = acc[i];
+  __syncthreads();
+  if (wave == 0 && active) {
+    u32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const float a = part[0][lane][2 * q] + part[1][lane][2 * q] + part[2][lane][2 * q] + part[3][lane][2 * q];
+      const float b = part[0][lane][2 * q + 1] + part[1][lane][2 * q + 1] + part[2][lane][2 * q + 1] +
+                      part[3][lane][2 * q + 1];
+      o[q] = pack_bf16x2(a, b);
+    }
+    *(u32x4*)(out + (int64_t)e * ncols + col) = o;
+  }
+}
+
+int launch_expert_colsum(const uint16_t* src, int64_t src_stride, int ncols, const int32_t* gidx, const float* scores,
+                         const int32_t* sidx, const int32_t* off, int E, uint16_t* out, hipStream_t st) {
+  SMOE_REQUIRE(ncols % 8 == 0, SMOE_ERR_UNSUPPORTED, "bias gradient: %d columns are not a multiple of 8", ncols);
+  hipLaunchKernelGGL(expert_colsum_kernel, dim3((unsigned)E, (unsigned)ceil_div(ncols, 512)), dim3(256), 0, st, src,
+                     src_stride, ncols, gidx, scores, sidx, off, out);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+// One wavefront per grouped row m: its expert by bisection of the offsets, then a dot product over H.
+__global__ __launch_bounds__(256) void ds_bias_term_kernel(const uint16_t* __restrict__ dout,
+                                                           const uint16_t* __restrict__ b2,
+                                                           const int32_t* __restrict__ gidx,
+                                                           const int32_t* __restrict__ sidx,
+                                                           const int32_t* __restrict__ off, int E, int H,
+                                                           float* __restrict__ ds, int64_t TK) {
+  const int64_t m = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (m >= TK) return;
+  const int lane = threadIdx.x & 63;
+  int lo = 0, hi = E;  // largest e with off[e] <= m
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (off[mid] <= m) lo = mid; else hi = mid;
+  }
+  const uint16_t* row = dout + (int64_t)gidx[m] * H;
+  const uint16_t* bias = b2 + (int64_t)lo * H;
+  float s = 0.f;
+  for (int c = lane * 8; c < H; c += 512) {
+    const u32x4 a = *(const u32x4*)(row + c), b = *(const u32x4*)(bias + c);
+#pragma unroll
+    for (int q = 0; q < 4; q++) s += bf16_lo(a[q]) * bf16_lo(b[q]) + bf16_hi(a[q]) * bf16_hi(b[q]);
+  }
+#pragma unroll
+  for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);
+  if (lane == 0) ds[sidx[m]] += s;
+}
+
+int launch_ds_bias_term(const uint16_t* dout, const uint16_t* b2, const int32_t* gidx, const int32_t* sidx,
+                        const int32_t* off, int E, int H, float* ds, int64_t TK, hipStream_t st) {
+  if (TK == 0) return SMOE_OK;
+  hipLaunchKernelGGL(ds_bias_term_kernel, dim3((unsigned)ceil_div(TK, 4)), dim3(256), 0, st, dout, b2, gidx, sidx, off,
+                     E, H, ds, TK);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }

@@ -212,6 +212,47 @@ SMOE_DEV void epi_park_y(char* area, int row, int col_bytes, V v) {
   *(V*)(area + row * RB + (chunk << 4) + (col_bytes & 15)) = v;
 }
 
+// ---- activations -------------------------------------------------------------------------------------------------
+// The seven activation codes (smoe_activation) are four pointwise functions, gated (y = f(gate) * up, codes 0-2) or
+// not (y = f(z)).  GELU is the exact erf form, the one the reference's torch backend evaluates.
+enum Pointwise { PW_SILU = 0, PW_GELU = 1, PW_RELU = 2, PW_RELU_SQ = 3 };
+constexpr bool act_is_glu(int act) { return act <= SMOE_ACT_REGLU; }
+constexpr int act_pointwise(int act) {
+  return act == SMOE_ACT_SWIGLU || act == SMOE_ACT_SILU ? PW_SILU
+         : act == SMOE_ACT_GEGLU || act == SMOE_ACT_GELU ? PW_GELU
+         : act == SMOE_ACT_REGLU || act == SMOE_ACT_RELU ? PW_RELU
+                                                         : PW_RELU_SQ;
+}
+
+template <int PW>
+SMOE_DEV float pointwise(float t) {
+  if constexpr (PW == PW_SILU) return t * fast_sigmoid(t);
+  else if constexpr (PW == PW_GELU) return t * (0.5f + 0.5f * erff(t * 0.70710678f));
+  else if constexpr (PW == PW_RELU) return fmaxf(t, 0.f);
+  else { const float r = fmaxf(t, 0.f); return r * r; }
+}
+
+// f(t) and f'(t)
+template <int PW>
+SMOE_DEV void pointwise_grad(float t, float& f, float& fp) {
+  if constexpr (PW == PW_SILU) {
+    const float sig = fast_sigmoid(t);
+    f = t * sig;
+    fp = f * (1.f - sig) + sig;
+  } else if constexpr (PW == PW_GELU) {
+    const float cdf = 0.5f + 0.5f * erff(t * 0.70710678f);
+    f = t * cdf;
+    fp = cdf + t * (0.39894228f * __expf(-0.5f * t * t));
+  } else if constexpr (PW == PW_RELU) {
+    f = fmaxf(t, 0.f);
+    fp = t > 0.f ? 1.f : 0.f;
+  } else {
+    const float r = fmaxf(t, 0.f);
+    f = r * r;
+    fp = 2.f * r;
+  }
+}
+
 // ---- tile map ------------------------------------------------------------------------------------------------
 // Built on the device from the expert offsets; header[0] = number of token tiles.  Entry i = (expert, first row).
 struct TileMap {
@@ -252,5 +293,13 @@ SMOE_DEV int64_t xcd_linear_tile(int64_t total) {
 }
 
 int launch_ds_finalize(const float* ds_partial, int ncols, const int32_t* sidx, float* ds, int64_t TK, hipStream_t st);
+
+// out[e][c] = sum_{m in [off[e], off[e+1])} w_m * src[row(m)][c]  (bf16 out, fp32 accumulate, zeros for empty experts);
+// row(m) = gidx[m] or m, w_m = scores[sidx[m]] or 1.  The per-expert bias gradients db1 (src = dz) and db2 (src = dout).
+int launch_expert_colsum(const uint16_t* src, int64_t src_stride, int ncols, const int32_t* gidx, const float* scores,
+                         const int32_t* sidx, const int32_t* off, int E, uint16_t* out, hipStream_t st);
+// ds[sidx[m]] += <dout[gidx[m]], b2[e(m)]>: the bias term of the score gradient
+int launch_ds_bias_term(const uint16_t* dout, const uint16_t* b2, const int32_t* gidx, const int32_t* sidx,
+                        const int32_t* off, int E, int H, float* ds, int64_t TK, hipStream_t st);
 
 }  // namespace smoe

@@ -241,9 +241,9 @@ static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st) {
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
               void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
-              const int32_t* sidx, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st);
+              const int32_t* sidx, int64_t TK, int H, int I, int E, int activation, void* workspace, hipStream_t st);
 int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
-              const int32_t* off, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st);
+              const int32_t* off, int64_t TK, int H, int N1, int E, void* workspace, hipStream_t st);
 
 }  // namespace smoe
 
@@ -260,27 +260,42 @@ static int check_bwd(int64_t TK, int H, int I, int E, const void* ws, size_t ws_
 }
 
 extern "C" int smoe_down_projection_backward(const void* dout, const void* z, const void* w2, int64_t w2_stride_e,
-                                             int64_t w2_stride_row, void* dw2, int64_t dw2_stride_e,
-                                             int64_t dw2_stride_row, void* dz, void* y1s, float* ds, float* ds_partial,
-                                             const float* scores, const int32_t* off, const int32_t* x_gather_idx,
-                                             const int32_t* s_scatter_idx, int64_t T, int64_t TK, int H, int I, int E,
-                                             int activation, void* workspace, size_t workspace_bytes, void* stream) {
+                                             int64_t w2_stride_row, const void* b2, void* dw2, int64_t dw2_stride_e,
+                                             int64_t dw2_stride_row, void* db2, void* dz, void* y1s, float* ds,
+                                             float* ds_partial, const float* scores, const int32_t* off,
+                                             const int32_t* x_gather_idx, const int32_t* s_scatter_idx, int64_t T,
+                                             int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                             size_t workspace_bytes, void* stream) {
   int rc = check_bwd(TK, H, I, E, workspace, workspace_bytes, "down_projection_backward");
   if (rc) return rc;
-  SMOE_REQUIRE(activation == SMOE_ACT_SWIGLU, SMOE_ERR_UNSUPPORTED,
-               "down_projection_backward: only SwiGLU is implemented (activation=%d)", activation);
+  SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
+               "down_projection_backward: unknown activation code %d", activation);
   SMOE_REQUIRE(off, SMOE_ERR_INVALID, "down_projection_backward: null pointer");
-  SMOE_REQUIRE(dz || dw2, SMOE_ERR_INVALID, "down_projection_backward: nothing to compute (dz and dw2 are both null)");
-  SMOE_REQUIRE(TK == 0 || (dout && y1s && x_gather_idx), SMOE_ERR_INVALID, "down_projection_backward: null pointer");
-  SMOE_REQUIRE(TK == 0 || !dz || (z && w2 && ds && ds_partial && scores && s_scatter_idx), SMOE_ERR_INVALID,
+  SMOE_REQUIRE(dz || dw2 || db2, SMOE_ERR_INVALID,
+               "down_projection_backward: nothing to compute (dz, dw2 and db2 are all null)");
+  SMOE_REQUIRE(TK == 0 || (dout && x_gather_idx && (!dw2 || y1s)), SMOE_ERR_INVALID,
                "down_projection_backward: null pointer");
+  SMOE_REQUIRE(TK == 0 || !dz || (z && w2 && y1s && ds && ds_partial && scores && s_scatter_idx), SMOE_ERR_INVALID,
+               "down_projection_backward: null pointer");
+  SMOE_REQUIRE(!db2 || (scores && s_scatter_idx), SMOE_ERR_INVALID,
+               "down_projection_backward: db2 needs scores and s_scatter_idx");
   (void)T;
   hipStream_t st = (hipStream_t)stream;
   if (TK > 0 && dz) {
     rc = launch_dz(dout, z, w2, w2_stride_e, w2_stride_row, dz, y1s, ds_partial, scores, off, x_gather_idx,
-                   s_scatter_idx, TK, H, I, E, workspace, st);
+                   s_scatter_idx, TK, H, I, E, activation, workspace, st);
     if (rc) return rc;
     rc = launch_ds_finalize(ds_partial, smoe_dz_partial_cols(I), s_scatter_idx, ds, TK, st);
+    if (rc) return rc;
+    if (b2) {  // y2 = y1 W2^T + b2 puts <dout, b2> into the score gradient
+      rc = launch_ds_bias_term((const uint16_t*)dout, (const uint16_t*)b2, x_gather_idx, s_scatter_idx, off, E, H, ds,
+                               TK, st);
+      if (rc) return rc;
+    }
+  }
+  if (db2) {
+    rc = launch_expert_colsum((const uint16_t*)dout, H, H, x_gather_idx, scores, s_scatter_idx, off, E,
+                              (uint16_t*)db2, st);
     if (rc) return rc;
   }
   if (!dw2) return SMOE_OK;
@@ -302,24 +317,29 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
 
 extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
                                            const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row,
-                                           void* dx_expanded, const int32_t* off, const int32_t* x_gather_idx,
-                                           int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
-                                           size_t workspace_bytes, void* stream) {
+                                           void* db1, void* dx_expanded, const int32_t* off,
+                                           const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                           int activation, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_bwd(TK, H, I, E, workspace, workspace_bytes, "up_projection_backward");
   if (rc) return rc;
-  SMOE_REQUIRE(activation == SMOE_ACT_SWIGLU, SMOE_ERR_UNSUPPORTED,
-               "up_projection_backward: only SwiGLU is implemented (activation=%d)", activation);
+  SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
+               "up_projection_backward: unknown activation code %d", activation);
   SMOE_REQUIRE(off, SMOE_ERR_INVALID, "up_projection_backward: null pointer");
-  SMOE_REQUIRE(dw1 || dx_expanded, SMOE_ERR_INVALID,
-               "up_projection_backward: nothing to compute (dw1 and dx_expanded are both null)");
+  SMOE_REQUIRE(dw1 || dx_expanded || db1, SMOE_ERR_INVALID,
+               "up_projection_backward: nothing to compute (dw1, db1 and dx_expanded are all null)");
   SMOE_REQUIRE(TK == 0 || (dz && x_gather_idx && (!dw1 || x) && (!dx_expanded || w1)), SMOE_ERR_INVALID,
                "up_projection_backward: null pointer");
   (void)T;
   hipStream_t st = (hipStream_t)stream;
+  const int N1 = activation <= SMOE_ACT_REGLU ? 2 * I : I;  // columns of z and dz: (gate, up) pairs when gated
+  if (db1) {
+    rc = launch_expert_colsum((const uint16_t*)dz, N1, N1, nullptr, nullptr, nullptr, off, E, (uint16_t*)db1, st);
+    if (rc) return rc;
+  }
   if (dw1) {
     VarlenKParams p = {};
     p.R = (const uint16_t*)dz;
-    p.r_stride = 2 * I;
+    p.r_stride = N1;
     p.S = (const uint16_t*)x;
     p.s_stride = H;
     p.gidx = x_gather_idx;
@@ -327,14 +347,14 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     p.out = (uint16_t*)dw1;
     p.out_stride_e = dw1_stride_e;
     p.out_stride_row = dw1_stride_row;
-    p.NA = 2 * I;
+    p.NA = N1;
     p.NB = H;
     p.E = E;
     rc = launch_varlen_k_variant<false, true>(p, st);
     if (rc) return rc;
   }
   if (TK > 0 && dx_expanded) {
-    rc = launch_dx(dz, w1, w1_stride_e, w1_stride_row, dx_expanded, off, TK, H, I, E, workspace, st);
+    rc = launch_dx(dz, w1, w1_stride_e, w1_stride_row, dx_expanded, off, TK, H, N1, E, workspace, st);
     if (rc) return rc;
   }
   return SMOE_OK;

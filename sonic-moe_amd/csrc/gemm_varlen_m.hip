@@ -1,12 +1,10 @@
 // Grouped GEMM over ragged token groups ("varlen-M"): for every expert e and every grouped row m of that expert
 //     C[m, n] = sum_k P[row(m), k] * Q_e[n, k]
 // with fused epilogues.  Four roles of the MoE layer share the main loop:
-//   up-projection forward    P = x rows gathered by x_gather_idx, Q = W1[e] (K-major)   -> z, y1 = SwiGLU(z)
-//   down-projection forward  P = y1 rows,                          Q = W2[e] (K-major)   -> y2
+//   up-projection forward    P = x rows gathered by x_gather_idx, Q = W1[e] (K-major)   -> z (+b1), y1 = act(z)
+//   down-projection forward  P = y1 rows,                          Q = W2[e] (K-major)   -> y2 (+b2)
 //   down-proj activation grad P = dout rows gathered,              Q = W2[e] (MN-major)  -> dz, y1s, ds partials
 //   up-proj activation grad  P = dz rows,                          Q = W1[e] (MN-major)  -> dx_expanded
-#include <stdlib.h>
-
 #include "gemm_common.h"
 
 namespace smoe {
@@ -26,6 +24,7 @@ struct VarlenMParams {
   int64_t out0_stride;
   uint16_t* out1;
   int64_t out1_stride;
+  const uint16_t* bias;  // nullable: (E, N) added to the accumulator before the epilogue
   const uint16_t* zin;
   int64_t zin_stride;
   const float* scores;
@@ -60,8 +59,12 @@ struct Cfg {
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
-template <class C, int ROLE>
+// ACT (an smoe_activation) matters to ROLE_UP_FWD and ROLE_DZ only.  p.N counts accumulator columns: the z columns
+// (2I gated, I otherwise) for ROLE_UP_FWD, the y1 columns I for ROLE_DZ.
+template <class C, int ROLE, int ACT>
 __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) {
+  constexpr bool GLU = act_is_glu(ACT);
+  constexpr int PW = act_pointwise(ACT);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
   const uint32_t smem_base = lds_address(smem);
@@ -196,6 +199,24 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #endif
 
   if constexpr (ROLE == ROLE_PLAIN || ROLE == ROLE_UP_FWD) {
+    if (p.bias != nullptr) {
+      // register quad (fn, rg) of a lane holds columns n_base + fn*32 + 8*rg + 4*(lane>>5) + 0..3 of every fragment row
+      const uint16_t* be = p.bias + (int64_t)e * p.N;
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        int n = n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
+        n = n <= p.N - 4 ? n : p.N - 4;
+        const u32x2 b = *(const u32x2*)(be + n);
+        const float b0 = bf16_lo(b[0]), b1 = bf16_hi(b[0]), b2 = bf16_lo(b[1]), b3 = bf16_hi(b[1]);
+        static_for<FM>([&](auto fm_c) {
+          constexpr int fm = decltype(fm_c)::value;
+          acc[fn][fm][4 * rg + 0] += b0;
+          acc[fn][fm][4 * rg + 1] += b1;
+          acc[fn][fm][4 * rg + 2] += b2;
+          acc[fn][fm][4 * rg + 3] += b3;
+        });
+      });
+    }
     // ---- epilogue through LDS: every wave parks its tile in its own region, then stores 16 B per lane ----
     using LZ = EpiLayout<C::TN>;
     using LY = EpiLayout<C::TN / 2>;
@@ -214,34 +235,49 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       });
       epilogue_flush<C::TM, C::TN>(region, lane, p.out0, p.out0_stride, m_base, row_end, n_base, p.N);
     }
-    if constexpr (ROLE == ROLE_UP_FWD) {
+    if constexpr (ROLE == ROLE_UP_FWD && GLU) {
       static_for<FM>([&](auto fm_c) {
         constexpr int fm = decltype(fm_c)::value;
         static_for<FN * 4>([&](auto q_c) {
           constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
           const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
           const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
-          const uint32_t v = pack_bf16x2(g0 * fast_sigmoid(g0) * u0, g1 * fast_sigmoid(g1) * u1);
+          const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
           *(uint32_t*)(region + (fm * 32 + (lane & 31)) * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * (lane >> 5)) * 2) = v;
         });
       });
       epilogue_flush<C::TM, C::TN / 2>(region, lane, p.out1, p.out1_stride, m_base, row_end, n_base / 2, p.N / 2);
+    } else if constexpr (ROLE == ROLE_UP_FWD) {
+      static_for<FM>([&](auto fm_c) {
+        constexpr int fm = decltype(fm_c)::value;
+        static_for<FN * 4>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+          u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
+                     pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
+          *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+        });
+      });
+      epilogue_flush<C::TM, C::TN>(region, lane, p.out1, p.out1_stride, m_base, row_end, n_base, p.N);
     }
   } else {
     // ---- dz epilogue ----
-    // acc = dy1[i][m].  Per 32-row fragment row the wavefront stages its z sub-tile (32 x 2*TN bf16) through LDS:
-    // row-contiguous 16-byte global loads (two fragment rows in flight in registers) -> LDS -> each lane picks the
-    // four (gate, up) pairs of its token row, computes dz in place and y1s into a second area -> both are written back
+    // acc = dy1[i][m].  Per 32-row fragment row the wavefront stages its z sub-tile (32 rows x ZW*TN bf16; ZW = 2
+    // interleaved (gate, up) columns per dy1 column for gated activations, 1 otherwise) through LDS: row-contiguous
+    // 16-byte global loads (two fragment rows in flight in registers) -> LDS -> each lane picks the z values of its four
+    // dy1 columns of its token row, computes dz in place and y1s into a second area -> both are written back
     // row-contiguous.  All global traffic of the epilogue is full 128-byte lines.
-    constexpr int ZB = C::TN * 4, YB = C::TN * 2;            // bytes per staged z/dz row, y1s row
+    constexpr int ZW = GLU ? 2 : 1;
+    constexpr int ZB = C::TN * 2 * ZW, YB = C::TN * 2;       // bytes per staged z/dz row, y1s row
     constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
     constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
+    constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;               // row swizzle of the staged z chunks
     static_assert(C::NW * 32 * (ZB + YB) <= NSTAGE * C::STAGE, "dz staging must fit into the idle ring");
     char* zbuf = smem + wave * (32 * (ZB + YB));
     char* ybuf = zbuf + 32 * ZB;
     const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
-    const int zcol = 2 * n_base + zc * 8;  // first z column of this lane's 16-byte chunk
-    const int zcol_c = zcol <= 2 * p.N - 8 ? zcol : 2 * p.N - 8;
+    const int zlimit = ZW * p.N;
+    const int zcol = ZW * n_base + zc * 8;  // first z column of this lane's 16-byte chunk
+    const int zcol_c = zcol <= zlimit - 8 ? zcol : zlimit - 8;
     u32x4 zreg[2][ZN];
     auto fetch_z = [&](int fm, u32x4(&dst)[ZN]) {
 #pragma unroll
@@ -260,7 +296,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int it = 0; it < ZN; it++) {
         const int r = it * ZR + zr;
-        *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & 15)) << 4)) = zreg[fm & 1][it];
+        *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4)) = zreg[fm & 1][it];
       }
       if constexpr (fm + 2 < FM) fetch_z(fm + 2, zreg[fm & 1]);
       const int mrow = lane & 31;
@@ -270,24 +306,41 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       if (mvalid) sc = p.scores[p.sidx[m]];
       static_for<FN * 4>([&](auto q_c) {
         constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        const int il = fn * 32 + 8 * rg + 4 * (lane >> 5);  // first of this lane's 4 intermediate features (wave-local)
-        char* zaddr = zbuf + mrow * ZB + ((((il * 4) >> 4) ^ (mrow & 15)) << 4);
-        const u32x4 zz = *(const u32x4*)zaddr;
-        u32x4 dzv;
+        const int il = fn * 32 + 8 * rg + 4 * (lane >> 5);  // first of this lane's 4 dy1 columns (wave-local)
+        const int zbyte = il * 2 * ZW;                      // their z bytes inside the staged row
+        char* zaddr = zbuf + mrow * ZB + (((zbyte >> 4) ^ (mrow & ZSW)) << 4) + (zbyte & 15);
         float ys[4];
+        if constexpr (GLU) {
+          const u32x4 zz = *(const u32x4*)zaddr;
+          u32x4 dzv;
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-          const float dy = acc[fn][fm][4 * rg + q];
-          const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
-          const float sig = fast_sigmoid(g);
-          const float silu = g * sig;
-          const float y1v = silu * u;
-          if (n_base + il + q < p.N) dsum += dy * y1v;
-          const float sd = sc * dy;
-          dzv[q] = pack_bf16x2(sd * u * (silu * (1.f - sig) + sig), sd * silu);
-          ys[q] = sc * y1v;
+          for (int q = 0; q < 4; q++) {
+            const float dy = acc[fn][fm][4 * rg + q];
+            const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
+            float f, fp;
+            pointwise_grad<PW>(g, f, fp);
+            const float y1v = f * u;
+            if (n_base + il + q < p.N) dsum += dy * y1v;
+            const float sd = sc * dy;
+            dzv[q] = pack_bf16x2(sd * u * fp, sd * f);
+            ys[q] = sc * y1v;
+          }
+          *(u32x4*)zaddr = dzv;
+        } else {
+          const u32x2 zz = *(const u32x2*)zaddr;
+          float dzf[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float dy = acc[fn][fm][4 * rg + q];
+            const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
+            float f, fp;
+            pointwise_grad<PW>(t, f, fp);
+            if (n_base + il + q < p.N) dsum += dy * f;
+            dzf[q] = sc * dy * fp;
+            ys[q] = sc * f;
+          }
+          *(u32x2*)zaddr = u32x2{pack_bf16x2(dzf[0], dzf[1]), pack_bf16x2(dzf[2], dzf[3])};
         }
-        *(u32x4*)zaddr = dzv;
         u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
         epi_park_y<YB>(ybuf, mrow, il * 2, yv);
       });
@@ -296,9 +349,9 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int it = 0; it < ZN; it++) {
         const int r = it * ZR + zr;
-        const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & 15)) << 4));
+        const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4));
         const int mm = m_base + fm * 32 + r;
-        if (mm < row_end && zcol < 2 * p.N) *(u32x4*)(p.out0 + (int64_t)mm * p.out0_stride + zcol) = v;
+        if (mm < row_end && zcol < zlimit) *(u32x4*)(p.out0 + (int64_t)mm * p.out0_stride + zcol) = v;
       }
 #pragma unroll
       for (int it = 0; it < YN; it++) {
@@ -311,14 +364,19 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   }
 }
 
-template <class C, int ROLE>
-static int launch_varlen_m(const VarlenMParams& p, int64_t TK, int E, hipStream_t st) {
+template <class C, int ROLE, int ACT>
+static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
   static bool attr_set = false;
-  auto kern = varlen_m_kernel<C, ROLE>;
+  auto kern = varlen_m_kernel<C, ROLE, ACT>;
   if (!attr_set) {
     SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
     attr_set = true;
   }
+  p.tm = carve_tile_map(workspace, TK, E, C::BM);
+  int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
+  if (rc) return rc;
+  p.n_tiles = (int)ceil_div(p.N, C::BN);
+  if (ROLE == ROLE_DZ) p.ds_cols = p.n_tiles * C::WN;
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
@@ -327,53 +385,29 @@ static int launch_varlen_m(const VarlenMParams& p, int64_t TK, int E, hipStream_
   return SMOE_OK;
 }
 
-// tile configurations ------------------------------------------------------------------------------------------
-// SMOE_GEMM_VARIANT (environment, read once) picks the tile configuration of the varlen-M kernels; 3 is the default.
+// 256 x 256 tile, 8 wavefronts as 2 (token) x 4 (feature), 64 of the contraction per stage, double buffer
 template <bool QMN>
-using CfgV0 = Cfg<256, 256, 2, 2, QMN, 32, 5>;  // 4 waves, BK 32, 5-stage ring
-template <bool QMN>
-using CfgV1 = Cfg<256, 256, 2, 2, QMN, 64, 2>;  // 4 waves, BK 64, double buffer
-template <bool QMN>
-using CfgV2 = Cfg<256, 256, 2, 4, QMN, 32, 5>;  // 8 waves (2 per SIMD), BK 32, 5-stage ring
-template <bool QMN>
-using CfgV3 = Cfg<256, 256, 2, 4, QMN, 64, 2>;  // 8 waves, BK 64, double buffer
+using TileCfg = Cfg<256, 256, 2, 4, QMN, 64, 2>;
 
-int gemm_variant() {
-  static int v = -1;
-  if (v < 0) {
-    const char* e = getenv("SMOE_GEMM_VARIANT");
-    v = e ? atoi(e) : 3;
-    if (v < 0 || v > 3) v = 3;
-  }
-  return v;
-}
-
+// one kernel per activation: the epilogue math and (gated or not) the tile geometry of z / y1 depend on it
 template <bool QMN, int ROLE>
-static int launch_varlen_m_variant(VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E,
-                                   hipStream_t st) {
-  auto go = [&](auto cfg) {
-    using C = decltype(cfg);
-    p.tm = carve_tile_map(workspace, TK, E, C::BM);
-    int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
-    if (rc) return rc;
-    p.n_tiles = (int)ceil_div(p.N, C::BN);
-    if (ROLE == ROLE_DZ) p.ds_cols = p.n_tiles * C::WN;
-    return launch_varlen_m<C, ROLE>(p, TK, E, st);
-  };
-  switch (gemm_variant()) {
-    case 0: return go(CfgV0<QMN>{});
-    case 1: return go(CfgV1<QMN>{});
-    case 2: return go(CfgV2<QMN>{});
-    default: return go(CfgV3<QMN>{});
+static int launch_by_activation(int act, VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E,
+                                hipStream_t st) {
+  switch (act) {
+    case SMOE_ACT_SWIGLU: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
+    case SMOE_ACT_GEGLU: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_GEGLU>(p, off, workspace, TK, E, st);
+    case SMOE_ACT_REGLU: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_REGLU>(p, off, workspace, TK, E, st);
+    case SMOE_ACT_RELU_SQ: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_RELU_SQ>(p, off, workspace, TK, E, st);
+    case SMOE_ACT_RELU: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_RELU>(p, off, workspace, TK, E, st);
+    case SMOE_ACT_GELU: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_GELU>(p, off, workspace, TK, E, st);
+    case SMOE_ACT_SILU: return launch_varlen_m<TileCfg<QMN>, ROLE, SMOE_ACT_SILU>(p, off, workspace, TK, E, st);
   }
+  set_error("unknown activation code %d", act);
+  return SMOE_ERR_INVALID;
 }
 
-int dz_wave_cols() {
-  switch (gemm_variant()) {
-    case 0: case 1: return 2;
-    default: return 4;
-  }
-}
+int dz_wave_cols() { return TileCfg<true>::WN; }
+int dz_tile_cols() { return TileCfg<true>::BN; }
 
 }  // namespace smoe
 
@@ -394,16 +428,16 @@ extern "C" size_t smoe_gemm_workspace_bytes(int64_t TK, int E) {
   return tile_map_bytes(TK, E);
 }
 
-extern "C" int smoe_dz_partial_cols(int I) { return (int)ceil_div(I, 256) * dz_wave_cols(); }
+extern "C" int smoe_dz_partial_cols(int I) { return (int)ceil_div(I, dz_tile_cols()) * dz_wave_cols(); }
 
 extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
-                                          void* z, void* y1, const int32_t* off, const int32_t* x_gather_idx,
-                                          int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
-                                          size_t workspace_bytes, void* stream) {
+                                          const void* b1, void* z, void* y1, const int32_t* off,
+                                          const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                          int activation, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "up_projection_forward");
   if (rc) return rc;
-  SMOE_REQUIRE(activation == SMOE_ACT_SWIGLU, SMOE_ERR_UNSUPPORTED,
-               "up_projection_forward: only SwiGLU is implemented (activation=%d)", activation);
+  SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
+               "up_projection_forward: unknown activation code %d", activation);
   if (TK == 0) return SMOE_OK;
   SMOE_REQUIRE(x && w1 && y1 && off && x_gather_idx, SMOE_ERR_INVALID, "up_projection_forward: null pointer");
   SMOE_REQUIRE(T > 0, SMOE_ERR_INVALID, "up_projection_forward: T must be positive");
@@ -416,18 +450,19 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
   p.off = off;
-  p.N = 2 * I;
+  p.N = act_is_glu(activation) ? 2 * I : I;
   p.Kdim = H;
+  p.bias = (const uint16_t*)b1;
   p.out0 = (uint16_t*)z;
-  p.out0_stride = 2 * I;
+  p.out0_stride = p.N;
   p.out1 = (uint16_t*)y1;
   p.out1_stride = I;
-  return launch_varlen_m_variant<false, ROLE_UP_FWD>(p, off, workspace, TK, E, st);
+  return launch_by_activation<false, ROLE_UP_FWD>(activation, p, off, workspace, TK, E, st);
 }
 
 extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
-                                            void* y2, const int32_t* off, int64_t TK, int H, int I, int E,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+                                            const void* b2, void* y2, const int32_t* off, int64_t TK, int H, int I,
+                                            int E, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "down_projection_forward");
   if (rc) return rc;
   if (TK == 0) return SMOE_OK;
@@ -442,9 +477,10 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
   p.off = off;
   p.N = H;
   p.Kdim = I;
+  p.bias = (const uint16_t*)b2;
   p.out0 = (uint16_t*)y2;
   p.out0_stride = H;
-  return launch_varlen_m_variant<false, ROLE_PLAIN>(p, off, workspace, TK, E, st);
+  return launch_varlen_m<TileCfg<false>, ROLE_PLAIN, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
 }
 
 // activation-gradient halves of the two backward operators; the weight-gradient halves live in gemm_varlen_k.hip
@@ -452,7 +488,8 @@ namespace smoe {
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
               void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
-              const int32_t* sidx, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st) {
+              const int32_t* sidx, int64_t TK, int H, int I, int E, int activation, void* workspace, hipStream_t st) {
+  const int zw = act_is_glu(activation) ? 2 : 1;
   VarlenMParams p = {};
   p.P = (const uint16_t*)dout;
   p.p_stride = H;
@@ -464,31 +501,31 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.N = I;
   p.Kdim = H;
   p.out0 = (uint16_t*)dz;
-  p.out0_stride = 2 * I;
+  p.out0_stride = zw * I;
   p.out1 = (uint16_t*)y1s;
   p.out1_stride = I;
   p.zin = (const uint16_t*)z;
-  p.zin_stride = 2 * I;
+  p.zin_stride = zw * I;
   p.scores = scores;
   p.sidx = sidx;
   p.ds_partial = ds_partial;
-  return launch_varlen_m_variant<true, ROLE_DZ>(p, off, workspace, TK, E, st);
+  return launch_by_activation<true, ROLE_DZ>(activation, p, off, workspace, TK, E, st);
 }
 
 int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
-              const int32_t* off, int64_t TK, int H, int I, int E, void* workspace, hipStream_t st) {
+              const int32_t* off, int64_t TK, int H, int N1, int E, void* workspace, hipStream_t st) {
   VarlenMParams p = {};
   p.P = (const uint16_t*)dz;
-  p.p_stride = 2 * I;
-  p.Q = (const uint16_t*)w1;  // W1[e] is (2I, H): k = j rows, n = h contiguous
+  p.p_stride = N1;
+  p.Q = (const uint16_t*)w1;  // W1[e] is (N1, H): k = j rows, n = h contiguous
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
   p.off = off;
   p.N = H;
-  p.Kdim = 2 * I;
+  p.Kdim = N1;
   p.out0 = (uint16_t*)dx_expanded;
   p.out0_stride = H;
-  return launch_varlen_m_variant<true, ROLE_PLAIN>(p, off, workspace, TK, E, st);
+  return launch_varlen_m<TileCfg<true>, ROLE_PLAIN, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
 }
 
 }  // namespace smoe

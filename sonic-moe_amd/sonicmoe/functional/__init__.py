@@ -138,7 +138,8 @@ class TC_Softmax_Topk_Router_Function(torch.autograd.Function):
 class _ExpertsFunction(torch.autograd.Function):
     """o = combine(down(act(up(gather(x))))) over the routed (token, expert) pairs.
 
-    Differentiable inputs: x (T, H), w1 (2I, H, E) view, w2 (H, I, E) view, scores (flat, fp32).
+    Differentiable inputs: x (T, H), w1 (N1, H, E) view, b1 (E, N1) or None, w2 (H, I, E) view, b2 (E, H) or None,
+    scores (flat, fp32); N1 = 2I for the gated activations, I otherwise.
     """
 
     @staticmethod
@@ -146,7 +147,9 @@ class _ExpertsFunction(torch.autograd.Function):
         ctx,
         x,
         w1,
+        b1,
         w2,
+        b2,
         scores_flat,
         off,
         gidx,
@@ -169,18 +172,16 @@ class _ExpertsFunction(torch.autograd.Function):
 
         z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
         y1 = torch.empty(TK, I, dtype=x.dtype, device=x.device)
-        _up_projection_forward(
-            x, w1, z, y1, None, off, None, gidx, stream_id, activation_type.value, glu, inference
-        )
+        _up_projection_forward(x, w1, z, y1, b1, off, None, gidx, stream_id, activation_type.value, glu, inference)
         y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
-        _down_projection_forward(w2, y1, y2, None, off, None, gidx, stream_id)
+        _down_projection_forward(w2, y1, y2, b2, off, None, gidx, stream_id)
         del y1
         o = torch.empty(T, H, dtype=x.dtype, device=x.device)
         _router_forward(y2, o, scores_flat, ridx, tok_off, K_or_maxK, H, is_varlen_K)
         del y2
 
         if not inference:
-            ctx.save_for_backward(x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
+            ctx.save_for_backward(x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference)
         return o
 
@@ -189,32 +190,35 @@ class _ExpertsFunction(torch.autograd.Function):
         K_or_maxK, is_varlen_K, activation_type, stream_id, inference = ctx.cfg
         if inference:
             raise RuntimeError("backward through an inference-mode MoE forward: z was not stored")
-        x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
+        x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
         T, H = x.shape
         TK = gidx.numel()
         glu = is_glu(activation_type)
         dout = dout.contiguous()
 
         dw2 = torch.empty_like(w2)  # keeps the (E, H, I)-contiguous layout of the parameter view
+        db2 = None if b2 is None else torch.empty_like(b2)
         dz = torch.empty_like(z)
         ds = torch.empty(TK, dtype=torch.float32, device=x.device)
         _down_projection_backward(
-            dout, z, w2, dw2, dz, ds, None, None, scores_flat, off, None, gidx, sidx, stream_id, glu,
+            dout, z, w2, dw2, dz, ds, b2, db2, scores_flat, off, None, gidx, sidx, stream_id, glu,
             activation_type.value,
         )
         dw1 = torch.empty_like(w1)
+        db1 = None if b2 is None else torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device)
         dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
-        _up_projection_backward(x, w1, dx_expanded, dw1, dz, None, off, None, gidx, sidx, glu, stream_id)
+        _up_projection_backward(x, w1, dx_expanded, dw1, dz, db1, off, None, gidx, sidx, glu, stream_id)
         del dz
         dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
         _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
-        return dx, dw1, dw2, ds, None, None, None, None, None, None, None, None, None, None
+        return dx, dw1, db1, dw2, db2, ds, None, None, None, None, None, None, None, None, None, None
 
 
 def _check_bias(b1, b2):
     assert (b1 is None) == (b2 is None), "b1 and b2 has to be None or not None at the same time!"
     if b1 is not None:
-        raise NotImplementedError("expert biases are not implemented in the HIP backend")
+        return b1.contiguous(), b2.contiguous()
+    return None, None
 
 
 def _as_activation(activation_type) -> ActivationType:
@@ -243,14 +247,14 @@ def moe_TC_softmax_topk_layer(
     x (T, H); router_w (E, H); w1 (2I, H, E) and w2 (H, I, E) are permuted views of the (E, out, in) parameters.
     Returns (o (T, H), router_logits (T, E), expert_frequency (E,) int32).
     """
-    _check_bias(b1, b2)
+    b1, b2 = _check_bias(b1, b2)
     activation_type = _as_activation(activation_type)
     T, E = x.size(0), router_w.size(0)
     router_logits = F.linear(x, router_w)
     topk_scores, topk_indices = TC_Softmax_Topk_Router_Function.apply(router_logits, E, K)
     freq, off, gidx, sidx, ridx, tok_off = _build_metadata(topk_indices.view(-1), None, T, E, K)
     o = _ExpertsFunction.apply(
-        x, w1, w2, topk_scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id,
+        x, w1, b1, w2, b2, topk_scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id,
         is_inference_mode_enabled,
     )
     return o, router_logits, freq
@@ -273,13 +277,13 @@ def moe_general_routing_inputs(
     """MoE layer for arbitrary routing (interface of sonicmoe/functional/__init__.py:497-562): pair j sends token
     token_indices[j] (SORTED ascending) to expert expert_indices[j] with weight router_scores[j].
     Returns (o (T, H), expert_frequency (E,) int32); d(router_scores) comes back in the pairs' order."""
-    _check_bias(b1, b2)
+    b1, b2 = _check_bias(b1, b2)
     activation_type = _as_activation(activation_type)
     T = x.size(0)
     E = w2.size(-1)
     freq, off, gidx, sidx, ridx, tok_off = _build_metadata(expert_indices, token_indices, T, E, 1)
     o = _ExpertsFunction.apply(
-        x, w1, w2, router_scores.float(), off, gidx, sidx, ridx, tok_off, E, True, activation_type, stream_id,
+        x, w1, b1, w2, b2, router_scores.float(), off, gidx, sidx, ridx, tok_off, E, True, activation_type, stream_id,
         is_inference_mode_enabled,
     )
     return o, freq

@@ -27,20 +27,17 @@ def _up_projection_backward(
     is_glu_activation: bool,
     stream_id: int,
 ) -> None:
-    """dw1[e] = sum_m dz[m]^T x[t_m] (zeros for empty experts), dx_expanded = dz W1[e]; either output may be None
-    to skip it."""
-    if db1 is not None:
-        raise NotImplementedError("_up_projection_backward: bias is not implemented in the HIP path")
+    """dw1[e] = sum_m dz[m]^T x[t_m], db1[e] = sum_m dz[m] (zeros for empty experts), dx_expanded = dz W1[e]; any
+    output may be None to skip it."""
     if expert_schedule_order is not None:
         raise NotImplementedError("_up_projection_backward: expert_schedule_order is not supported")
-    if not is_glu_activation:
-        raise NotImplementedError("_up_projection_backward: only GLU activations are implemented in the HIP path")
-    _lib.require_device(x, w1, dx_expanded, dw1, dz, expert_frequency_offset, x_gather_idx)
-    _check_bf16(("x", x), ("w1", w1), ("dx_expanded", dx_expanded), ("dw1", dw1), ("dz", dz))
+    _lib.require_device(x, w1, dx_expanded, dw1, db1, dz, expert_frequency_offset, x_gather_idx)
+    _check_bf16(("x", x), ("w1", w1), ("dx_expanded", dx_expanded), ("dw1", dw1), ("db1", db1), ("dz", dz))
     N1, H, E = w1.shape
-    I = N1 // 2
+    I = N1 // 2 if is_glu_activation else N1
     T, TK = x.size(0), dz.size(0)
     assert x.is_contiguous() and dz.is_contiguous() and (dx_expanded is None or dx_expanded.is_contiguous())
+    assert dz.size(1) == N1 and (db1 is None or (db1.shape == (E, N1) and db1.is_contiguous()))
     w_se, w_sr = expert_major_strides(w1, "w1")
     d_se, d_sr = expert_major_strides(dw1, "dw1") if dw1 is not None else (0, 0)
     ws = _gemm_workspace(TK, E, x.device)
@@ -53,6 +50,7 @@ def _up_projection_backward(
         _lib.ptr(dw1),
         d_se,
         d_sr,
+        _lib.ptr(db1),
         _lib.ptr(dx_expanded),
         _lib.ptr(expert_frequency_offset),
         _lib.ptr(x_gather_idx),
@@ -61,7 +59,8 @@ def _up_projection_backward(
         H,
         I,
         E,
-        ACTIVATION_CODE[ActivationType.SWIGLU],
+        # only the column count of dz depends on the activation here: any gated / any plain code will do
+        ACTIVATION_CODE[ActivationType.SWIGLU if is_glu_activation else ActivationType.SILU],
         _lib.ptr(ws),
         ws.numel(),
         stream_id,
@@ -88,15 +87,17 @@ def _down_projection_backward(
     is_glu_activation: bool,
     activation_type: str,
 ) -> None:
-    """dz, ds (flat routing-slot order) and dw2 of the down projection + weighted combine; y1 is recomputed from z and
-    the dout rows are re-gathered, nothing of size (TK, H) is kept from the forward."""
-    if b2 is not None or db2 is not None:
-        raise NotImplementedError("_down_projection_backward: bias is not implemented in the HIP path")
+    """dz, ds (flat routing-slot order), dw2 and db2 of the down projection + weighted combine; y1 is recomputed from z
+    and the dout rows are re-gathered, nothing of size (TK, H) is kept from the forward."""
     if expert_schedule_order is not None:
         raise NotImplementedError("_down_projection_backward: expert_schedule_order is not supported")
-    _lib.require_device(dout, z, w2, dw2, dz, ds, topk_scores, expert_frequency_offset, x_gather_idx, s_scatter_idx)
-    _check_bf16(("dout", dout), ("z", z), ("w2", w2), ("dw2", dw2), ("dz", dz))
+    _lib.require_device(dout, z, w2, dw2, dz, ds, b2, db2, topk_scores, expert_frequency_offset, x_gather_idx,
+                        s_scatter_idx)
+    _check_bf16(("dout", dout), ("z", z), ("w2", w2), ("dw2", dw2), ("dz", dz), ("b2", b2), ("db2", db2))
     H, I, E = w2.shape
+    assert (b2 is None) == (db2 is None), "b2 and db2 have to be given together"
+    assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous() and db2.shape == (E, H) and db2.is_contiguous())
+    assert z.size(1) == (2 * I if is_glu_activation else I)
     T, TK = dout.size(0), x_gather_idx.size(0)
     dout = dout.contiguous()
     assert z.is_contiguous() and dz.is_contiguous() and ds.is_contiguous() and ds.dtype == torch.float32
@@ -113,9 +114,11 @@ def _down_projection_backward(
         _lib.ptr(w2),
         w_se,
         w_sr,
+        _lib.ptr(b2),
         _lib.ptr(dw2),
         d_se,
         d_sr,
+        _lib.ptr(db2),
         _lib.ptr(dz),
         _lib.ptr(y1s),
         _lib.ptr(ds),

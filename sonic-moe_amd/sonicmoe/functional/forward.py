@@ -74,17 +74,17 @@ def _up_projection_forward(
     is_glu_activation: bool,
     is_inference_mode_enabled: bool = False,
 ) -> None:
-    """z = gather(x) W1^T, y1 = act(z); w1 is the (2I, H, E) view of the (E, 2I, H) parameter."""
-    if b1 is not None:
-        raise NotImplementedError("_up_projection_forward: bias is not implemented in the HIP path")
+    """z = gather(x) W1^T (+ b1), y1 = act(z); w1 is the (N1, H, E) view of the (E, N1, H) parameter, N1 = 2I for the
+    gated activations and I otherwise; b1 is (E, N1)."""
     if expert_schedule_order is not None:
         raise NotImplementedError("_up_projection_forward: expert_schedule_order is not supported")
-    _lib.require_device(x, w1, y1, expert_frequency_offset, x_gather_idx)
-    _check_bf16(("x", x), ("w1", w1), ("z", z), ("y1", y1))
+    _lib.require_device(x, w1, y1, b1, expert_frequency_offset, x_gather_idx)
+    _check_bf16(("x", x), ("w1", w1), ("z", z), ("y1", y1), ("b1", b1))
     N1, H, E = w1.shape
     I = N1 // 2 if is_glu_activation else N1
     T, TK = x.size(0), y1.size(0)
     assert x.is_contiguous() and y1.is_contiguous() and (z is None or z.is_contiguous())
+    assert b1 is None or (b1.shape == (E, N1) and b1.is_contiguous())
     s_e, s_row = expert_major_strides(w1, "w1")
     ws = _gemm_workspace(TK, E, x.device)
     rc = _lib.lib().smoe_up_projection_forward(
@@ -92,6 +92,7 @@ def _up_projection_forward(
         _lib.ptr(w1),
         s_e,
         s_row,
+        _lib.ptr(b1),
         None if is_inference_mode_enabled else _lib.ptr(z),
         _lib.ptr(y1),
         _lib.ptr(expert_frequency_offset),
@@ -120,16 +121,15 @@ def _down_projection_forward(
     x_gather_idx: torch.Tensor,
     stream_id: int,
 ) -> None:
-    """y2 = y1 W2^T per expert; w2 is the (H, I, E) view of the (E, H, I) parameter."""
-    if b2 is not None:
-        raise NotImplementedError("_down_projection_forward: bias is not implemented in the HIP path")
+    """y2 = y1 W2^T (+ b2) per expert; w2 is the (H, I, E) view of the (E, H, I) parameter, b2 is (E, H)."""
     if expert_schedule_order is not None:
         raise NotImplementedError("_down_projection_forward: expert_schedule_order is not supported")
-    _lib.require_device(w2, y1, y2, expert_frequency_offset)
-    _check_bf16(("w2", w2), ("y1", y1), ("y2", y2))
+    _lib.require_device(w2, y1, y2, b2, expert_frequency_offset)
+    _check_bf16(("w2", w2), ("y1", y1), ("y2", y2), ("b2", b2))
     H, I, E = w2.shape
     TK = y1.size(0)
     assert y1.is_contiguous() and y2.is_contiguous()
+    assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous())
     s_e, s_row = expert_major_strides(w2, "w2")
     ws = _gemm_workspace(TK, E, y1.device)
     rc = _lib.lib().smoe_down_projection_forward(
@@ -137,6 +137,7 @@ def _down_projection_forward(
         _lib.ptr(w2),
         s_e,
         s_row,
+        _lib.ptr(b2),
         _lib.ptr(y2),
         _lib.ptr(expert_frequency_offset),
         TK,

@@ -38,7 +38,7 @@ def test_header_and_binding_agree(lib):
 
 
 def test_version_and_error_text(lib):
-    assert lib.smoe_version() >= 100
+    assert lib.smoe_version() >= 200
     assert isinstance(lib.smoe_last_error(), bytes)
 
 
@@ -53,12 +53,16 @@ def test_argument_checks_return_status_codes(lib):
     # K > E
     assert lib.smoe_topk_softmax_fwd(p, 0, 4, 8, 9, 8, p, p, 1, None) == 2
     # H not a multiple of 64
-    assert lib.smoe_up_projection_forward(p, p, 0, 0, p, p, p, p, 4, 8, 96, 64, 2, 0, p, 1 << 20, None) == 2
+    assert lib.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, p, 4, 8, 96, 64, 2, 0, p, 1 << 20, None) == 2
     assert b"multiple of 64" in lib.smoe_last_error()
     # workspace too small
-    assert lib.smoe_down_projection_forward(p, p, 0, 0, p, p, 1 << 20, 64, 64, 2, p, 8, None) == 4
-    # unsupported activation
-    assert lib.smoe_up_projection_forward(p, p, 0, 0, p, p, p, p, 4, 8, 64, 64, 2, 5, p, 1 << 20, None) == 2
+    assert lib.smoe_down_projection_forward(p, p, 0, 0, None, p, p, 1 << 20, 64, 64, 2, p, 8, None) == 4
+    # activation code outside the enum -> SMOE_ERR_INVALID
+    assert lib.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, p, 4, 8, 64, 64, 2, 7, p, 1 << 20, None) == 1
+    assert b"activation" in lib.smoe_last_error()
+    # a backward call with every output null has nothing to do
+    assert lib.smoe_up_projection_backward(p, p, 0, 0, p, None, 0, 0, None, None, p, p, 4, 8, 64, 64, 2, 0, p, 1 << 20,
+                                           None) == 1
     # workspace size queries are pure host functions
     assert lib.smoe_gemm_workspace_bytes(262144, 128) > 0
     assert lib.smoe_routing_metadata_workspace_bytes(262144, 128) == 2 * 128 * 256 * 4

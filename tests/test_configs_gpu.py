@@ -34,8 +34,8 @@ def test_zipf_skewed_load_with_empty_experts(dev):
     freq, off, gidx, sidx, ridx, tok_off = _build_metadata(i.view(-1), None, T, E, K)
     assert int((freq == 0).sum()) > 0, "the skew should leave some experts empty"
     assert int(freq.max()) > 4 * T * K // E
-    o = _ExpertsFunction.apply(x, w1.permute(1, 2, 0), w2.permute(1, 2, 0), s.view(-1), off, gidx, sidx, ridx, tok_off,
-                               K, False, ActivationType.SWIGLU, torch.cuda.current_stream().cuda_stream, False)
+    o = _ExpertsFunction.apply(x, w1.permute(1, 2, 0), None, w2.permute(1, 2, 0), None, s.view(-1), off, gidx, sidx, ridx,
+                               tok_off, K, False, ActivationType.SWIGLU, torch.cuda.current_stream().cuda_stream, False)
     grads = torch.autograd.grad(o, [x, wr, w1, w2], grad_outputs=dy)
 
     # routing bit-exact against the oracle on the same logits

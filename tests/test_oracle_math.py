@@ -65,6 +65,71 @@ def test_explicit_backward_matches_autograd():
     torch.testing.assert_close(y1s, scores.reshape(-1)[sidx.long()][:, None] * M.swiglu(z.detach()), **kw)
 
 
+ALL_ACTIVATIONS = ["swiglu", "geglu", "reglu", "relu_sq", "relu", "gelu", "silu"]
+
+
+@pytest.mark.parametrize("activation", ALL_ACTIVATIONS)
+def test_activation_forms(activation):
+    """activation_forward reduces to the library routines the reference's torch backend calls (moe.py:24-60); the
+    hand-written derivative equals autograd's, and the gated forms split gate = even / up = odd columns."""
+    g = torch.Generator().manual_seed(1)
+    z = torch.randn(7, 12, generator=g, dtype=D)
+    z[0, 0] = 0.25  # keep clear of the kink of relu at 0
+    lib = {"swiglu": F.silu, "geglu": F.gelu, "reglu": F.relu, "relu_sq": lambda t: F.relu(t).square(),
+           "relu": F.relu, "gelu": F.gelu, "silu": F.silu}[activation]
+    y = M.activation_forward(z, activation)
+    if M.is_glu(activation):
+        assert y.shape == (7, 6)
+        torch.testing.assert_close(y, lib(z[:, 0::2]) * z[:, 1::2], rtol=1e-12, atol=1e-12)
+    else:
+        assert y.shape == z.shape
+        torch.testing.assert_close(y, lib(z), rtol=1e-12, atol=1e-12)
+    zr = z.clone().requires_grad_()
+    dy = torch.randn(y.shape, generator=g, dtype=D)
+    (gz,) = torch.autograd.grad(M.activation_forward(zr, activation), zr, grad_outputs=dy)
+    dz, y_again = M.activation_backward(z, dy, activation)
+    torch.testing.assert_close(dz, gz, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(y_again, y, rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("activation", ALL_ACTIVATIONS)
+def test_explicit_backward_with_bias_and_activation(activation):
+    """dz, ds, dW2, db2, dW1, db1, dx with expert biases, for every activation == autograd of the operator chain."""
+    glu = M.is_glu(activation)
+    x, w1, w2, wr, idx, meta, scores, dout = _problem(seed=4)
+    if not glu:
+        w1 = w1[:, : w1.size(1) // 2].contiguous()  # (E, I, H)
+    E, N1, H = w1.shape
+    g = torch.Generator().manual_seed(8)
+    b1 = torch.randn(E, N1, generator=g, dtype=D) * 0.2
+    b2 = torch.randn(E, H, generator=g, dtype=D) * 0.2
+    off, gidx, sidx, ridx, tok_off = (meta[k] for k in ("expert_frequency_offset", "x_gather_idx", "s_scatter_idx",
+                                                        "s_reverse_scatter_idx", "num_activated_expert_per_token_offset"))
+    xr, w1r, w2r, sr, b1r, b2r = (t.clone().requires_grad_() for t in (x, w1, w2, scores, b1, b2))
+    z, y1 = M.up_projection_forward(xr, w1r, off, gidx, b1=b1r, math_dtype=D, activation=activation)
+    y2 = M.down_projection_forward(y1, w2r, off, b2=b2r, math_dtype=D)
+    o = M.router_forward(y2, sr.reshape(-1), ridx, tok_off, math_dtype=D)
+    gx, gw1, gw2, gs, gz, gb1, gb2 = torch.autograd.grad(o, [xr, w1r, w2r, sr, z, b1r, b2r], grad_outputs=dout)
+
+    dz, y1s, ds, dw2, db2 = M.down_projection_backward(dout, z.detach(), w2, scores.reshape(-1), off, gidx, sidx,
+                                                       math_dtype=D, b2=b2, activation=activation)
+    dw1, dxe, db1 = M.up_projection_backward(x, w1, dz, off, gidx, math_dtype=D, with_db1=True)
+    dx = M.token_broadcast_backward(dxe, ridx, tok_off, math_dtype=D)
+    kw = dict(rtol=1e-9, atol=1e-11)
+    for name, a, b in [("dz", dz, gz), ("ds", ds.view_as(gs), gs), ("dw2", dw2, gw2), ("db2", db2, gb2),
+                       ("dw1", dw1, gw1), ("db1", db1, gb1), ("dx", dx, gx)]:
+        torch.testing.assert_close(a, b, msg=lambda m, n=name: f"{n}: {m}", **kw)
+
+    # the layer-level restatement with the same biases and activation is the same function
+    out_ref, logits, _ = M.moe_torch_backend(x, wr, w1, w2, idx.shape[1], b1=b1, b2=b2,
+                                             selected_experts=torch.from_numpy(idx), math_dtype=D, gate_dtype=D,
+                                             activation=activation)
+    gates = F.softmax(logits.gather(1, torch.from_numpy(idx).long()), dim=-1).reshape(-1)
+    z2, y1b = M.up_projection_forward(x, w1, off, gidx, b1=b1, math_dtype=D, activation=activation)
+    o2 = M.router_forward(M.down_projection_forward(y1b, w2, off, b2=b2, math_dtype=D), gates, ridx, tok_off, math_dtype=D)
+    torch.testing.assert_close(o2, out_ref, rtol=1e-5, atol=1e-7)
+
+
 def test_single_expert_is_a_dense_swiglu_mlp():
     g = torch.Generator().manual_seed(5)
     T, H, I = 30, 12, 6
