@@ -156,6 +156,34 @@ int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride
                                 int64_t TK, int H, int I, int E, int activation, void* workspace,
                                 size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * fp8 forward path (OCP e4m3 elements, one power-of-two scale per 32 contraction elements)
+ * No counterpart in the reference, which computes in bf16 only; the shapes and epilogues are those of
+ * smoe_up_projection_forward / smoe_down_projection_forward above.
+ * ------------------------------------------------------------------------------------------------------ */
+
+/* Quantise a bf16 matrix along its rows.
+ *   src (R, C) bf16 with row stride `src_stride` elements; C % 128 == 0
+ *   q (R, C) bytes: e4m3 of src / scale, round to nearest even, never saturating
+ *   scales (C / 128, R) uint32: byte b of word [g][r] is the biased exponent (2^(byte-127)) shared by elements
+ *          [128 g + 32 b, 128 g + 32 b + 32) of row r: the smallest power of two with amax / scale <= 448 */
+int smoe_mx_quantize(const void* src, int64_t src_stride, int64_t R, int C, void* q, void* scales, void* stream);
+
+/* As smoe_up_projection_forward with x and W1 given in the quantised form above:
+ *   xq (T, H) bytes + x_scales (H/128, T); w1q (E, N1, H) bytes contiguous + w1_scales (H/128, E*N1)
+ *   z (TK, N1) bf16 or NULL; y1 (TK, I) bf16.  Limits: H % 128 == 0, I % 64 == 0. */
+int smoe_up_projection_forward_fp8(const void* xq, const void* x_scales, const void* w1q, const void* w1_scales,
+                                   const void* b1, void* z, void* y1, const int32_t* off,
+                                   const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                   int activation, void* workspace, size_t workspace_bytes, void* stream);
+
+/* As smoe_down_projection_forward with y1 and W2 quantised:
+ *   y1q (TK, I) bytes + y1_scales (I/128, TK); w2q (E, H, I) bytes contiguous + w2_scales (I/128, E*H)
+ *   y2 (TK, H) bf16.  Limits: I % 128 == 0, H % 64 == 0. */
+int smoe_down_projection_forward_fp8(const void* y1q, const void* y1_scales, const void* w2q, const void* w2_scales,
+                                     const void* b2, void* y2, const int32_t* off, int64_t TK, int H, int I, int E,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

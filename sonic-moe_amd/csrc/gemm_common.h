@@ -116,12 +116,18 @@ SMOE_DEV void lds_barrier() {
 //            current stage's slot with stage s+NSTAGE, read slice 0 of the next stage while the last MFMAs run.
 //   issue(buf, s)                 start this wave's LPS direct-to-LDS loads of stage s into ring slot buf
 //   load(buf, s, ks, qf, pf)      read the fragments of slice ks of stage s from ring slot buf
-template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Issue, class Load>
+// MFMA operand fragment + instruction of the bf16 kernels; the fp8 kernels bring their own pair
+struct Bf16Mma {
+  typedef bf16x8 Frag;
+  static __device__ __forceinline__ f32x16 run(const Frag& q, const Frag& p, f32x16 c) { return mfma32(q, p, c); }
+};
+
+template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Mma = Bf16Mma, class Issue, class Load>
 SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, Load&& load) {
   if (S <= 0) return;
   static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
   static_assert(SLICES % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 6, "unsupported pipeline shape");
-  bf16x8 qf[2][NQ], pf[2][NP];
+  typename Mma::Frag qf[2][NQ], pf[2][NP];
   const int pre = S < NSTAGE ? S : NSTAGE;
   for (int s = 0; s < pre; s++) issue(s, s);
 
@@ -139,7 +145,7 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
 #pragma unroll
     for (int q = 0; q < NQ; q++)
 #pragma unroll
-      for (int pp = 0; pp < NP; pp++) acc[q][pp] = mfma32(qf[cur][q], pf[cur][pp], acc[q][pp]);
+      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
     constexpr int NM = NQ * NP, NR = NREADS < NM ? NREADS : NM - 1;
 #pragma unroll
     for (int i = 0; i < NR; i++) {
@@ -250,6 +256,82 @@ SMOE_DEV void pointwise_grad(float t, float& f, float& fp) {
     const float r = fmaxf(t, 0.f);
     f = r * r;
     fp = 2.f * r;
+  }
+}
+
+// ---- epilogue of the forward GEMMs ---------------------------------------------------------------------------------
+struct FwdEpilogueArgs {
+  const uint16_t* bias;  // this expert's bias row (N values) or null
+  uint16_t* out0;        // accumulator (+bias) as bf16: z resp. y2; null = not stored
+  int64_t out0_stride;
+  uint16_t* out1;        // activation output y1 (WITH_ACT only)
+  int64_t out1_stride;
+  int m_base, row_end;   // first grouped row of this wave's tile, end of the expert's rows
+  int n_base, N;         // first accumulator column of this wave's tile, number of accumulator columns
+};
+
+// acc[fn][fm] is the wave's TM x TN tile (lane = token row l%32 of fragment row fm; register quad rg of fragment column
+// fn = columns fn*32 + 8*rg + 4*(l/32) + 0..3).  Adds the bias, stores out0, and with WITH_ACT evaluates activation ACT
+// from the un-rounded accumulator into out1 (TN/2 columns for the gated activations, TN otherwise).  The caller has
+// made sure that no wave still reads the LDS ring: every wave parks its tile in its own region of it.
+template <int TM, int TN, int FM, int FN, bool WITH_ACT, int ACT>
+SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int lane, const FwdEpilogueArgs& a) {
+  constexpr bool GLU = act_is_glu(ACT);
+  constexpr int PW = act_pointwise(ACT);
+  if (a.bias != nullptr) {
+    static_for<FN * 4>([&](auto q_c) {
+      constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+      int n = a.n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
+      n = n <= a.N - 4 ? n : a.N - 4;
+      const u32x2 b = *(const u32x2*)(a.bias + n);
+      const float b0 = bf16_lo(b[0]), b1 = bf16_hi(b[0]), b2 = bf16_lo(b[1]), b3 = bf16_hi(b[1]);
+      static_for<FM>([&](auto fm_c) {
+        constexpr int fm = decltype(fm_c)::value;
+        acc[fn][fm][4 * rg + 0] += b0;
+        acc[fn][fm][4 * rg + 1] += b1;
+        acc[fn][fm][4 * rg + 2] += b2;
+        acc[fn][fm][4 * rg + 3] += b3;
+      });
+    });
+  }
+  using LZ = EpiLayout<TN>;
+  using LY = EpiLayout<TN / 2>;
+  char* region = smem + wave * (TM * LZ::ROW_BYTES);
+  if (!WITH_ACT || a.out0 != nullptr) {
+    static_for<FM>([&](auto fm_c) {
+      constexpr int fm = decltype(fm_c)::value;
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
+                   pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
+        *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+      });
+    });
+    epilogue_flush<TM, TN>(region, lane, a.out0, a.out0_stride, a.m_base, a.row_end, a.n_base, a.N);
+  }
+  if constexpr (WITH_ACT && GLU) {
+    static_for<FM>([&](auto fm_c) {
+      constexpr int fm = decltype(fm_c)::value;
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
+        const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
+        const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
+        *(uint32_t*)(region + (fm * 32 + (lane & 31)) * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * (lane >> 5)) * 2) = v;
+      });
+    });
+    epilogue_flush<TM, TN / 2>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base / 2, a.N / 2);
+  } else if constexpr (WITH_ACT) {
+    static_for<FM>([&](auto fm_c) {
+      constexpr int fm = decltype(fm_c)::value;
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
+                   pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
+        *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+      });
+    });
+    epilogue_flush<TM, TN>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base, a.N);
   }
 }
 

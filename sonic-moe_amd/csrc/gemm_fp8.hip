@@ -1,0 +1,416 @@
+// fp8 (OCP e4m3) forward grouped GEMMs with per-block scales, and the quantiser that produces their operands.
+//
+// Operand format ("MX" block scaling): along the contraction dimension every 32 consecutive elements share one
+// power-of-two scale, stored as its biased exponent (e8m0, value 2^(byte - 127)); elements are e4m3 bytes.  This is the
+// format v_mfma_scale_f32_32x32x64_f8f6f4 multiplies natively: the scale is applied inside the matrix instruction, so
+// the main loop has no per-block floating-point work.
+//   data   q (R, C) bytes, row-major
+//   scales s (C / 128, R) 32-bit words: byte b of word [g][r] scales elements [128 g + 32 b, 128 g + 32 b + 32) of row r
+// (one word per row and 128-element group = one pipeline stage, so that a stage's scales of 64 rows are one
+// direct-to-LDS load of a wavefront).
+//
+// The GEMM is the K-major / K-major kernel of the bf16 path with 128 BYTES of contraction per row and stage:
+//   up-projection    P = x rows gathered (fp8), Q = W1[e] (fp8)  -> z (bf16), y1 = act(z) (bf16)
+//   down-projection  P = y1 rows (fp8),        Q = W2[e] (fp8)  -> y2 (bf16)
+// Accumulation is fp32; outputs, biases and epilogues are those of the bf16 kernels.
+#include "gemm_common.h"
+
+namespace smoe {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+
+// ---- quantiser ---------------------------------------------------------------------------------------------------
+// e8m0 exponent of the smallest power of two s with amax / s <= 448 (the largest e4m3 value): no element saturates
+SMOE_DEV int mx_scale_exponent(float amax) {
+  if (!(amax > 0.f)) return 0;
+  // amax = m * 2^e with m in [1, 2): 448 = 1.75 * 2^8 -> need 2^k >= amax / 448
+  const uint32_t bits = __float_as_uint(amax);
+  const int e = (int)((bits >> 23) & 0xff) - 127;
+  const uint32_t mant = bits & 0x7fffffu;
+  int k = e - 8;                      // 2^(e-8) * 448 = 1.75 * 2^e
+  if (mant > 0x600000u) k += 1;       // m > 1.75
+  k += 127;
+  return k < 0 ? 0 : (k > 254 ? 254 : k);
+}
+
+// one lane = one 32-element block: 64 bytes in, 32 bytes + 1 scale byte out
+__global__ __launch_bounds__(256) void mx_quantize_kernel(const uint16_t* __restrict__ src, int64_t src_stride,
+                                                          int64_t R, int C, uint8_t* __restrict__ q,
+                                                          uint32_t* __restrict__ scales) {
+  const int blocks_per_row = C >> 5;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t total = R * blocks_per_row;
+  const bool live = gid < total;
+  const int64_t r = live ? gid / blocks_per_row : 0;
+  const int b = live ? (int)(gid - r * blocks_per_row) : 0;
+  float v[32];
+  float amax = 0.f;
+  if (live) {
+    const u32x4* p = (const u32x4*)(src + r * src_stride + (int64_t)b * 32);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const u32x4 w = p[i];
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        v[i * 8 + 2 * j] = bf16_lo(w[j]);
+        v[i * 8 + 2 * j + 1] = bf16_hi(w[j]);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 32; i++) amax = fmaxf(amax, fabsf(v[i]));
+  }
+  const int ex = mx_scale_exponent(amax);
+  const float inv = __uint_as_float((uint32_t)(254 - ex) << 23);  // 2^-(ex-127); ex <= 254 keeps it finite, ex = 0 only for amax = 0
+  if (live) {
+    uint32_t out[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      int w = 0;
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(v[4 * i] * inv, v[4 * i + 1] * inv, w, false);
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(v[4 * i + 2] * inv, v[4 * i + 3] * inv, w, true);
+      out[i] = (uint32_t)w;
+    }
+    u32x4* dst = (u32x4*)(q + r * C + (int64_t)b * 32);
+    dst[0] = u32x4{out[0], out[1], out[2], out[3]};
+    dst[1] = u32x4{out[4], out[5], out[6], out[7]};
+  }
+  // blocks 4g..4g+3 of a row sit in 4 consecutive lanes (C % 128 == 0): gather their bytes into one word
+  uint32_t word = (uint32_t)ex << (8 * (b & 3));
+  word |= __shfl_xor(word, 1, 64);
+  word |= __shfl_xor(word, 2, 64);
+  if (live && (b & 3) == 0) scales[(int64_t)(b >> 2) * R + r] = word;
+}
+
+// ---- GEMM --------------------------------------------------------------------------------------------------------
+struct Fp8Params {
+  const uint8_t* P;
+  int64_t p_stride;  // bytes
+  const uint32_t* p_scales;
+  int64_t p_rows;    // rows of the P scale table (T or TK)
+  const int32_t* gidx;
+  const uint8_t* Q;
+  int64_t q_stride_e, q_stride_row;  // bytes
+  const uint32_t* q_scales;
+  int64_t q_rows;    // rows of the Q scale table (E * N)
+  const int32_t* off;
+  TileMap tm;
+  int N, Kdim, n_tiles;
+  const uint16_t* bias;
+  uint16_t* out0;
+  int64_t out0_stride;
+  uint16_t* out1;
+  int64_t out1_stride;
+};
+
+struct Fp8Cfg {
+  // 4 wavefronts, 128 x 128 each: the fragments of an fp8 slice are twice as large as bf16 ones, and two register sets
+  // of them beside a 128 x 64 accumulator tile do not fit the 256 registers of an 8-wavefront workgroup
+  static constexpr int BM = 256, BN = 256, WM = 2, WN = 2, BKB = 128, NSTAGE = 2;  // BKB: contraction bytes per stage
+  static constexpr int NW = WM * WN, NT = NW * 64;
+  static constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
+  static constexpr int P_STAGE = BM * BKB, Q_STAGE = BN * BKB, S_STAGE = (BM + BN) * 4;
+  static constexpr int STAGE = P_STAGE + Q_STAGE + S_STAGE;
+  static constexpr int P_INSTR = P_STAGE / 1024 / NW, Q_INSTR = Q_STAGE / 1024 / NW;
+  static constexpr int KPR = BKB / 16, KRPI = 64 / KPR;  // 16-byte pieces per row, rows per load instruction
+  static constexpr int EPI = NW * TM * (TN * 2 + 16);
+  static constexpr int SMEM = NSTAGE * STAGE > EPI ? NSTAGE * STAGE : EPI;
+  static constexpr int S_INSTR = (BM + BN) / 64 / NW;  // scale loads (64 rows each) per wave and stage
+  static_assert(S_INSTR * NW * 64 == BM + BN, "the scale rows must split evenly over the wavefronts");
+  static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
+};
+
+// direct-to-LDS load of one 32-bit word per lane: the wavefront's 64 words land at lds_wave_base + 4 * lane
+SMOE_DEV void load4_to_lds(const void* g, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(lds_wave_base) : "memory");
+}
+
+// Operand fragment of v_mfma_scale_f32_32x32x64_f8f6f4: lane l holds row l%32 and, of the 64 contraction bytes of the
+// slice, bytes [16h, 16h+16) and [32+16h, 48+16h) with h = l/32; its scale byte (bits 0-7) belongs to the 32-element
+// block h of the slice.
+struct Fp8Frag {
+  i32x8 data;
+  int scale;
+};
+struct Fp8Mma {
+  typedef Fp8Frag Frag;
+  static __device__ __forceinline__ f32x16 run(const Frag& q, const Frag& p, f32x16 c) {
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(q.data, p.data, c, 0, 0, 0, q.scale, 0, p.scale);
+  }
+};
+
+template <bool WITH_ACT, int ACT>
+__global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Params p) {
+  using C = Fp8Cfg;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int FM = C::FM, FN = C::FN, SLICES = C::BKB / 64;
+  const uint32_t smem_base = lds_address(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % C::WM, wn = wave / C::WM;
+
+  const int num_m_tiles = p.tm.header[0];
+  const int64_t total = (int64_t)num_m_tiles * p.n_tiles;
+  const int64_t lin = xcd_linear_tile(total);
+  if (lin < 0) return;
+  constexpr int GM = 8;
+  const int64_t per_group = (int64_t)GM * p.n_tiles;
+  const int group = (int)(lin / per_group);
+  const int first_m = group * GM;
+  const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
+  const int within = (int)(lin - (int64_t)group * per_group);
+  const int mt = first_m + within % gm;
+  const int nt = within / gm;
+  const int e = p.tm.expert[mt];
+  const int row0 = p.tm.row0[mt];
+  const int row_end = p.off[e + 1];
+  const int n0 = nt * C::BN;
+
+  // per-lane global source pointers of the data pieces (advance by one stage per k-step)
+  const uint8_t* p_src[C::P_INSTR];
+#pragma unroll
+  for (int i = 0; i < C::P_INSTR; i++) {
+    const int r = (wave * C::P_INSTR + i) * C::KRPI + lane / C::KPR;
+    int m = row0 + r;
+    m = m < row_end ? m : row_end - 1;
+    const int64_t src_row = p.gidx ? (int64_t)p.gidx[m] : (int64_t)m;
+    p_src[i] = p.P + src_row * p.p_stride + (((lane % C::KPR) ^ kswz<64>(r)) << 4);
+  }
+  const uint8_t* q_src[C::Q_INSTR];
+  const uint8_t* qe = p.Q + (int64_t)e * p.q_stride_e;
+#pragma unroll
+  for (int i = 0; i < C::Q_INSTR; i++) {
+    const int r = (wave * C::Q_INSTR + i) * C::KRPI + lane / C::KPR;
+    int n = n0 + r;
+    n = n < p.N ? n : p.N - 1;
+    q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane % C::KPR) ^ kswz<64>(r)) << 4);
+  }
+  // this lane's scale words: load j of wave w covers rows (w * S_INSTR + j) * 64 .. + 63 of the tile's 256 token rows
+  // followed by its 256 feature rows
+  const uint32_t* s_src[C::S_INSTR];
+  int64_t s_step[C::S_INSTR];
+#pragma unroll
+  for (int j = 0; j < C::S_INSTR; j++) {
+    const int r = (wave * C::S_INSTR + j) * 64 + lane;
+    if (r < C::BM) {
+      int m = row0 + r;
+      m = m < row_end ? m : row_end - 1;
+      s_src[j] = p.p_scales + (p.gidx ? (int64_t)p.gidx[m] : (int64_t)m);
+      s_step[j] = p.p_rows;
+    } else {
+      int n = n0 + r - C::BM;
+      n = n < p.N ? n : p.N - 1;
+      s_src[j] = p.q_scales + (int64_t)e * p.N + n;
+      s_step[j] = p.q_rows;
+    }
+  }
+
+  const int S_total = p.Kdim / C::BKB;
+
+  // per-lane LDS fragment offsets (bytes inside a stage): two 16-byte pieces per slice, one scale word per stage
+  const int half = lane >> 5;
+  int p_off[SLICES][2], q_off[SLICES][2];
+  {
+    const int prow = wm * C::TM + (lane & 31), qrow = wn * C::TN + (lane & 31);
+    const int psw = kswz<64>(prow), qsw = kswz<64>(qrow);
+#pragma unroll
+    for (int ks = 0; ks < SLICES; ks++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int piece = 4 * ks + 2 * j + half;
+        p_off[ks][j] = prow * C::BKB + ((piece ^ psw) << 4);
+        q_off[ks][j] = C::P_STAGE + qrow * C::BKB + ((piece ^ qsw) << 4);
+      }
+  }
+  const int ps_off = C::P_STAGE + C::Q_STAGE + (wm * C::TM + (lane & 31)) * 4;
+  const int qs_off = C::P_STAGE + C::Q_STAGE + (C::BM + wn * C::TN + (lane & 31)) * 4;
+
+  f32x16 acc[FN][FM];
+#pragma unroll
+  for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
+
+  auto issue = [&](int buf, int /*s*/) {
+    const uint32_t base = smem_base + buf * C::STAGE;
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) {
+      load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
+      p_src[i] += C::BKB;
+    }
+#pragma unroll
+    for (int i = 0; i < C::Q_INSTR; i++) {
+      load16_to_lds(q_src[i], base + C::P_STAGE + (wave * C::Q_INSTR + i) * 1024);
+      q_src[i] += C::BKB;
+    }
+#pragma unroll
+    for (int j = 0; j < C::S_INSTR; j++) {
+      load4_to_lds(s_src[j], base + C::P_STAGE + C::Q_STAGE + (wave * C::S_INSTR + j) * 256);
+      s_src[j] += s_step[j];
+    }
+  };
+  auto load = [&](int buf, int /*s*/, int ks, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[FM]) {
+    const char* st = smem + buf * C::STAGE;
+    const int shift = 8 * (2 * ks + half);
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++) {
+      const i32x4 lo = *(const i32x4*)(st + p_off[ks][0] + fm * 32 * C::BKB);
+      const i32x4 hi = *(const i32x4*)(st + p_off[ks][1] + fm * 32 * C::BKB);
+      pf[fm].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      pf[fm].scale = (int)(*(const uint32_t*)(st + ps_off + fm * 32 * 4) >> shift);
+    }
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+      const i32x4 lo = *(const i32x4*)(st + q_off[ks][0] + fn * 32 * C::BKB);
+      const i32x4 hi = *(const i32x4*)(st + q_off[ks][1] + fn * 32 * C::BKB);
+      qf[fn].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      qf[fn].scale = (int)(*(const uint32_t*)(st + qs_off + fn * 32 * 4) >> shift);
+    }
+  };
+  gemm_mainloop<FN, FM, 3 * (FN + FM), C::P_INSTR + C::Q_INSTR + C::S_INSTR, SLICES, C::NSTAGE, Fp8Mma>(S_total, acc, issue, load);
+
+  FwdEpilogueArgs ea;
+  ea.bias = p.bias ? p.bias + (int64_t)e * p.N : nullptr;
+  ea.out0 = p.out0;
+  ea.out0_stride = p.out0_stride;
+  ea.out1 = p.out1;
+  ea.out1_stride = p.out1_stride;
+  ea.m_base = row0 + wm * C::TM;
+  ea.row_end = row_end;
+  ea.n_base = n0 + wn * C::TN;
+  ea.N = p.N;
+  wait_vmem_all();
+  lds_barrier();  // all waves are done reading the last stage
+  forward_epilogue<C::TM, C::TN, FM, FN, WITH_ACT, ACT>(acc, smem, wave, lane, ea);
+}
+
+template <bool WITH_ACT, int ACT>
+static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
+  using C = Fp8Cfg;
+  static bool attr_set = false;
+  auto kern = fp8_varlen_m_kernel<WITH_ACT, ACT>;
+  if (!attr_set) {
+    SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
+    attr_set = true;
+  }
+  p.tm = carve_tile_map(workspace, TK, E, C::BM);
+  int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
+  if (rc) return rc;
+  p.n_tiles = (int)ceil_div(p.N, C::BN);
+  const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
+  const int64_t grid = ((max_tiles + 7) / 8) * 8;
+  SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: too many tiles");
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+static int launch_fp8_up(int act, Fp8Params& p, const int32_t* off, void* ws, int64_t TK, int E, hipStream_t st) {
+  switch (act) {
+    case SMOE_ACT_SWIGLU: return launch_fp8<true, SMOE_ACT_SWIGLU>(p, off, ws, TK, E, st);
+    case SMOE_ACT_GEGLU: return launch_fp8<true, SMOE_ACT_GEGLU>(p, off, ws, TK, E, st);
+    case SMOE_ACT_REGLU: return launch_fp8<true, SMOE_ACT_REGLU>(p, off, ws, TK, E, st);
+    case SMOE_ACT_RELU_SQ: return launch_fp8<true, SMOE_ACT_RELU_SQ>(p, off, ws, TK, E, st);
+    case SMOE_ACT_RELU: return launch_fp8<true, SMOE_ACT_RELU>(p, off, ws, TK, E, st);
+    case SMOE_ACT_GELU: return launch_fp8<true, SMOE_ACT_GELU>(p, off, ws, TK, E, st);
+    case SMOE_ACT_SILU: return launch_fp8<true, SMOE_ACT_SILU>(p, off, ws, TK, E, st);
+  }
+  set_error("unknown activation code %d", act);
+  return SMOE_ERR_INVALID;
+}
+
+}  // namespace smoe
+
+using namespace smoe;
+
+extern "C" int smoe_mx_quantize(const void* src, int64_t src_stride, int64_t R, int C, void* q, void* scales,
+                                void* stream) {
+  SMOE_REQUIRE(R >= 0 && C > 0, SMOE_ERR_INVALID, "mx_quantize: bad shape");
+  SMOE_REQUIRE(C % 128 == 0, SMOE_ERR_UNSUPPORTED, "mx_quantize: %d columns are not a multiple of 128", C);
+  SMOE_REQUIRE(src_stride % 8 == 0, SMOE_ERR_UNSUPPORTED, "mx_quantize: row stride must be a multiple of 8 elements");
+  if (R == 0) return SMOE_OK;
+  SMOE_REQUIRE(src && q && scales, SMOE_ERR_INVALID, "mx_quantize: null pointer");
+  const int64_t blocks = R * (C / 32);
+  SMOE_REQUIRE(ceil_div(blocks, 256) < (1ll << 31), SMOE_ERR_UNSUPPORTED, "mx_quantize: tensor too large");
+  hipLaunchKernelGGL(mx_quantize_kernel, dim3((unsigned)ceil_div(blocks, 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint16_t*)src, src_stride, R, C, (uint8_t*)q, (uint32_t*)scales);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+static int check_fp8(int64_t TK, int Kdim, int N, int E, const void* ws, size_t ws_bytes, const char* who) {
+  SMOE_REQUIRE(TK >= 0 && TK < (1ll << 31), SMOE_ERR_INVALID, "%s: TK out of range", who);
+  SMOE_REQUIRE(E >= 1, SMOE_ERR_INVALID, "%s: E must be >= 1", who);
+  SMOE_REQUIRE(Kdim >= 128 && Kdim % 128 == 0, SMOE_ERR_UNSUPPORTED,
+               "%s: the contraction size %d must be a multiple of 128", who, Kdim);
+  SMOE_REQUIRE(N >= 64 && N % 64 == 0, SMOE_ERR_UNSUPPORTED, "%s: the output width %d must be a multiple of 64", who, N);
+  SMOE_REQUIRE(ws != nullptr && ws_bytes >= smoe_gemm_workspace_bytes(TK, E), SMOE_ERR_WORKSPACE,
+               "%s: workspace too small", who);
+  return SMOE_OK;
+}
+
+extern "C" int smoe_up_projection_forward_fp8(const void* xq, const void* x_scales, const void* w1q,
+                                              const void* w1_scales, const void* b1, void* z, void* y1,
+                                              const int32_t* off, const int32_t* x_gather_idx, int64_t T, int64_t TK,
+                                              int H, int I, int E, int activation, void* workspace,
+                                              size_t workspace_bytes, void* stream) {
+  SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
+               "up_projection_forward_fp8: unknown activation code %d", activation);
+  const int N1 = act_is_glu(activation) ? 2 * I : I;
+  int rc = check_fp8(TK, H, N1, E, workspace, workspace_bytes, "up_projection_forward_fp8");
+  if (rc) return rc;
+  SMOE_REQUIRE(I % 64 == 0, SMOE_ERR_UNSUPPORTED, "up_projection_forward_fp8: I=%d must be a multiple of 64", I);
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(xq && x_scales && w1q && w1_scales && y1 && off && x_gather_idx && T > 0, SMOE_ERR_INVALID,
+               "up_projection_forward_fp8: null pointer");
+  Fp8Params p = {};
+  p.P = (const uint8_t*)xq;
+  p.p_stride = H;
+  p.p_scales = (const uint32_t*)x_scales;
+  p.p_rows = T;
+  p.gidx = x_gather_idx;
+  p.Q = (const uint8_t*)w1q;
+  p.q_stride_e = (int64_t)N1 * H;
+  p.q_stride_row = H;
+  p.q_scales = (const uint32_t*)w1_scales;
+  p.q_rows = (int64_t)E * N1;
+  p.off = off;
+  p.N = N1;
+  p.Kdim = H;
+  p.bias = (const uint16_t*)b1;
+  p.out0 = (uint16_t*)z;
+  p.out0_stride = N1;
+  p.out1 = (uint16_t*)y1;
+  p.out1_stride = I;
+  return launch_fp8_up(activation, p, off, workspace, TK, E, (hipStream_t)stream);
+}
+
+extern "C" int smoe_down_projection_forward_fp8(const void* y1q, const void* y1_scales, const void* w2q,
+                                                const void* w2_scales, const void* b2, void* y2, const int32_t* off,
+                                                int64_t TK, int H, int I, int E, void* workspace,
+                                                size_t workspace_bytes, void* stream) {
+  int rc = check_fp8(TK, I, H, E, workspace, workspace_bytes, "down_projection_forward_fp8");
+  if (rc) return rc;
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(y1q && y1_scales && w2q && w2_scales && y2 && off, SMOE_ERR_INVALID,
+               "down_projection_forward_fp8: null pointer");
+  Fp8Params p = {};
+  p.P = (const uint8_t*)y1q;
+  p.p_stride = I;
+  p.p_scales = (const uint32_t*)y1_scales;
+  p.p_rows = TK;
+  p.Q = (const uint8_t*)w2q;
+  p.q_stride_e = (int64_t)H * I;
+  p.q_stride_row = I;
+  p.q_scales = (const uint32_t*)w2_scales;
+  p.q_rows = (int64_t)E * H;
+  p.off = off;
+  p.N = H;
+  p.Kdim = I;
+  p.bias = (const uint16_t*)b2;
+  p.out0 = (uint16_t*)y2;
+  p.out0_stride = H;
+  return launch_fp8<false, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, (hipStream_t)stream);
+}

@@ -199,66 +199,19 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #endif
 
   if constexpr (ROLE == ROLE_PLAIN || ROLE == ROLE_UP_FWD) {
-    if (p.bias != nullptr) {
-      // register quad (fn, rg) of a lane holds columns n_base + fn*32 + 8*rg + 4*(lane>>5) + 0..3 of every fragment row
-      const uint16_t* be = p.bias + (int64_t)e * p.N;
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        int n = n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
-        n = n <= p.N - 4 ? n : p.N - 4;
-        const u32x2 b = *(const u32x2*)(be + n);
-        const float b0 = bf16_lo(b[0]), b1 = bf16_hi(b[0]), b2 = bf16_lo(b[1]), b3 = bf16_hi(b[1]);
-        static_for<FM>([&](auto fm_c) {
-          constexpr int fm = decltype(fm_c)::value;
-          acc[fn][fm][4 * rg + 0] += b0;
-          acc[fn][fm][4 * rg + 1] += b1;
-          acc[fn][fm][4 * rg + 2] += b2;
-          acc[fn][fm][4 * rg + 3] += b3;
-        });
-      });
-    }
-    // ---- epilogue through LDS: every wave parks its tile in its own region, then stores 16 B per lane ----
-    using LZ = EpiLayout<C::TN>;
-    using LY = EpiLayout<C::TN / 2>;
-    char* region = smem + wave * (C::TM * LZ::ROW_BYTES);
+    FwdEpilogueArgs ea;
+    ea.bias = p.bias ? p.bias + (int64_t)e * p.N : nullptr;
+    ea.out0 = p.out0;
+    ea.out0_stride = p.out0_stride;
+    ea.out1 = p.out1;
+    ea.out1_stride = p.out1_stride;
+    ea.m_base = m_base;
+    ea.row_end = row_end;
+    ea.n_base = n_base;
+    ea.N = p.N;
     wait_vmem_all();
     lds_barrier();  // all waves are done reading the last stage
-    if (ROLE == ROLE_PLAIN || p.out0 != nullptr) {
-      static_for<FM>([&](auto fm_c) {
-        constexpr int fm = decltype(fm_c)::value;
-        static_for<FN * 4>([&](auto q_c) {
-          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-          u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
-                     pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
-          *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
-        });
-      });
-      epilogue_flush<C::TM, C::TN>(region, lane, p.out0, p.out0_stride, m_base, row_end, n_base, p.N);
-    }
-    if constexpr (ROLE == ROLE_UP_FWD && GLU) {
-      static_for<FM>([&](auto fm_c) {
-        constexpr int fm = decltype(fm_c)::value;
-        static_for<FN * 4>([&](auto q_c) {
-          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-          const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
-          const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
-          const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
-          *(uint32_t*)(region + (fm * 32 + (lane & 31)) * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * (lane >> 5)) * 2) = v;
-        });
-      });
-      epilogue_flush<C::TM, C::TN / 2>(region, lane, p.out1, p.out1_stride, m_base, row_end, n_base / 2, p.N / 2);
-    } else if constexpr (ROLE == ROLE_UP_FWD) {
-      static_for<FM>([&](auto fm_c) {
-        constexpr int fm = decltype(fm_c)::value;
-        static_for<FN * 4>([&](auto q_c) {
-          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-          u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
-                     pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
-          *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
-        });
-      });
-      epilogue_flush<C::TM, C::TN>(region, lane, p.out1, p.out1_stride, m_base, row_end, n_base, p.N);
-    }
+    forward_epilogue<C::TM, C::TN, FM, FN, ROLE == ROLE_UP_FWD, ACT>(acc, smem, wave, lane, ea);
   } else {
     // ---- dz epilogue ----
     // acc = dy1[i][m].  Per 32-row fragment row the wavefront stages its z sub-tile (32 rows x ZW*TN bf16; ZW = 2

@@ -18,6 +18,14 @@ from ..count_cumsum import count_cumsum
 from ..enums import LIBRARY_NAME, ActivationType, is_glu
 from .backward import _down_projection_backward, _softmax_topk_bwd, _token_broadcast_backward, _up_projection_backward
 from .forward import _down_projection_forward, _router_forward, _softmax_topk_fwd, _up_projection_forward
+from .fp8 import (
+    _down_projection_forward_fp8,
+    _up_projection_forward_fp8,
+    enable_fp8_forward,
+    is_using_fp8_forward,
+    mx_quantize,
+    quantize_expert_weight,
+)
 from .utils import enable_quack_gemm, is_using_quack_gemm
 
 
@@ -172,9 +180,19 @@ class _ExpertsFunction(torch.autograd.Function):
 
         z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
         y1 = torch.empty(TK, I, dtype=x.dtype, device=x.device)
-        _up_projection_forward(x, w1, z, y1, b1, off, None, gidx, stream_id, activation_type.value, glu, inference)
         y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
-        _down_projection_forward(w2, y1, y2, b2, off, None, gidx, stream_id)
+        if is_using_fp8_forward():
+            xq, xs = mx_quantize(x)
+            w1q, w1s = quantize_expert_weight(w1)
+            _up_projection_forward_fp8(xq, xs, w1q, w1s, z, y1, b1, off, gidx, E, stream_id, activation_type.value, glu)
+            del xq, xs, w1q, w1s
+            y1q, y1s = mx_quantize(y1)
+            w2q, w2s = quantize_expert_weight(w2)
+            _down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, b2, off, E, stream_id)
+            del y1q, y1s, w2q, w2s
+        else:
+            _up_projection_forward(x, w1, z, y1, b1, off, None, gidx, stream_id, activation_type.value, glu, inference)
+            _down_projection_forward(w2, y1, y2, b2, off, None, gidx, stream_id)
         del y1
         o = torch.empty(T, H, dtype=x.dtype, device=x.device)
         _router_forward(y2, o, scores_flat, ridx, tok_off, K_or_maxK, H, is_varlen_K)
@@ -296,6 +314,8 @@ __all__ = [
     "count_cumsum",
     "enable_quack_gemm",
     "is_using_quack_gemm",
+    "enable_fp8_forward",
+    "is_using_fp8_forward",
     "moe_TC_softmax_topk_layer",
     "moe_general_routing_inputs",
 ]

@@ -1,0 +1,153 @@
+"""fp8 forward path: block-scaled e4m3 operands for the two forward grouped GEMMs.
+
+The reference has no fp8 path; this module has the shape of its `enable_quack_gemm` switch
+(sonicmoe/functional/utils.py:9-25): inside `with enable_fp8_forward():` the expert forward quantises x, W1, y1 and W2
+(one power-of-two scale per 32 contraction elements) and runs the fp8 MFMA kernels; z is still stored in bf16 and the
+backward pass is the bf16 one.
+"""
+
+from __future__ import annotations
+
+from contextlib import contextmanager
+
+import torch
+
+from .. import _lib
+from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
+from .forward import _check_bf16, _gemm_workspace
+
+_FP8_FORWARD = False
+
+
+@contextmanager
+def enable_fp8_forward(enable: bool = True):
+    global _FP8_FORWARD
+    previous, _FP8_FORWARD = _FP8_FORWARD, enable
+    try:
+        yield
+    finally:
+        _FP8_FORWARD = previous
+
+
+def is_using_fp8_forward() -> bool:
+    return _FP8_FORWARD
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_mx_quantize", mutates_args={"q", "scales"})
+def _mx_quantize(src: torch.Tensor, q: torch.Tensor, scales: torch.Tensor) -> None:
+    """src (R, C) bf16 -> q (R, C) uint8 e4m3 codes, scales (C/128, R) int32 (four exponent bytes per word)."""
+    _lib.require_device(src, q, scales)
+    _check_bf16(("src", src))
+    R, C = src.shape
+    assert src.stride(1) == 1 and q.is_contiguous() and scales.is_contiguous()
+    assert q.dtype == torch.uint8 and q.shape == (R, C) and scales.dtype == torch.int32 and scales.shape == (C // 128, R)
+    rc = _lib.lib().smoe_mx_quantize(
+        _lib.ptr(src), src.stride(0), R, C, _lib.ptr(q), _lib.ptr(scales), _lib.current_stream_handle()
+    )
+    _lib.check(rc, "_mx_quantize")
+
+
+def mx_quantize(t: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Quantise the rows of a 2-D bf16 tensor; see `_mx_quantize` for the layouts."""
+    R, C = t.shape
+    if C % 128:
+        raise NotImplementedError(f"mx_quantize: {C} columns are not a multiple of 128")
+    q = torch.empty(R, C, dtype=torch.uint8, device=t.device)
+    scales = torch.empty(C // 128, R, dtype=torch.int32, device=t.device)
+    _mx_quantize(t, q, scales)
+    return q, scales
+
+
+def quantize_expert_weight(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """w_view is the (out, in, E) permuted view of an (E, out, in) parameter; quantised along `in`."""
+    w = w_view.permute(2, 0, 1)
+    if not w.is_contiguous():
+        w = w.contiguous()
+    E, N, K = w.shape
+    return mx_quantize(w.reshape(E * N, K))
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_forward_fp8", mutates_args={"z", "y1"})
+def _up_projection_forward_fp8(
+    xq: torch.Tensor,
+    x_scales: torch.Tensor,
+    w1q: torch.Tensor,
+    w1_scales: torch.Tensor,
+    z: torch.Tensor | None,
+    y1: torch.Tensor,
+    b1: torch.Tensor | None,
+    expert_frequency_offset: torch.Tensor,
+    x_gather_idx: torch.Tensor,
+    E: int,
+    stream_id: int,
+    activation_type: str,
+    is_glu_activation: bool,
+) -> None:
+    """z = gather(xq) w1q^T (+ b1) with the block scales applied, y1 = act(z); xq (T, H), w1q (E*N1, H)."""
+    _lib.require_device(xq, x_scales, w1q, w1_scales, y1, b1, expert_frequency_offset, x_gather_idx)
+    _check_bf16(("z", z), ("y1", y1), ("b1", b1))
+    T, H = xq.shape
+    TK, I = y1.shape
+    N1 = 2 * I if is_glu_activation else I
+    assert w1q.shape == (E * N1, H) and x_scales.shape == (H // 128, T) and w1_scales.shape == (H // 128, E * N1)
+    assert z is None or (z.shape == (TK, N1) and z.is_contiguous())
+    ws = _gemm_workspace(TK, E, xq.device)
+    rc = _lib.lib().smoe_up_projection_forward_fp8(
+        _lib.ptr(xq),
+        _lib.ptr(x_scales),
+        _lib.ptr(w1q),
+        _lib.ptr(w1_scales),
+        _lib.ptr(b1),
+        _lib.ptr(z),
+        _lib.ptr(y1),
+        _lib.ptr(expert_frequency_offset),
+        _lib.ptr(x_gather_idx),
+        T,
+        TK,
+        H,
+        I,
+        E,
+        ACTIVATION_CODE[ActivationType(activation_type)],
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_up_projection_forward_fp8")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_down_projection_forward_fp8", mutates_args={"y2"})
+def _down_projection_forward_fp8(
+    y1q: torch.Tensor,
+    y1_scales: torch.Tensor,
+    w2q: torch.Tensor,
+    w2_scales: torch.Tensor,
+    y2: torch.Tensor,
+    b2: torch.Tensor | None,
+    expert_frequency_offset: torch.Tensor,
+    E: int,
+    stream_id: int,
+) -> None:
+    """y2 = y1q w2q^T (+ b2) with the block scales applied; y1q (TK, I), w2q (E*H, I)."""
+    _lib.require_device(y1q, y1_scales, w2q, w2_scales, y2, b2, expert_frequency_offset)
+    _check_bf16(("y2", y2), ("b2", b2))
+    TK, I = y1q.shape
+    H = y2.size(1)
+    assert w2q.shape == (E * H, I) and y1_scales.shape == (I // 128, TK) and w2_scales.shape == (I // 128, E * H)
+    ws = _gemm_workspace(TK, E, y1q.device)
+    rc = _lib.lib().smoe_down_projection_forward_fp8(
+        _lib.ptr(y1q),
+        _lib.ptr(y1_scales),
+        _lib.ptr(w2q),
+        _lib.ptr(w2_scales),
+        _lib.ptr(b2),
+        _lib.ptr(y2),
+        _lib.ptr(expert_frequency_offset),
+        TK,
+        H,
+        I,
+        E,
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_down_projection_forward_fp8")
