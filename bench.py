@@ -29,6 +29,7 @@ import torch  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA peak
 
 CONFIGS = {
     "C2": dict(T=32768, H=4096, I=1024, E=128, K=8, zipf=False),
@@ -116,13 +117,35 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
             ("token_broadcast_backward", lambda: backward._token_broadcast_backward(dx, dxe, ridx, tok_off, K, H, False), None, TK * H * 2 + T * H * 2 + TK * 4),
             ("softmax_topk_bwd", lambda: backward._softmax_topk_bwd(dlog, None, ds.view(T, K), scores, idx, K), None, T * K * 12 + T * E * 2),
         ]
+        if H % 128 == 0 and I % 128 == 0 and only is None:
+            # fp8 forward (config 5 = this shape with block-scaled e4m3 operands): quantisers and the two fp8 GEMMs
+            from sonicmoe.functional import fp8
+
+            xq, xs = fp8.mx_quantize(xd)
+            w1q, w1s = fp8.quantize_expert_weight(w1v)
+            w2q, w2s = fp8.quantize_expert_weight(w2v)
+            y1q, y1s = fp8.mx_quantize(y1)
+            w1_2d, w2_2d = w1.detach().view(E * 2 * I, H), w2.detach().view(E * H, I)
+            ops += [
+                ("fp8:quantize(x)", lambda: fp8._mx_quantize(xd, xq, xs), None, T * H * 3 + T * H // 32),
+                ("fp8:quantize(W1)", lambda: fp8._mx_quantize(w1_2d, w1q, w1s), None, E * 2 * I * H * 3 + E * 2 * I * H // 32),
+                ("fp8:up_projection_forward", lambda: fp8._up_projection_forward_fp8(xq, xs, w1q, w1s, z, y1, None, off, gidx, E, stream, "swiglu", True), 2 * gemm, None),
+                ("fp8:quantize(y1)", lambda: fp8._mx_quantize(y1, y1q, y1s), None, TK * I * 3 + TK * I // 32),
+                ("fp8:quantize(W2)", lambda: fp8._mx_quantize(w2_2d, w2q, w2s), None, E * H * I * 3 + E * H * I // 32),
+                ("fp8:down_projection_forward", lambda: fp8._down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, None, off, E, stream), gemm, None),
+            ]
         rows = []
         for name, fn, flops, nbytes in ops:
             if only is not None and name != only:
                 continue
             ms, _ = time_region(fn, steps, 2)
             row = dict(op=name, ms=round(ms, 4))
-            if flops:
+            if flops and name.startswith("fp8:"):
+                row["tflops"] = round(flops / ms / 1e9, 1)
+                row["frac_fp8_mfma_peak"] = round(flops / ms / 1e9 / PEAK_FP8_TFLOPS, 4)
+                row["frac_mfma_peak"] = row["frac_fp8_mfma_peak"]
+                row["flops"] = flops
+            elif flops:
                 row["tflops"] = round(flops / ms / 1e9, 1)
                 row["frac_mfma_peak"] = round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)
                 row["flops"] = flops
@@ -291,6 +314,32 @@ def main():
     log(f"{a.config}: fwd {fwd_ms:.3f} ms ({flops_fwd / fwd_ms / 1e9:.1f} TFLOP/s), fwd+bwd {ms:.3f} ms "
         f"({tflops:.1f} TFLOP/s = {100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak), host wall {wall_ms:.3f} ms/step")
 
+    fp8_info = None
+    if not rounding and not cfg["zipf"] and H % 128 == 0 and I % 128 == 0:
+        from sonicmoe import enable_fp8_forward
+
+        with torch.no_grad():
+            ref_out = layer()
+            from sonicmoe.functional.fp8 import cache_quantized_weights
+
+            with enable_fp8_forward():
+                fp8_out = layer()
+                with cache_quantized_weights(False):
+                    fp8_ms, _ = time_region(fwd_only, a.steps, a.warmup)
+                fp8_cached_ms, _ = time_region(fwd_only, a.steps, a.warmup)
+        rel = float((fp8_out.float() - ref_out.float()).norm() / ref_out.float().norm())
+        fp8_info = dict(
+            what="forward with block-scaled e4m3 operands (x, W1, y1, W2 quantised inside the timed region), bf16 outputs; "
+            "fwd_ms_weights_quantised_once: W1, W2 quantised before the timed region (inference)",
+            fwd_ms=round(fp8_ms, 4),
+            fwd_ms_weights_quantised_once=round(fp8_cached_ms, 4),
+            fwd_tflops=round(flops_fwd / fp8_ms / 1e9, 2),
+            frac_of_fp8_peak=round(flops_fwd / fp8_ms / 1e9 / PEAK_FP8_TFLOPS, 4),
+            rel_l2_vs_bf16_forward=round(rel, 4),
+        )
+        log(f"fp8 forward: {fp8_ms:.3f} ms ({fp8_info['fwd_tflops']:.1f} TFLOP/s), rel-L2 vs bf16 forward {rel:.4f}")
+        del ref_out, fp8_out
+
     rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, x, wr, w1, w2, dout, max(5, a.steps // 2))
     # dominant kernel = the single grouped-GEMM launch with the largest average duration
     single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS]
@@ -333,6 +382,7 @@ def main():
         fwd_ms=round(fwd_ms, 4),
         fwd_tflops=round(flops_fwd / fwd_ms / 1e9, 2),
         roofline=roofline,
+        fp8_forward=fp8_info,
         kernels=[{k: v for k, v in r.items() if k != "flops"} for r in rows],
     )
     if not a.no_cpu_baseline:

@@ -58,13 +58,40 @@ def mx_quantize(t: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return q, scales
 
 
+# quantised copies of expert weights, valid while the parameter has not been written to (its version counter is
+# unchanged): inference and repeated forwards quantise a weight once, a training step re-quantises after the optimizer
+_WEIGHT_CACHE: dict[tuple, tuple] = {}
+_WEIGHT_CACHE_MAX = 8
+_CACHE_WEIGHTS = True
+
+
+@contextmanager
+def cache_quantized_weights(enable: bool = True):
+    global _CACHE_WEIGHTS
+    previous, _CACHE_WEIGHTS = _CACHE_WEIGHTS, enable
+    try:
+        yield
+    finally:
+        _CACHE_WEIGHTS = previous
+
+
 def quantize_expert_weight(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """w_view is the (out, in, E) permuted view of an (E, out, in) parameter; quantised along `in`."""
     w = w_view.permute(2, 0, 1)
     if not w.is_contiguous():
         w = w.contiguous()
     E, N, K = w.shape
-    return mx_quantize(w.reshape(E * N, K))
+    if not _CACHE_WEIGHTS or torch.compiler.is_compiling():
+        return mx_quantize(w.detach().reshape(E * N, K))
+    key = (w.data_ptr(), tuple(w.shape), w.device.index)
+    hit = _WEIGHT_CACHE.get(key)
+    if hit is not None and hit[0] == w._version:
+        return hit[1], hit[2]
+    q, scales = mx_quantize(w.detach().reshape(E * N, K))
+    if len(_WEIGHT_CACHE) >= _WEIGHT_CACHE_MAX:
+        _WEIGHT_CACHE.pop(next(iter(_WEIGHT_CACHE)))
+    _WEIGHT_CACHE[key] = (w._version, q, scales)
+    return q, scales
 
 
 @torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_forward_fp8", mutates_args={"z", "y1"})

@@ -112,3 +112,24 @@ def test_layer_with_fp8_forward(dev):
     assert 1e-2 < err < 8e-2, err   # measured ~6e-2: two quantised GEMMs in series exceed the per-operator 5e-2
     for a, b in zip(grads8, grads):
         assert rel_l2(a, b) < 8e-2  # bf16 backward from the fp8-forward z
+
+
+def test_quantised_weight_cache_follows_parameter_updates(dev):
+    """The cached quantised weights are dropped when the parameter is written to (optimizer step)."""
+    from sonicmoe import MoE, enable_fp8_forward
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional.fp8 import cache_quantized_weights
+
+    torch.manual_seed(5)
+    moe = MoE(8, 2, 256, 128, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+    x = torch.randn(512, 256, device=dev).to(torch.bfloat16)
+    with torch.no_grad(), enable_fp8_forward():
+        a, _ = moe(x)
+        b, _ = moe(x)                      # second call: cache hit
+        moe.c_proj.weight.mul_(2.0)        # in-place update bumps the version counter
+        c, _ = moe(x)
+        with cache_quantized_weights(False):
+            d, _ = moe(x)
+    assert torch.equal(a, b)
+    assert torch.equal(c, d)
+    assert rel_l2(c, 2.0 * a.float()) < 1e-2
