@@ -20,6 +20,9 @@ tests/test_oracle_*.py):
   moe_math.moe_torch_backend      pinned: reduces to F.linear / F.silu / index_add; E=1 dense MLP special case
   moe_math.* explicit backward    pinned: torch.autograd through the restated forward in fp64
   moe_math.switch_aux_loss        pinned: closed form (uniform routing -> 1)
-  fp8.*                           PARITY UNPINNED: the reference has no fp8 implementation, test or number;
-                                  checked only against the bf16 oracle within the stated tolerance
+  moe_math.activation_forward / activation_backward   pinned: torch.nn.functional routines; autograd in fp64
+  moe_math bias terms (db1, db2, ds bias term)        pinned: torch.autograd through the restated forward in fp64
+  fp8.*                           PARITY UNPINNED against the reference, which has no fp8 implementation, test or
+                                  number; the format itself is pinned: decode table and element rounding against
+                                  torch.float8_e4m3fn, block scales against their defining inequalities
 """
