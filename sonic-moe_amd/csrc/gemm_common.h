@@ -114,7 +114,8 @@ SMOE_DEV void lds_barrier() {
 //   last slice: wait until this wave's pieces of the NEXT stage have landed (vmcnt leaves the younger stages in
 //            flight), workgroup barrier (everyone's pieces landed; everyone drained the current stage), refill the
 //            current stage's slot with stage s+NSTAGE, read slice 0 of the next stage while the last MFMAs run.
-//   issue(buf, s)                 start this wave's LPS direct-to-LDS loads of stage s into ring slot buf
+//   issue(buf, s, i)              start the i-th (compile-time index, 0 <= i < LPS) of this wave's direct-to-LDS loads of
+//                                 stage s into ring slot buf; called with i ascending, stages in order
 //   load(buf, s, ks, qf, pf)      read the fragments of slice ks of stage s from ring slot buf
 // MFMA operand fragment + instruction of the bf16 kernels; the fp8 kernels bring their own pair
 struct Bf16Mma {
@@ -128,8 +129,10 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
   static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
   static_assert(SLICES % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 6, "unsupported pipeline shape");
   typename Mma::Frag qf[2][NQ], pf[2][NP];
+  constexpr int NM = NQ * NP;
+  auto issue_all = [&](int buf, int s) { static_for<LPS>([&](auto i_c) { issue(buf, s, i_c); }); };
   const int pre = S < NSTAGE ? S : NSTAGE;
-  for (int s = 0; s < pre; s++) issue(s, s);
+  for (int s = 0; s < pre; s++) issue_all(s, s);
 
   auto wait_next_stage = [&](int younger) {  // `younger` stages were issued after the one we need
     if constexpr (NSTAGE >= 6) if (younger >= 4) { wait_vmem_upto<4 * LPS>(); return; }
@@ -146,13 +149,27 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
     for (int q = 0; q < NQ; q++)
 #pragma unroll
       for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
-    constexpr int NM = NQ * NP, NR = NREADS < NM ? NREADS : NM - 1;
+    constexpr int NR = NREADS < NM ? NREADS : NM - 1;
 #pragma unroll
     for (int i = 0; i < NR; i++) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
       __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  };
+  // the last slice of a stage whose ring slot is refilled: the refill's load instructions (address arithmetic, M0
+  // set-up, the load) are dealt out between the MFMAs instead of standing in front of them, so the matrix pipe does
+  // not idle while every wave of the SIMD issues its loads right after the barrier
+  auto slice_mfma_refill = [&](int buf, int s_new) {
+    static_for<NM>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
+      static_for<LPS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        if constexpr (j * NM / LPS == i) issue(buf, s_new, j_c);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
   };
   auto inner_slices = [&](int buf, int s) {
     static_for<SLICES - 1>([&](auto ks_c) {
@@ -166,14 +183,24 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
   lds_barrier();
   load(0, 0, 0, qf[0], pf[0]);
   int buf = 0;
-  for (int s = 0; s < S - 1; s++) {
+  int s = 0;
+#ifndef SMOE_PROBE_NO_REFILL
+  for (; s + NSTAGE < S; s++) {  // steady state: every stage boundary refills the slot it frees
+    inner_slices(buf, s);
+    wait_next_stage(NSTAGE - 2);
+    lds_barrier();
+    const int next = buf + 1 == NSTAGE ? 0 : buf + 1;
+    load(next, s + 1, 0, qf[0], pf[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    slice_mfma_refill(buf, s + NSTAGE);
+    buf = next;
+  }
+#endif
+  for (; s < S - 1; s++) {  // drain: nothing left to fetch
     inner_slices(buf, s);
     const int younger = S - 2 - s < NSTAGE - 2 ? S - 2 - s : NSTAGE - 2;
     wait_next_stage(younger);
     lds_barrier();
-#ifndef SMOE_PROBE_NO_REFILL
-    if (s + NSTAGE < S) issue(buf, s + NSTAGE);
-#endif
     buf = buf + 1 == NSTAGE ? 0 : buf + 1;
     load(buf, s + 1, 0, qf[0], pf[0]);
     slice_mfma(std::integral_constant<int, 1>{});

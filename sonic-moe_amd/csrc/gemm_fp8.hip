@@ -233,20 +233,18 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
 
-  auto issue = [&](int buf, int /*s*/) {
+  auto issue = [&](int buf, int /*s*/, auto i_c) {
+    constexpr int i = decltype(i_c)::value;
     const uint32_t base = smem_base + buf * C::STAGE;
-#pragma unroll
-    for (int i = 0; i < C::P_INSTR; i++) {
+    if constexpr (i < C::P_INSTR) {
       load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
       p_src[i] += C::BKB;
-    }
-#pragma unroll
-    for (int i = 0; i < C::Q_INSTR; i++) {
-      load16_to_lds(q_src[i], base + C::P_STAGE + (wave * C::Q_INSTR + i) * 1024);
-      q_src[i] += C::BKB;
-    }
-#pragma unroll
-    for (int j = 0; j < C::S_INSTR; j++) {
+    } else if constexpr (i < C::P_INSTR + C::Q_INSTR) {
+      constexpr int j = i - C::P_INSTR;
+      load16_to_lds(q_src[j], base + C::P_STAGE + (wave * C::Q_INSTR + j) * 1024);
+      q_src[j] += C::BKB;
+    } else {
+      constexpr int j = i - C::P_INSTR - C::Q_INSTR;
       load4_to_lds(s_src[j], base + C::P_STAGE + C::Q_STAGE + (wave * C::S_INSTR + j) * 256);
       s_src[j] += s_step[j];
     }

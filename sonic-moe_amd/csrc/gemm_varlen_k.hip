@@ -152,17 +152,19 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     const uint16_t* src = base + row * stride + col;
     return t < 0 ? zero : src;
   };
-  auto issue = [&](int buf, int s) {
+  auto issue = [&](int buf, int s, auto i_c) {
+    constexpr int i = decltype(i_c)::value;
     const uint32_t base = smem_base + buf * C::STAGE;
-#pragma unroll
-    for (int i = 0; i < C::R_INSTR; i++)
+    if constexpr (i < C::R_INSTR) {
       load16_to_lds(piece(p.R, p.r_stride, C::R_GATHER, C::R_RPI, C::R_LPR, s, i, r_col[i]),
                     base + (wave * C::R_INSTR + i) * 1024);
-#pragma unroll
-    for (int i = 0; i < C::S_INSTR; i++)
-      load16_to_lds(piece(p.S, p.s_stride, C::S_GATHER, C::S_RPI, C::S_LPR, s, i, s_col[i]),
-                    base + C::R_STAGE + (wave * C::S_INSTR + i) * 1024);
-    if (s + 1 < S) fetch(s + 1);  // stages are issued in order: have the next one's rows ready
+    } else {
+      constexpr int j = i - C::R_INSTR;
+      load16_to_lds(piece(p.S, p.s_stride, C::S_GATHER, C::S_RPI, C::S_LPR, s, j, s_col[j]),
+                    base + C::R_STAGE + (wave * C::S_INSTR + j) * 1024);
+    }
+    if constexpr (i == C::R_INSTR + C::S_INSTR - 1)
+      if (s + 1 < S) fetch(s + 1);  // stages are issued in order: have the next one's rows ready
   };
   auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
     const char* st = smem + buf * C::STAGE;

@@ -162,17 +162,16 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
 
-  auto issue = [&](int buf, int /*s*/) {
+  auto issue = [&](int buf, int /*s*/, auto i_c) {
+    constexpr int i = decltype(i_c)::value;
     const uint32_t base = smem_base + buf * C::STAGE;
-#pragma unroll
-    for (int i = 0; i < C::P_INSTR; i++) {
+    if constexpr (i < C::P_INSTR) {
       load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
       p_src[i] += BK;
-    }
-#pragma unroll
-    for (int i = 0; i < C::Q_INSTR; i++) {
-      load16_to_lds(q_src[i], base + C::P_STAGE + (wave * C::Q_INSTR + i) * 1024);
-      q_src[i] += q_step;
+    } else {
+      constexpr int j = i - C::P_INSTR;
+      load16_to_lds(q_src[j], base + C::P_STAGE + (wave * C::Q_INSTR + j) * 1024);
+      q_src[j] += q_step;
     }
   };
   auto load = [&](int buf, int /*s*/, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
