@@ -279,7 +279,7 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
                "down_projection_backward: null pointer");
   SMOE_REQUIRE(TK == 0 || !dz || (z && w2 && y1s && ds && ds_partial && scores && s_scatter_idx), SMOE_ERR_INVALID,
                "down_projection_backward: null pointer");
-  SMOE_REQUIRE(!db2 || (scores && s_scatter_idx), SMOE_ERR_INVALID,
+  SMOE_REQUIRE(TK == 0 || !db2 || (scores && s_scatter_idx), SMOE_ERR_INVALID,
                "down_projection_backward: db2 needs scores and s_scatter_idx");
   (void)T;
   hipStream_t st = (hipStream_t)stream;

@@ -157,6 +157,9 @@ def _gather_sum(src, out, weights, ridx, tok_off, K, H, is_varlen_K, what):
     assert src.is_contiguous() and out.is_contiguous() and ridx.dtype == torch.int32
     if weights is not None:
         assert weights.dtype == torch.float32 and weights.is_contiguous()
+    if src.size(0) == 0:  # no routed row at all: every token's sum is empty
+        out.zero_()
+        return
     rc = _lib.lib().smoe_gather_sum(
         _lib.ptr(src),
         _lib.ptr(out),

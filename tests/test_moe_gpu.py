@@ -144,3 +144,36 @@ def test_torch_compile_fullgraph(dev):
     assert torch.equal(out, out_c)
     for a, b in zip(grads, grads_c):
         assert rel_l2(a, b) < 5e-3  # dx: the compiled graph fuses the two dx contributions before the bf16 rounding
+
+
+def test_empty_batch(dev):
+    """Zero tokens: every operator accepts empty tensors; the weight gradients are zeros."""
+    from sonicmoe import MoE
+    from sonicmoe.enums import ActivationType
+
+    torch.manual_seed(0)
+    moe = MoE(8, 2, 256, 128, ActivationType.SWIGLU, True, 0.02).to(device=dev, dtype=torch.bfloat16)
+    x = torch.zeros(0, 256, dtype=torch.bfloat16, device=dev, requires_grad=True)
+    out, aux = moe(x)
+    assert out.shape == (0, 256)
+    params = [moe.c_fc.weight, moe.c_fc.bias, moe.c_proj.weight, moe.c_proj.bias]
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=torch.zeros_like(out))
+    assert grads[0].shape == (0, 256)
+    for g in grads[1:]:
+        assert bool((g == 0).all())
+
+
+def test_general_routing_without_pairs(dev):
+    """General routing entry with no (token, expert) pair at all: the output is zero."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import moe_general_routing_inputs
+    from helpers import make_weights
+
+    T, H, I, E = 64, 256, 128, 4
+    _, w1, w2 = make_weights(E, H, I, dev, seed=1)
+    x = torch.randn(T, H, device=dev).to(torch.bfloat16)
+    empty_i = torch.zeros(0, dtype=torch.int32, device=dev)
+    o, freq = moe_general_routing_inputs(x, torch.zeros(0, device=dev), empty_i, empty_i, w1.permute(1, 2, 0), None,
+                                         w2.permute(1, 2, 0), None, E, torch.cuda.current_stream().cuda_stream,
+                                         ActivationType.SWIGLU, False)
+    assert o.shape == (T, H) and bool((o == 0).all()) and bool((freq == 0).all())
