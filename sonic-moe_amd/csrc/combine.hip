@@ -32,7 +32,7 @@ __global__ __launch_bounds__(256) void gather_sum_kernel(const uint16_t* __restr
         if (j < hi) {
           const int64_t r = ridx[j];
           ws[u] = w ? w[j] : 1.0f;
-          v[u] = *(const u32x4*)(src + r * H + (int64_t)c * 8);
+          v[u] = __builtin_nontemporal_load((const u32x4*)(src + r * H + (int64_t)c * 8));
         } else {
           ws[u] = 0.f;
           v[u] = u32x4{0, 0, 0, 0};
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(256) void gather_sum_kernel(const uint16_t* __restr
     u32x4 o;
 #pragma unroll
     for (int q = 0; q < 4; q++) o[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
-    *(u32x4*)(out + t * H + (int64_t)c * 8) = o;
+    __builtin_nontemporal_store(o, (u32x4*)(out + t * H + (int64_t)c * 8));
   }
 }
 
