@@ -123,7 +123,8 @@ struct Bf16Mma {
   static __device__ __forceinline__ f32x16 run(const Frag& q, const Frag& p, f32x16 c) { return mfma32(q, p, c); }
 };
 
-template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Mma = Bf16Mma, class Issue, class Load>
+// RPM: LDS reads slotted in behind each of the first MFMAs of a slice
+template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Mma = Bf16Mma, int RPM = 1, class Issue, class Load>
 SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, Load&& load) {
   if (S <= 0) return;
   static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
@@ -149,11 +150,11 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
     for (int q = 0; q < NQ; q++)
 #pragma unroll
       for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
-    constexpr int NR = NREADS < NM ? NREADS : NM - 1;
+    constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
 #pragma unroll
     for (int i = 0; i < NR; i++) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
     }
     __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
   };

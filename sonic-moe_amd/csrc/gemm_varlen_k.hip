@@ -177,7 +177,8 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   };
   if (S > 0) fetch(0);
   // MFMA as D[b][a] += S[b][k] R[k][a]: lane owns output row a = l%32, register quads hold 4 consecutive columns b
-  gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE>(S, acc, issue, load);
+  // two transpose loads per fragment: 12 reads for the 8 MFMAs of a slice, issued two per MFMA
+  gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE, Bf16Mma, 2>(S, acc, issue, load);
 
   // epilogue through LDS (also writes the zeros of experts without tokens)
   using L = EpiLayout<C::TB>;
