@@ -363,6 +363,22 @@ SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int 
   }
 }
 
+// ---- launch helper -------------------------------------------------------------------------------------------------
+// Raise a kernel's dynamic-LDS limit once per device (the attribute is per device; a repeated call is harmless, so the
+// flags need no lock).
+struct LdsLimitOnce {
+  bool done[64] = {};
+  int ensure(const void* kernel, int bytes) {
+    int dev = 0;
+    SMOE_HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64 || !done[dev]) {
+      SMOE_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+      if (dev >= 0 && dev < 64) done[dev] = true;
+    }
+    return SMOE_OK;
+  }
+};
+
 // ---- tile map ------------------------------------------------------------------------------------------------
 // Built on the device from the expert offsets; header[0] = number of token tiles.  Entry i = (expert, first row).
 struct TileMap {

@@ -287,11 +287,11 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
 template <bool WITH_ACT, int ACT>
 static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
   using C = Fp8Cfg;
-  static bool attr_set = false;
+  static LdsLimitOnce lds_limit;
   auto kern = fp8_varlen_m_kernel<WITH_ACT, ACT>;
-  if (!attr_set) {
-    SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
-    attr_set = true;
+  {
+    const int rc_attr = lds_limit.ensure((const void*)kern, C::SMEM);
+    if (rc_attr) return rc_attr;
   }
   p.tm = carve_tile_map(workspace, TK, E, C::BM);
   int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);

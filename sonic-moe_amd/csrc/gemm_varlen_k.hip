@@ -200,11 +200,11 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 
 template <class C>
 static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
-  static bool attr_set = false;
+  static LdsLimitOnce lds_limit;
   auto kern = varlen_k_kernel<C>;
-  if (!attr_set) {
-    SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
-    attr_set = true;
+  {
+    const int rc_attr = lds_limit.ensure((const void*)kern, C::SMEM);
+    if (rc_attr) return rc_attr;
   }
   VarlenKParams p = pin;
   p.tiles_a = (int)ceil_div(p.NA, C::BA);

@@ -318,11 +318,11 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 
 template <class C, int ROLE, int ACT>
 static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
-  static bool attr_set = false;
+  static LdsLimitOnce lds_limit;
   auto kern = varlen_m_kernel<C, ROLE, ACT>;
-  if (!attr_set) {
-    SMOE_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, C::SMEM));
-    attr_set = true;
+  {
+    const int rc_attr = lds_limit.ensure((const void*)kern, C::SMEM);
+    if (rc_attr) return rc_attr;
   }
   p.tm = carve_tile_map(workspace, TK, E, C::BM);
   int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
