@@ -157,6 +157,35 @@ int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride
                                 size_t workspace_bytes, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------
+ * Token-rounding router (benchmarks/moe-token-rounding.py:139-191 of the reference, there a chain of torch ops
+ * with a dense (T, E) argsort).  Chain: smoe_tr_softmax -> smoe_topk_softmax_fwd(probs, softmax = 0) ->
+ * smoe_count_cumsum -> smoe_tr_rank -> (targets = rounded counts) -> smoe_tr_select -> smoe_tr_row_counts ->
+ * (exclusive scan of the counts) -> smoe_tr_compact.  `dtype` is SMOE_DT_BF16 or SMOE_DT_F16; E <= 4096.
+ * ------------------------------------------------------------------------------------------------------ */
+
+/* probs (T, E) = softmax(logits, fp32) rounded to `dtype` (:149) */
+int smoe_tr_softmax(const void* logits, int dtype, int64_t T, int E, int64_t row_stride, void* probs, void* stream);
+
+/* Renormalise the K picks of every token by their sum, write them back into probs, and fill
+ * rank[t, e] = renormalised value for a pick, probs[t, e] - 1 otherwise (:158-164); top_v / top_i (T, K) are the
+ * picks' values (fp32 images of the 16-bit probabilities) and columns. */
+int smoe_tr_rank(void* probs, void* rank, int dtype, const float* top_v, const int32_t* top_i, int64_t T, int E,
+                 int K, void* stream);
+
+/* keep[t, e] = 1 for the target[e] tokens of expert e with the largest rank[t, e] (ties: lower token first), else 0
+ * (:167-184). */
+int smoe_tr_select(const void* rank, int dtype, const int32_t* target, uint8_t* keep, int64_t T, int E,
+                   void* stream);
+
+/* counts[t] = number of kept experts of token t */
+int smoe_tr_row_counts(const uint8_t* keep, int64_t T, int E, int32_t* counts, void* stream);
+
+/* The kept pairs of token t, experts ascending, at positions [tok_off[t], tok_off[t+1]): scores = probs[t, e] in
+ * `dtype`, token_idx = t, expert_idx = e (:187-191; the reference leaves the order inside a token unspecified). */
+int smoe_tr_compact(const uint8_t* keep, const void* probs, int dtype, const int32_t* tok_off, int64_t T, int E,
+                    void* scores, int32_t* token_idx, int32_t* expert_idx, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------
  * fp8 forward path (OCP e4m3 elements, one power-of-two scale per 32 contraction elements)
  * No counterpart in the reference, which computes in bf16 only; the shapes and epilogues are those of
  * smoe_up_projection_forward / smoe_down_projection_forward above.

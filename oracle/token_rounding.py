@@ -12,17 +12,20 @@ import numpy as np
 from .routing import round_half_even_multiple
 
 
-def token_choice_rounding(probs: np.ndarray, K: int, tile: int, mode: str):
+def token_choice_rounding(probs: np.ndarray, K: int, tile: int, mode: str, rnd=None):
     """`probs` (T, E) float32: softmax probabilities already rounded to the activation dtype (:149).
+    `rnd` rounds a float32 array to the activation dtype (the reference's tensors are in that dtype, so the sum of the
+    picks, their quotients and `scores - 1` are each rounded to it: :158, :163); None = float32 tensors.
     Returns (scores (TK',), token_idx (TK',) int32 ascending, expert_idx (TK',) int32, rounded counts (E,))."""
     T, E = probs.shape
+    rnd = (lambda a: a) if rnd is None else rnd
     p = probs.astype(np.float32).copy()
     top_i = np.argsort(-p, axis=1, kind="stable")[:, :K]  # :152
     top_v = np.take_along_axis(p, top_i, axis=1)
     freq = np.bincount(top_i.reshape(-1), minlength=E).astype(np.int32)  # :154
-    top_v = top_v / top_v.sum(axis=1, keepdims=True)  # :158
+    top_v = rnd(top_v / rnd(top_v.sum(axis=1, keepdims=True, dtype=np.float32)))  # :158
     np.put_along_axis(p, top_i, top_v, axis=1)  # :160
-    rank = p - 1.0  # :162-163
+    rank = rnd(p - np.float32(1.0))  # :162-163
     np.put_along_axis(rank, top_i, top_v, axis=1)  # :164
     target = np.minimum(round_half_even_multiple(freq, tile, mode), T)  # :169-179
     order = np.stack([np.argsort(-rank[:, e], kind="stable") for e in range(E)], axis=1)  # :167, (T, E)

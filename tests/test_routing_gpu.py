@@ -147,3 +147,36 @@ def test_softmax_topk_bwd(dev, dtype):
         np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-7)
     else:
         np.testing.assert_allclose(got, torch.from_numpy(ref).to(dtype).float().numpy(), rtol=1e-2, atol=1e-6)
+
+
+@pytest.mark.parametrize("mode", ["nr", "up", "down"])
+@pytest.mark.parametrize("T,E,K,tile,dtype", [
+    (512, 16, 2, 32, torch.bfloat16),
+    (4096, 64, 4, 128, torch.bfloat16),
+    (3000, 256, 8, 128, torch.float16),     # T not a multiple of the select kernel's 1024-token chunks
+    (200, 8, 2, 128, torch.bfloat16),       # every target is 0 or clamps to T
+])
+def test_token_rounding_router_on_device(dev, mode, T, E, K, tile, dtype):
+    """The HIP token-rounding router against the oracle driven with the same rounded probabilities: the same set of
+    (token, expert) pairs and the same scores (the order inside a token is ascending expert here, unspecified in the
+    reference)."""
+    from oracle import token_rounding as TR
+    from sonicmoe.routing import token_choice_rounding_device
+
+    g = torch.Generator().manual_seed(T + E)
+    logits = (torch.randn(T, E, generator=g) * 1.5).to(dtype).to(dev)
+    sc, tok, exp, probs = token_choice_rounding_device(logits, K, tile, mode)
+    # the device softmax against torch's (both fp32, rounded to the 16-bit dtype): at most one unit in the last place
+    ref_p = torch.softmax(logits.float(), dim=-1).to(dtype)
+    assert float((probs.float() - ref_p.float()).abs().max()) <= float(ref_p.float().max()) * 2.0 ** -7
+
+    rnd = lambda a: torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(dtype).float().numpy()  # noqa: E731
+    sc_o, tok_o, exp_o, target = TR.token_choice_rounding(probs.float().cpu().numpy(), K, tile, mode, rnd=rnd)
+    order = np.lexsort((exp_o, tok_o))
+    tok_o, exp_o, sc_o = tok_o[order], exp_o[order], sc_o[order]
+    assert tok.cpu().numpy().tolist() == tok_o.tolist()
+    assert exp.cpu().numpy().tolist() == exp_o.tolist()
+    assert np.array_equal(sc.float().cpu().numpy(), sc_o)  # same dtype arithmetic: identical bits
+    counts = np.bincount(exp.cpu().numpy(), minlength=E)
+    assert counts.tolist() == target.tolist()
+    assert bool((torch.diff(tok) >= 0).all())
