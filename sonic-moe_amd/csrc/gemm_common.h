@@ -167,7 +167,11 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
       acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
       static_for<LPS>([&](auto j_c) {
         constexpr int j = decltype(j_c)::value;
+#ifdef SMOE_PROBE_HALF_REFILL
+        if constexpr (j * NM / LPS == i && j < LPS / 2) issue(buf, s_new, j_c);
+#else
         if constexpr (j * NM / LPS == i) issue(buf, s_new, j_c);
+#endif
       });
       __builtin_amdgcn_sched_barrier(0);
     });
