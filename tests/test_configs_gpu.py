@@ -145,3 +145,61 @@ def test_full_size_properties(dev):
         y = torch.nn.functional.silu(h[:, 0::2]) * h[:, 1::2]
         ref += scores[sample, j, None] * torch.einsum("ti,thi->th", y, w2.detach()[e].float())
     assert rel_l2(o1.detach()[sample], ref) < TOL
+
+
+def test_tensors_beyond_2_31_elements(dev):
+    """T=65536, K=8, H=4096: the grouped (TK, H) tensors hold 2^31 elements, so any 32-bit element index would wrap.
+    The LAST expert's rows sit at the highest addresses: its weight gradients and the outputs of the last tokens are
+    compared with a dense fp32 evaluation of that expert alone."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import _build_metadata, forward, moe_TC_softmax_topk_layer
+
+    T, H, I, E, K = 65536, 4096, 512, 64, 8
+    g = torch.Generator(device=dev).manual_seed(3)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16).requires_grad_()
+    wr = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    w1 = (0.02 * torch.randn(E, 2 * I, H, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    w2 = (0.02 * torch.randn(E, H, I, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    dout = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    st = torch.cuda.current_stream().cuda_stream
+    o, logits, freq = moe_TC_softmax_topk_layer(x, wr, w1.permute(1, 2, 0), None, w2.permute(1, 2, 0), None, K, st,
+                                                ActivationType.SWIGLU, False)
+    dx, dw1, dw2 = torch.autograd.grad(o, [x, w1, w2], grad_outputs=dout)
+    assert T * K * H >= 2**31
+
+    with torch.no_grad():
+        scores = torch.empty(T, K, dtype=torch.float32, device=dev)
+        idx = torch.empty(T, K, dtype=torch.int32, device=dev)
+        forward._topk_fwd(logits, K, scores, idx, True)
+        _, off, gidx, sidx, _, _ = _build_metadata(idx.view(-1), None, T, E, K)
+        e = E - 1
+        a, b = int(off[e]), int(off[e + 1])
+        assert b == T * K and b - a > 1000
+        tok = gidx[a:b].long()
+        s = scores.view(-1)[sidx[a:b].long()]
+        xe, de = x.detach()[tok].float(), dout[tok].float()
+        z = xe @ w1.detach()[e].float().t()
+        gate, up = z[:, 0::2], z[:, 1::2]
+        sig = torch.sigmoid(gate)
+        y1 = gate * sig * up
+        dy1 = de @ w2.detach()[e].float()
+        dz = torch.empty_like(z)
+        dz[:, 0::2] = s[:, None] * dy1 * up * (gate * sig * (1 - sig) + sig)
+        dz[:, 1::2] = s[:, None] * dy1 * gate * sig
+        dw2_ref = de.t() @ (s[:, None] * y1)
+        dw1_ref = dz.t() @ xe
+    assert rel_l2(dw2[e], dw2_ref) < TOL
+    assert rel_l2(dw1[e], dw1_ref) < TOL
+
+    # forward of the last 32 tokens, densely
+    with torch.no_grad():
+        sample = torch.arange(T - 32, T, device=dev)
+        xs = x.detach()[sample].float()
+        ref = torch.zeros(32, H, device=dev)
+        for j in range(K):
+            ee = idx[sample, j].long()
+            h = torch.einsum("th,tnh->tn", xs, w1.detach()[ee].float())
+            y = torch.nn.functional.silu(h[:, 0::2]) * h[:, 1::2]
+            ref += scores[sample, j, None] * torch.einsum("ti,thi->th", y, w2.detach()[ee].float())
+    assert rel_l2(o.detach()[sample], ref) < TOL
+    assert bool(torch.isfinite(dx.float()).all())
