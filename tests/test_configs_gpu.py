@@ -1,4 +1,4 @@
-"""GPU parity at the remaining BASELINE configurations: Zipf-skewed load with empty experts (config 3, reduced T so
+"""GPU parity at the remaining benchmark configurations: Zipf-skewed load with empty experts (config 3, reduced T so
 that the fp32 oracle finishes in seconds), token-rounding routing through moe_general_routing_inputs (config 4), and
 size-independent properties at the full size of config 2."""
 

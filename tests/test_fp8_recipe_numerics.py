@@ -1,7 +1,7 @@
-"""CPU simulation of the fp8 recipe BASELINE config 5 describes (OCP e4m3, one fp32 scale amax/448 per 128 contiguous
+"""CPU simulation of an fp8 recipe for the layer at its headline shape (OCP e4m3, one fp32 scale amax/448 per 128 contiguous
 elements of the contraction, fp32 accumulation, both operands of every GEMM quantised).
 
-No fp8 kernel is built yet and the reference has no fp8 path to compare with (parity unpinned); this test records what
+The reference has no fp8 path to compare with (parity unpinned); this test records what
 the recipe itself can deliver against the fp32 evaluation: the first GEMM stays inside the 5e-2 bar, but the error of
 SwiGLU(z) and of everything downstream of a second quantised GEMM lands between 5e-2 and 8e-2.  e4m3 keeps 3 mantissa
 bits, i.e. ~2.6 % rms relative rounding error per element, ~3.7 % per product; block scaling cannot change that."""

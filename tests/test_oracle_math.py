@@ -181,7 +181,8 @@ def test_aux_loss_closed_forms():
 
 
 def test_module_torch_backend_on_cpu_matches_oracle():
-    """BASELINE config 1: the module's torch backend in fp32 on the CPU, forward and backward."""
+    """The CPU-runnable configuration (T=1024, H=512, I=256, E=8, K=2): the module's torch backend in fp32, forward and
+    backward."""
     from sonicmoe import KernelBackendMoE, MoE
     from sonicmoe.enums import ActivationType
 
