@@ -338,8 +338,14 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
 }
 
 // 256 x 256 tile, 8 wavefronts as 2 (token) x 4 (feature), 64 of the contraction per stage, double buffer
+#ifdef SMOE_PROBE_TILE_256x128x3
+// timing probe: a 256 x 128 tile leaves room for a third 64-deep stage (two in flight)
+template <bool QMN>
+using TileCfg = Cfg<256, 128, 2, 4, QMN, 64, 3>;
+#else
 template <bool QMN>
 using TileCfg = Cfg<256, 256, 2, 4, QMN, 64, 2>;
+#endif
 
 // one kernel per activation: the epilogue math and (gated or not) the tile geometry of z / y1 depend on it
 template <bool QMN, int ROLE>
