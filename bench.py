@@ -129,8 +129,7 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
             ops += [
                 ("fp8:quantize(x)", lambda: fp8._mx_quantize(xd, xq, xs), None, T * H * 3 + T * H // 32),
                 ("fp8:quantize(W1)", lambda: fp8._mx_quantize(w1_2d, w1q, w1s), None, E * 2 * I * H * 3 + E * 2 * I * H // 32),
-                ("fp8:up_projection_forward", lambda: fp8._up_projection_forward_fp8(xq, xs, w1q, w1s, z, y1, None, off, gidx, E, stream, "swiglu", True), 2 * gemm, None),
-                ("fp8:quantize(y1)", lambda: fp8._mx_quantize(y1, y1q, y1s), None, TK * I * 3 + TK * I // 32),
+                ("fp8:up_projection_forward(+quantised y1)", lambda: fp8._up_projection_forward_fp8(xq, xs, w1q, w1s, z, None, None, off, gidx, E, stream, "swiglu", True, y1q, y1s), 2 * gemm, None),
                 ("fp8:quantize(W2)", lambda: fp8._mx_quantize(w2_2d, w2q, w2s), None, E * H * I * 3 + E * H * I // 32),
                 ("fp8:down_projection_forward", lambda: fp8._down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, None, off, E, stream), gemm, None),
             ]

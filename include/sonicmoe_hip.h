@@ -200,11 +200,15 @@ int smoe_mx_quantize(const void* src, int64_t src_stride, int64_t R, int C, void
 
 /* As smoe_up_projection_forward with x and W1 given in the quantised form above:
  *   xq (T, H) bytes + x_scales (H/128, T); w1q (E, N1, H) bytes contiguous + w1_scales (H/128, E*N1)
- *   z (TK, N1) bf16 or NULL; y1 (TK, I) bf16.  Limits: H % 128 == 0, I % 64 == 0. */
+ *   z (TK, N1) bf16 or NULL; y1 (TK, I) bf16 or NULL;
+ *   y1q (TK, I) bytes + y1q_scales (I/128, TK) or both NULL: the activation output quantised in the epilogue from
+ *   the fp32 values, ready for smoe_down_projection_forward_fp8 (needs I % 128 == 0).
+ * Limits: H % 128 == 0, I % 64 == 0; at least one of y1, y1q. */
 int smoe_up_projection_forward_fp8(const void* xq, const void* x_scales, const void* w1q, const void* w1_scales,
-                                   const void* b1, void* z, void* y1, const int32_t* off,
-                                   const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
-                                   int activation, void* workspace, size_t workspace_bytes, void* stream);
+                                   const void* b1, void* z, void* y1, void* y1q, void* y1q_scales,
+                                   const int32_t* off, const int32_t* x_gather_idx, int64_t T, int64_t TK, int H,
+                                   int I, int E, int activation, void* workspace, size_t workspace_bytes,
+                                   void* stream);
 
 /* As smoe_down_projection_forward with y1 and W2 quantised:
  *   y1q (TK, I) bytes + y1_scales (I/128, TK); w2q (E, H, I) bytes contiguous + w2_scales (I/128, E*H)

@@ -296,7 +296,7 @@ struct FwdEpilogueArgs {
   const uint16_t* bias;  // this expert's bias row (N values) or null
   uint16_t* out0;        // accumulator (+bias) as bf16: z resp. y2; null = not stored
   int64_t out0_stride;
-  uint16_t* out1;        // activation output y1 (WITH_ACT only)
+  uint16_t* out1;        // activation output y1 (WITH_ACT only); null = not stored
   int64_t out1_stride;
   int m_base, row_end;   // first grouped row of this wave's tile, end of the expert's rows
   int n_base, N;         // first accumulator column of this wave's tile, number of accumulator columns
@@ -342,6 +342,7 @@ SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int 
     epilogue_flush<TM, TN>(region, lane, a.out0, a.out0_stride, a.m_base, a.row_end, a.n_base, a.N);
   }
   if constexpr (WITH_ACT && GLU) {
+    if (a.out1 != nullptr) {
     static_for<FM>([&](auto fm_c) {
       constexpr int fm = decltype(fm_c)::value;
       static_for<FN * 4>([&](auto q_c) {
@@ -353,7 +354,9 @@ SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int 
       });
     });
     epilogue_flush<TM, TN / 2>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base / 2, a.N / 2);
+    }
   } else if constexpr (WITH_ACT) {
+    if (a.out1 != nullptr) {
     static_for<FM>([&](auto fm_c) {
       constexpr int fm = decltype(fm_c)::value;
       static_for<FN * 4>([&](auto q_c) {
@@ -364,6 +367,7 @@ SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int 
       });
     });
     epilogue_flush<TM, TN>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base, a.N);
+    }
   }
 }
 

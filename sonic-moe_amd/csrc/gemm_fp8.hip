@@ -101,6 +101,10 @@ struct Fp8Params {
   int64_t out0_stride;
   uint16_t* out1;
   int64_t out1_stride;
+  uint8_t* yq;         // nullable: the activation output quantised in the epilogue, (TK, I) e4m3 bytes
+  uint32_t* yq_scales; // its scale table (I / 128, TK)
+  int64_t yq_rows;     // TK
+  int I;
 };
 
 struct Fp8Cfg {
@@ -138,6 +142,76 @@ struct Fp8Mma {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(q.data, p.data, c, 0, 0, 0, q.scale, 0, p.scale);
   }
 };
+
+// Activation output of the wave's TM x TN accumulator tile (bias already added) quantised straight from the fp32
+// values: per 32-row fragment row, every 32 output columns get their power-of-two scale (lane-local maximum over the
+// lane's columns of the block, one shuffle for the other half-wave), the e4m3 bytes are parked in LDS and written back
+// 16 bytes per lane; the scale bytes go to the (I / 128, rows) table the down-projection reads.
+template <int TM, int TN, int FM, int FN, int ACT>
+SMOE_DEV void fp8_activation_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int lane, uint8_t* yq, int I,
+                                      uint32_t* yq_scales, int64_t yq_rows, int m_base, int row_end, int n_base) {
+  constexpr bool GLU = act_is_glu(ACT);
+  constexpr int PW = act_pointwise(ACT);
+  constexpr int YC = GLU ? TN / 2 : TN;      // output columns of the wave tile
+  constexpr int NB = YC / 32, FPB = FN / NB;  // 32-column blocks, accumulator fragments per block
+  constexpr int ROWB = YC + 16;               // parked row, padded against bank conflicts
+  constexpr int LPR = YC / 16, RPP = 64 / LPR;
+  // the wave's own parking region of forward_epilogue (other waves may still be flushing theirs)
+  char* region = smem + wave * (TM * (TN * 2 + 16));
+  const int half = lane >> 5, mrow = lane & 31;
+  const int y_base = GLU ? n_base / 2 : n_base;
+  static_for<FM>([&](auto fm_c) {
+    constexpr int fm = decltype(fm_c)::value;
+    const int m = m_base + fm * 32 + mrow;
+    static_for<NB>([&](auto b_c) {
+      constexpr int b = decltype(b_c)::value;
+      float y[FPB * 4 * (GLU ? 2 : 4)];
+      float amax = 0.f;
+      static_for<FPB * 4>([&](auto q_c) {
+        constexpr int f = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4, fn = b * FPB + f;
+        if constexpr (GLU) {
+          const float y0 = pointwise<PW>(acc[fn][fm][4 * rg + 0]) * acc[fn][fm][4 * rg + 1];
+          const float y1 = pointwise<PW>(acc[fn][fm][4 * rg + 2]) * acc[fn][fm][4 * rg + 3];
+          y[(f * 4 + rg) * 2 + 0] = y0;
+          y[(f * 4 + rg) * 2 + 1] = y1;
+          amax = fmaxf(amax, fmaxf(fabsf(y0), fabsf(y1)));
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float v = pointwise<PW>(acc[fn][fm][4 * rg + q]);
+            y[rg * 4 + q] = v;
+            amax = fmaxf(amax, fabsf(v));
+          }
+        }
+      });
+      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      const int ex = mx_scale_exponent(amax);
+      const float inv = __uint_as_float((uint32_t)(254 - ex) << 23);
+      static_for<FPB * 4>([&](auto q_c) {
+        constexpr int f = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        if constexpr (GLU) {
+          const int w = __builtin_amdgcn_cvt_pk_fp8_f32(y[(f * 4 + rg) * 2] * inv, y[(f * 4 + rg) * 2 + 1] * inv, 0, false);
+          *(uint16_t*)(region + mrow * ROWB + b * 32 + f * 16 + 4 * rg + 2 * half) = (uint16_t)w;
+        } else {
+          int w = __builtin_amdgcn_cvt_pk_fp8_f32(y[rg * 4] * inv, y[rg * 4 + 1] * inv, 0, false);
+          w = __builtin_amdgcn_cvt_pk_fp8_f32(y[rg * 4 + 2] * inv, y[rg * 4 + 3] * inv, w, true);
+          *(uint32_t*)(region + mrow * ROWB + b * 32 + 8 * rg + 4 * half) = (uint32_t)w;
+        }
+      });
+      const int col = y_base + b * 32;  // first output column of the block
+      if (half == 0 && m < row_end && col < I)
+        ((uint8_t*)yq_scales)[((int64_t)(col >> 7) * yq_rows + m) * 4 + ((col >> 5) & 3)] = (uint8_t)ex;
+    });
+    // the wavefront's own LDS accesses execute in order: the rows parked above are complete here
+#pragma unroll
+    for (int it = 0; it < 32 / RPP; it++) {
+      const int r = it * RPP + lane / LPR, c16 = lane % LPR;
+      const u32x4 v = *(const u32x4*)(region + r * ROWB + c16 * 16);
+      const int mm = m_base + fm * 32 + r, col = y_base + c16 * 16;
+      if (mm < row_end && col < I) *(u32x4*)(yq + (int64_t)mm * I + col) = v;
+    }
+  });
+}
 
 template <bool WITH_ACT, int ACT>
 __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Params p) {
@@ -282,6 +356,11 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
   wait_vmem_all();
   lds_barrier();  // all waves are done reading the last stage
   forward_epilogue<C::TM, C::TN, FM, FN, WITH_ACT, ACT>(acc, smem, wave, lane, ea);
+  if constexpr (WITH_ACT) {
+    if (p.yq != nullptr)  // the parking area of forward_epilogue is read back by the same wave that wrote it: no barrier
+      fp8_activation_epilogue<C::TM, C::TN, FM, FN, ACT>(acc, smem, wave, lane, p.yq, p.I, p.yq_scales, p.yq_rows,
+                                                          ea.m_base, row_end, ea.n_base);
+  }
 }
 
 template <bool WITH_ACT, int ACT>
@@ -350,10 +429,10 @@ static int check_fp8(int64_t TK, int Kdim, int N, int E, const void* ws, size_t 
 }
 
 extern "C" int smoe_up_projection_forward_fp8(const void* xq, const void* x_scales, const void* w1q,
-                                              const void* w1_scales, const void* b1, void* z, void* y1,
-                                              const int32_t* off, const int32_t* x_gather_idx, int64_t T, int64_t TK,
-                                              int H, int I, int E, int activation, void* workspace,
-                                              size_t workspace_bytes, void* stream) {
+                                              const void* w1_scales, const void* b1, void* z, void* y1, void* y1q,
+                                              void* y1q_scales, const int32_t* off, const int32_t* x_gather_idx,
+                                              int64_t T, int64_t TK, int H, int I, int E, int activation,
+                                              void* workspace, size_t workspace_bytes, void* stream) {
   SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
                "up_projection_forward_fp8: unknown activation code %d", activation);
   const int N1 = act_is_glu(activation) ? 2 * I : I;
@@ -361,8 +440,13 @@ extern "C" int smoe_up_projection_forward_fp8(const void* xq, const void* x_scal
   if (rc) return rc;
   SMOE_REQUIRE(I % 64 == 0, SMOE_ERR_UNSUPPORTED, "up_projection_forward_fp8: I=%d must be a multiple of 64", I);
   if (TK == 0) return SMOE_OK;
-  SMOE_REQUIRE(xq && x_scales && w1q && w1_scales && y1 && off && x_gather_idx && T > 0, SMOE_ERR_INVALID,
+  SMOE_REQUIRE(xq && x_scales && w1q && w1_scales && off && x_gather_idx && T > 0, SMOE_ERR_INVALID,
                "up_projection_forward_fp8: null pointer");
+  SMOE_REQUIRE(y1 || y1q, SMOE_ERR_INVALID, "up_projection_forward_fp8: neither y1 nor y1q is given");
+  SMOE_REQUIRE((y1q == nullptr) == (y1q_scales == nullptr), SMOE_ERR_INVALID,
+               "up_projection_forward_fp8: y1q and y1q_scales come together");
+  SMOE_REQUIRE(!y1q || I % 128 == 0, SMOE_ERR_UNSUPPORTED,
+               "up_projection_forward_fp8: a quantised y1 needs I=%d to be a multiple of 128", I);
   Fp8Params p = {};
   p.P = (const uint8_t*)xq;
   p.p_stride = H;
@@ -382,6 +466,10 @@ extern "C" int smoe_up_projection_forward_fp8(const void* xq, const void* x_scal
   p.out0_stride = N1;
   p.out1 = (uint16_t*)y1;
   p.out1_stride = I;
+  p.yq = (uint8_t*)y1q;
+  p.yq_scales = (uint32_t*)y1q_scales;
+  p.yq_rows = TK;
+  p.I = I;
   return launch_fp8_up(activation, p, off, workspace, TK, E, (hipStream_t)stream);
 }
 

@@ -48,7 +48,7 @@ _SIGNATURES = {
     "smoe_mx_quantize": (c_int, [_P, _L, _L, _I, _P, _P, _P]),
     "smoe_up_projection_forward_fp8": (
         c_int,
-        [_P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
+        [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
     "smoe_down_projection_forward_fp8": (c_int, [_P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P, _Z, _P]),
 }

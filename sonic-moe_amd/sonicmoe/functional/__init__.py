@@ -179,14 +179,18 @@ class _ExpertsFunction(torch.autograd.Function):
         scores_flat = scores_flat.contiguous()
 
         z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
-        y1 = torch.empty(TK, I, dtype=x.dtype, device=x.device)
+        y1 = None if is_using_fp8_forward() else torch.empty(TK, I, dtype=x.dtype, device=x.device)
         y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
         if is_using_fp8_forward():
             xq, xs = mx_quantize(x)
             w1q, w1s = quantize_expert_weight(w1)
-            _up_projection_forward_fp8(xq, xs, w1q, w1s, z, y1, b1, off, gidx, E, stream_id, activation_type.value, glu)
+            # y1 leaves the up-projection already quantised (from the fp32 accumulator); its bf16 form is not stored
+            y1q = torch.empty(TK, I, dtype=torch.uint8, device=x.device)
+            y1s = torch.empty(I // 128, TK, dtype=torch.int32, device=x.device)
+            _up_projection_forward_fp8(
+                xq, xs, w1q, w1s, z, None, b1, off, gidx, E, stream_id, activation_type.value, glu, y1q, y1s
+            )
             del xq, xs, w1q, w1s
-            y1q, y1s = mx_quantize(y1)
             w2q, w2s = quantize_expert_weight(w2)
             _down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, b2, off, E, stream_id)
             del y1q, y1s, w2q, w2s

@@ -94,14 +94,16 @@ def quantize_expert_weight(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Te
     return q, scales
 
 
-@torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_forward_fp8", mutates_args={"z", "y1"})
+@torch.library.custom_op(
+    f"{LIBRARY_NAME}::_up_projection_forward_fp8", mutates_args={"z", "y1", "y1q", "y1q_scales"}
+)
 def _up_projection_forward_fp8(
     xq: torch.Tensor,
     x_scales: torch.Tensor,
     w1q: torch.Tensor,
     w1_scales: torch.Tensor,
     z: torch.Tensor | None,
-    y1: torch.Tensor,
+    y1: torch.Tensor | None,
     b1: torch.Tensor | None,
     expert_frequency_offset: torch.Tensor,
     x_gather_idx: torch.Tensor,
@@ -109,12 +111,16 @@ def _up_projection_forward_fp8(
     stream_id: int,
     activation_type: str,
     is_glu_activation: bool,
+    y1q: torch.Tensor | None = None,
+    y1q_scales: torch.Tensor | None = None,
 ) -> None:
-    """z = gather(xq) w1q^T (+ b1) with the block scales applied, y1 = act(z); xq (T, H), w1q (E*N1, H)."""
-    _lib.require_device(xq, x_scales, w1q, w1_scales, y1, b1, expert_frequency_offset, x_gather_idx)
+    """z = gather(xq) w1q^T (+ b1) with the block scales applied, y1 = act(z); xq (T, H), w1q (E*N1, H).  y1 comes back
+    in bf16 (`y1`) and / or quantised in the epilogue (`y1q` (TK, I) uint8 with `y1q_scales` (I/128, TK) int32)."""
+    _lib.require_device(xq, x_scales, w1q, w1_scales, y1, y1q, y1q_scales, b1, expert_frequency_offset, x_gather_idx)
     _check_bf16(("z", z), ("y1", y1), ("b1", b1))
     T, H = xq.shape
-    TK, I = y1.shape
+    TK, I = (y1 if y1 is not None else y1q).shape
+    assert y1q is None or (y1q.dtype == torch.uint8 and y1q.is_contiguous() and y1q_scales.shape == (I // 128, TK))
     N1 = 2 * I if is_glu_activation else I
     assert w1q.shape == (E * N1, H) and x_scales.shape == (H // 128, T) and w1_scales.shape == (H // 128, E * N1)
     assert z is None or (z.shape == (TK, N1) and z.is_contiguous())
@@ -127,6 +133,8 @@ def _up_projection_forward_fp8(
         _lib.ptr(b1),
         _lib.ptr(z),
         _lib.ptr(y1),
+        _lib.ptr(y1q),
+        _lib.ptr(y1q_scales),
         _lib.ptr(expert_frequency_offset),
         _lib.ptr(x_gather_idx),
         T,

@@ -72,12 +72,31 @@ def test_fp8_forward_operators(dev, T, H, I, E, K, activation, with_bias, skew, 
     w1q, w1s = fp8.quantize_expert_weight(w1.to(dev).permute(1, 2, 0))
     z = torch.empty(TK, N1, **bf)
     y1 = torch.empty(TK, I, **bf)
-    fp8._up_projection_forward_fp8(xq, xs, w1q, w1s, z, y1, dv(b1), off, gidx, E, stream, activation, glu)
+    y1q_f = torch.empty(TK, I, dtype=torch.uint8, device=dev)
+    y1s_f = torch.zeros(I // 128, TK, dtype=torch.int32, device=dev)
+    fp8._up_projection_forward_fp8(xq, xs, w1q, w1s, z, y1, dv(b1), off, gidx, E, stream, activation, glu, y1q_f, y1s_f)
     z_fq, y1_fq = Q.up_projection_forward_fp8(x, w1, off, gidx, b1=b1, activation=activation)
     assert rel_l2(z, z_fq) < 5e-3      # same operands, fp32 accumulation: what is left is the bf16 rounding of z
     assert rel_l2(y1, y1_fq) < 5e-3
     z_ref, y1_ref = M.up_projection_forward(x, w1, off.cpu(), gidx.cpu(), b1=b1, activation=activation)
     assert rel_l2(z, z_ref) < 5e-2     # one quantised GEMM against the unquantised one: the fp8 tolerance
+
+    # y1 quantised inside the epilogue (from the fp32 values): de-quantised it is y1 up to the e4m3 rounding, every
+    # block's scale is the smallest power of two that avoids saturation, and without the bf16 output the bytes are the same
+    words = y1s_f.cpu().numpy().view(np.uint32).T                        # (TK, I/128)
+    ex = np.stack([(words >> (8 * b)) & 0xFF for b in range(4)], axis=-1).reshape(TK, I // 32).astype(np.uint8)
+    y1_deq = Q.mx_dequantize(y1q_f.cpu(), torch.from_numpy(ex))
+    assert rel_l2(y1_deq, y1_fq) < 4e-2
+    blocks = y1_fq.reshape(TK, I // 32, 32).abs().amax(-1).numpy()
+    scale = 2.0 ** (ex.astype(np.float64) - 127)
+    live = blocks > 1e-6
+    ratio = blocks[live] / scale[live]
+    assert bool((ratio < 448 * 1.02).all()) and bool((ratio > 224 * 0.98).all())
+    y1q_only = torch.empty_like(y1q_f)
+    y1s_only = torch.zeros_like(y1s_f)
+    fp8._up_projection_forward_fp8(xq, xs, w1q, w1s, None, None, dv(b1), off, gidx, E, stream, activation, glu,
+                                   y1q_only, y1s_only)
+    assert torch.equal(y1q_only, y1q_f) and torch.equal(y1s_only, y1s_f)
 
     y1q, y1s = fp8.mx_quantize(y1)
     w2q, w2s = fp8.quantize_expert_weight(w2.to(dev).permute(1, 2, 0))
