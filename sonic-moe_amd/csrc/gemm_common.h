@@ -214,6 +214,99 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
   slice_mfma(std::integral_constant<int, 1>{});
 }
 
+// ---- main loop with an asymmetric ring -------------------------------------------------------------------------------
+// Same pipeline, but the two operands have rings of different depth: the token operand P has 2 slots, the weight
+// operand Q has 3 (2 + 3 slots of 32 KiB are the whole 160 KiB of LDS for a 256 x 256 x 64 tile).  At the boundary
+// behind stage s the loads of P(s+2) and Q(s+3) are issued, in that order, so the wait for stage s+1 leaves only the
+// QI loads of Q(s+2) outstanding: half of a stage's bytes are requested two stages ahead, and only the other half has
+// to come back within one.
+//   issue_p(slot, i) / issue_q(slot, j)   start the i-th / j-th load of this wave into that operand's ring slot; stages
+//                                          are issued in order, so the callee advances its own source pointers
+//   load(p_slot, q_slot, ks, qf, pf)      read the fragments of slice ks
+template <int NQ, int NP, int NREADS, int PI, int QI, int SLICES, class Mma = Bf16Mma, int RPM = 1, class IssueP,
+          class IssueQ, class Load>
+SMOE_DEV void gemm_mainloop_asym(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issue_p, IssueQ&& issue_q, Load&& load) {
+  if (S <= 0) return;
+  static_assert(SLICES % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
+  typename Mma::Frag qf[2][NQ], pf[2][NP];
+  constexpr int NM = NQ * NP, LPS = PI + QI;
+  auto all_p = [&](int slot) { static_for<PI>([&](auto i_c) { issue_p(slot, i_c); }); };
+  auto all_q = [&](int slot) { static_for<QI>([&](auto j_c) { issue_q(slot, j_c); }); };
+  all_p(0);
+  all_q(0);
+  if (S > 1) {
+    all_p(1);
+    all_q(1);
+  }
+  if (S > 2) all_q(2);
+
+  auto slice_mfma = [&](auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+#pragma unroll
+    for (int q = 0; q < NQ; q++)
+#pragma unroll
+      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
+    constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  };
+  // last slice of a stage with the refill (P pieces first, then Q pieces) dealt out between its MFMAs
+  auto slice_mfma_refill = [&](int p_slot, int q_slot) {
+    static_for<NM>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
+      static_for<LPS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        if constexpr (j * NM / LPS == i) {
+          if constexpr (j < PI) issue_p(p_slot, j_c);
+          else issue_q(q_slot, std::integral_constant<int, j - PI>{});
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto inner_slices = [&](int bp, int bq) {
+    static_for<SLICES - 1>([&](auto ks_c) {
+      constexpr int ks = decltype(ks_c)::value;
+      load(bp, bq, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
+      slice_mfma(std::integral_constant<int, (ks & 1)>{});
+    });
+  };
+
+  if (S > 2) wait_vmem_upto<PI + 2 * QI>();  // stage 0 has landed; P1, Q1, Q2 may still be on their way
+  else wait_vmem_all();
+  lds_barrier();
+  load(0, 0, 0, qf[0], pf[0]);
+  int bp = 0, bq = 0, s = 0;
+  for (; s + 3 < S; s++) {  // steady state: P(s+2) and Q(s+3) exist
+    inner_slices(bp, bq);
+    wait_vmem_upto<QI>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
+    lds_barrier();
+    const int np = bp ^ 1, nq = bq == 2 ? 0 : bq + 1;
+    load(np, nq, 0, qf[0], pf[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    slice_mfma_refill(bp, bq);  // the slots stage s leaves behind
+    bp = np;
+    bq = nq;
+  }
+  for (; s < S - 1; s++) {  // drain: at most P(s+2) is left to request
+    inner_slices(bp, bq);
+    wait_vmem_all();
+    lds_barrier();
+    if (s + 2 < S) all_p(bp);
+    bp ^= 1;
+    bq = bq == 2 ? 0 : bq + 1;
+    load(bp, bq, 0, qf[0], pf[0]);
+    slice_mfma(std::integral_constant<int, 1>{});
+  }
+  inner_slices(bp, bq);
+  slice_mfma(std::integral_constant<int, 1>{});
+}
+
 // ---- epilogue through LDS ----------------------------------------------------------------------------------------
 // A wavefront parks its TR x TC accumulator tile (lane = tile row l%32, register quad = 4 consecutive columns) as
 // bf16 in its own LDS region with padded rows, then reads it back row-contiguous and writes 16 bytes per lane.

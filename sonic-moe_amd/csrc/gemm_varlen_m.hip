@@ -46,7 +46,10 @@ struct Cfg {
   static constexpr int Q_INSTR = Q_STAGE / 1024 / NW;
   static constexpr int KROW = BK * 2;                   // bytes per row of a K-major stage
   static constexpr int EPI = NW * TM * (TN * 2 + 16);   // per-wave parking regions of the LDS epilogue
-  static constexpr int SMEM = NSTAGE * STAGE > EPI ? NSTAGE * STAGE : EPI;
+  // ring: 2 slots of the token operand, then 3 slots of the weight operand (NSTAGE is not used by this kernel)
+  static constexpr int P_SLOTS = 2, Q_SLOTS = 3;
+  static constexpr int RING = P_SLOTS * P_STAGE + Q_SLOTS * Q_STAGE;
+  static constexpr int SMEM = RING > EPI ? RING : EPI;
   // MN-major Q stage geometry
   static constexpr int ROWB = BN * 2;     // bytes per k-row
   static constexpr int LPR = ROWB / 16;   // lanes (16-byte pieces) per k-row
@@ -66,7 +69,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
+  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, SLICES = C::BK / 16;
   const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -139,7 +142,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     const int row = wn * C::TN + (lane & 31);
     const int sw = kswz<BK>(row);
 #pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = C::P_STAGE + row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
   } else {
     const int grp = lane >> 4, i16 = lane & 15;
     const int kk = 8 * (grp >> 1) + (i16 >> 2);
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        q_off[fn * 2 + h] = C::P_STAGE + k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        q_off[fn * 2 + h] = k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
   }
@@ -162,35 +165,36 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
 
-  auto issue = [&](int buf, int /*s*/, auto i_c) {
+  constexpr int Q_RING = C::P_SLOTS * C::P_STAGE;  // byte offset of the weight operand's slots
+  auto issue_p = [&](int slot, auto i_c) {
     constexpr int i = decltype(i_c)::value;
-    const uint32_t base = smem_base + buf * C::STAGE;
-    if constexpr (i < C::P_INSTR) {
-      load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
-      p_src[i] += BK;
-    } else {
-      constexpr int j = i - C::P_INSTR;
-      load16_to_lds(q_src[j], base + C::P_STAGE + (wave * C::Q_INSTR + j) * 1024);
-      q_src[j] += q_step;
-    }
+    load16_to_lds(p_src[i], smem_base + slot * C::P_STAGE + (wave * C::P_INSTR + i) * 1024);
+    p_src[i] += BK;
   };
-  auto load = [&](int buf, int /*s*/, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
+  auto issue_q = [&](int slot, auto j_c) {
+    constexpr int j = decltype(j_c)::value;
+    load16_to_lds(q_src[j], smem_base + Q_RING + slot * C::Q_STAGE + (wave * C::Q_INSTR + j) * 1024);
+    q_src[j] += q_step;
+  };
+  auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
 #ifdef SMOE_PROBE_NO_LDSREAD
     return;
 #endif
-    const char* st = smem + buf * C::STAGE;
+    const char* sp = smem + p_slot * C::P_STAGE;
+    const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
 #pragma unroll
-    for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(st + p_off[ks] + fm * 32 * C::KROW);
+    for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(sp + p_off[ks] + fm * 32 * C::KROW);
 #pragma unroll
     for (int fn = 0; fn < FN; fn++) {
       if constexpr (!C::QMN) {
-        qf[fn] = lds_read_b128(st + q_off[ks] + fn * 32 * C::KROW);
+        qf[fn] = lds_read_b128(sq + q_off[ks] + fn * 32 * C::KROW);
       } else {
-        qf[fn] = lds_read_tr2(st + q_off[fn * 2] + ks * 16 * C::ROWB, st + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
+        qf[fn] = lds_read_tr2(sq + q_off[fn * 2] + ks * 16 * C::ROWB, sq + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
       }
     }
   };
-  gemm_mainloop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR + C::Q_INSTR, SLICES, NSTAGE>(S_total, acc, issue, load);
+  gemm_mainloop_asym<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR, C::Q_INSTR, SLICES>(S_total, acc, issue_p, issue_q,
+                                                                                          load);
 
   const int m_base = row0 + wm * C::TM, n_base = n0 + wn * C::TN;
 #ifdef SMOE_PROBE_NO_EPILOGUE
@@ -223,7 +227,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
     constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
     constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;               // row swizzle of the staged z chunks
-    static_assert(C::NW * 32 * (ZB + YB) <= NSTAGE * C::STAGE, "dz staging must fit into the idle ring");
+    static_assert(C::NW * 32 * (ZB + YB) <= C::RING, "dz staging must fit into the idle ring");
     char* zbuf = smem + wave * (32 * (ZB + YB));
     char* ybuf = zbuf + 32 * ZB;
     const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
