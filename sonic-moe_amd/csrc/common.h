@@ -44,15 +44,17 @@ typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2;
 
 #define SMOE_DEV static __device__ __forceinline__
 
-// bf16 <-> fp32 on raw bits; round-to-nearest-even, NaN kept quiet
+// bf16 <-> fp32.  fp32 -> bf16 is the hardware conversion (v_cvt_pk_bf16_f32: round to nearest even, NaN stays NaN);
+// written out in integer arithmetic it costs ten instructions and a divergent branch per value, which made the GEMM
+// epilogues instruction-bound.
 SMOE_DEV float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
-SMOE_DEV uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-}
 // two floats -> one 32-bit word holding (lo, hi) bf16
-SMOE_DEV uint32_t pack_bf16x2(float lo, float hi) { return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16); }
+SMOE_DEV uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+SMOE_DEV uint32_t f32_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
 SMOE_DEV float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 SMOE_DEV float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 

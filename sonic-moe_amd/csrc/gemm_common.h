@@ -307,6 +307,149 @@ SMOE_DEV void gemm_mainloop_asym(const int S, f32x16 (&acc)[NQ][NP], IssueP&& is
   slice_mfma(std::integral_constant<int, 1>{});
 }
 
+#ifdef SMOE_PROBE_PHASES
+// timing probe: ticks (100 MHz) wave 0 of every workgroup spends in the phases of a tile, summed over the launch
+static __device__ unsigned long long smoe_phase_ticks[8];
+#define SMOE_PHASE_MARK(k) { const unsigned long long now_ = wall_clock64(); phase_[k] += now_ - last_; last_ = now_; }
+#else
+#define SMOE_PHASE_MARK(k)
+#endif
+
+// ---- main loop over a STREAM of tiles ------------------------------------------------------------------------------
+// A workgroup that works through several output tiles keeps the asymmetric ring running across the tile boundary: the
+// stages of the next tile follow the last stage of the current one in the P and Q streams, so the first stages of the
+// next tile are already in LDS when the current tile's epilogue starts, and the epilogue's stores drain while the next
+// tile computes.  Only the epilogue itself (accumulators -> LDS -> global stores) is not overlapped.  It parks its rows
+// in the two ring slots the tile's last stage has just vacated; the refill of those slots waits for the epilogue.
+//   issue_p / issue_q / load   as in gemm_mainloop_asym
+//   issued_p() / issued_q()    called after every stage issued to a stream: the callee counts stages and moves the
+//                              stream's source pointers on to the next tile behind the S-th
+//   first_boundary()           called once per tile behind the wait of its first stage, where no vector-memory
+//                              operation of the wave is outstanding: the place to pick up ordinary loads issued in
+//                              tile_end (a wait for them anywhere else would also wait for the ring)
+//   tile_end(p_slot, q_slot)   epilogue of the finished tile; may use the two slots as scratch (every wave is past the
+//                              barrier behind the last stage); clears the accumulators, advances the caller's tile
+//                              state and returns false if the tile was the workgroup's last
+// Needs S >= 3 (stage 0 of the next tile is requested at the latest behind stage S-3 of the current one).  Stores and
+// loads share one counter and may retire out of order with respect to each other, so the first wait of a tile is for
+// everything; from then on only loads are outstanding and the counted waits are exact again.
+template <int NQ, int NP, int NREADS, int PI, int QI, int SLICES, class Mma = Bf16Mma, int RPM = 1, class IssueP,
+          class IssueQ, class Load, class IssuedP, class IssuedQ, class First, class TileEnd>
+SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issue_p, IssueQ&& issue_q, Load&& load,
+                               IssuedP&& issued_p, IssuedQ&& issued_q, First&& first_boundary, TileEnd&& tile_end) {
+  static_assert(SLICES % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
+  typename Mma::Frag qf[2][NQ], pf[2][NP];
+  constexpr int NM = NQ * NP, LPS = PI + QI;
+  auto all_p = [&](int slot) {
+    static_for<PI>([&](auto i_c) { issue_p(slot, i_c); });
+    issued_p();
+  };
+  auto all_q = [&](int slot) {
+    static_for<QI>([&](auto j_c) { issue_q(slot, j_c); });
+    issued_q();
+  };
+  auto slice_mfma = [&](auto cur_c) {
+    constexpr int cur = decltype(cur_c)::value;
+#pragma unroll
+    for (int q = 0; q < NQ; q++)
+#pragma unroll
+      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
+    constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
+#pragma unroll
+    for (int i = 0; i < NR; i++) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  };
+  auto slice_mfma_refill = [&](int p_slot, int q_slot) {
+    static_for<NM>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
+      static_for<LPS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        if constexpr (j * NM / LPS == i) {
+          if constexpr (j < PI) issue_p(p_slot, j_c);
+          else issue_q(q_slot, std::integral_constant<int, j - PI>{});
+        }
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    issued_p();
+    issued_q();
+  };
+  auto inner_slices = [&](int bp, int bq) {
+    static_for<SLICES - 1>([&](auto ks_c) {
+      constexpr int ks = decltype(ks_c)::value;
+      load(bp, bq, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
+      slice_mfma(std::integral_constant<int, (ks & 1)>{});
+    });
+  };
+
+  all_p(0);
+  all_q(0);
+  all_p(1);
+  all_q(1);
+  all_q(2);
+  wait_vmem_upto<PI + 2 * QI>();
+  lds_barrier();
+  load(0, 0, 0, qf[0], pf[0]);
+  int bp = 0, bq = 0;
+#ifdef SMOE_PROBE_PHASES
+  unsigned long long phase_[8] = {}, last_ = wall_clock64();
+#endif
+  // boundary behind a stage that is not the tile's last: read slice 0 of the next stage, refill the vacated slots
+  auto boundary = [&]() {
+    lds_barrier();
+    const int np = bp ^ 1, nq = bq == 2 ? 0 : bq + 1;
+    load(np, nq, 0, qf[0], pf[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    slice_mfma_refill(bp, bq);  // P(s+2), Q(s+3) into the slots stage s leaves behind
+    bp = np;
+    bq = nq;
+  };
+  for (;;) {
+    // stage 0: stores of the previous epilogue may still be outstanding, wait for everything
+    SMOE_PHASE_MARK(5)
+    inner_slices(bp, bq);
+#ifdef SMOE_PROBE_STREAM_COUNTED_WAIT
+    wait_vmem_upto<QI>();  // timing probe (unsafe: stores and loads may retire out of order)
+#else
+    wait_vmem_all();
+#endif
+    SMOE_PHASE_MARK(0)
+    first_boundary();
+    boundary();
+    for (int s = 1; s + 1 < S; s++) {
+      inner_slices(bp, bq);
+      wait_vmem_upto<QI>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
+      boundary();
+    }
+    // last stage: the stages of the next tile that are due are already requested; its own slots become scratch
+    SMOE_PHASE_MARK(1)
+    inner_slices(bp, bq);
+    wait_vmem_upto<QI>();
+    lds_barrier();
+    slice_mfma(std::integral_constant<int, 1>{});
+    SMOE_PHASE_MARK(2)
+    if (!tile_end(bp, bq)) break;
+    SMOE_PHASE_MARK(3)
+    wait_lds_all();
+    lds_barrier();  // every wave has read its parked rows back: the two slots may be refilled
+    all_p(bp);
+    all_q(bq);
+    bp ^= 1;
+    bq = bq == 2 ? 0 : bq + 1;
+    load(bp, bq, 0, qf[0], pf[0]);
+    SMOE_PHASE_MARK(4)
+  }
+#ifdef SMOE_PROBE_PHASES
+  if (threadIdx.x == 0)
+    for (int k = 0; k < 8; k++) atomicAdd(&smoe_phase_ticks[k], phase_[k]);
+#endif
+  wait_vmem_all();  // the streams ran ahead into ring slots nobody reads any more: let those loads land before the end
+}
+
 // ---- epilogue through LDS ----------------------------------------------------------------------------------------
 // A wavefront parks its TR x TC accumulator tile (lane = tile row l%32, register quad = 4 consecutive columns) as
 // bf16 in its own LDS region with padded rows, then reads it back row-contiguous and writes 16 bytes per lane.
@@ -328,7 +471,13 @@ SMOE_DEV void epilogue_flush(const char* region, int lane, uint16_t* out, int64_
     const int r = it * L::ROWS_PER_PASS + rr;
     const u32x4 v = *(const u32x4*)(region + r * L::ROW_BYTES + cc * 16);
     const int row = row_base + r, col = col_base + cc * 8;
+#ifdef SMOE_PROBE_EPI_NO_STORE
+    if (row < row_limit && col < col_limit && v[0] == 0x7fc12345u) *(u32x4*)(out + (int64_t)row * out_stride + col) = v;
+#elif defined(SMOE_PROBE_NT_STORE)
+    if (row < row_limit && col < col_limit) __builtin_nontemporal_store(v, (u32x4*)(out + (int64_t)row * out_stride + col));
+#else
     if (row < row_limit && col < col_limit) *(u32x4*)(out + (int64_t)row * out_stride + col) = v;
+#endif
   }
 }
 
@@ -462,6 +611,73 @@ SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int 
     epilogue_flush<TM, TN>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base, a.N);
     }
   }
+}
+
+// The same epilogue one 32-row fragment row at a time, parked in a caller-chosen LDS region of 32 padded rows
+// (32 * EpiLayout<TN>::ROW_BYTES bytes per wave): for kernels whose ring keeps running during the epilogue.
+template <int TN, int FM, int FN, bool WITH_ACT, int ACT>
+SMOE_DEV void forward_epilogue_rows(f32x16 (&acc)[FN][FM], char* region, int lane, const FwdEpilogueArgs& a) {
+  constexpr bool GLU = act_is_glu(ACT);
+  constexpr int PW = act_pointwise(ACT);
+  using LZ = EpiLayout<TN>;
+  using LY = EpiLayout<TN / 2>;
+  float bias[FN * 4][4];
+  const bool with_bias = a.bias != nullptr;
+  if (with_bias) {
+    static_for<FN * 4>([&](auto q_c) {
+      constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+      int n = a.n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
+      n = n <= a.N - 4 ? n : a.N - 4;
+      const u32x2 b = *(const u32x2*)(a.bias + n);
+      bias[fn * 4 + rg][0] = bf16_lo(b[0]);
+      bias[fn * 4 + rg][1] = bf16_hi(b[0]);
+      bias[fn * 4 + rg][2] = bf16_lo(b[1]);
+      bias[fn * 4 + rg][3] = bf16_hi(b[1]);
+    });
+  }
+  const int mrow = lane & 31, half = lane >> 5;
+  static_for<FM>([&](auto fm_c) {
+    constexpr int fm = decltype(fm_c)::value;
+    if (with_bias) {
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+#pragma unroll
+        for (int q = 0; q < 4; q++) acc[fn][fm][4 * rg + q] += bias[fn * 4 + rg][q];
+      });
+    }
+    const int m0 = a.m_base + fm * 32;
+    if (!WITH_ACT || a.out0 != nullptr) {
+      static_for<FN * 4>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+        u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
+                   pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
+        *(u32x2*)(region + mrow * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * half) * 2) = v;
+      });
+      epilogue_flush<32, TN>(region, lane, a.out0, a.out0_stride, m0, a.row_end, a.n_base, a.N);
+    }
+    if constexpr (WITH_ACT && GLU) {
+      if (a.out1 != nullptr) {
+        static_for<FN * 4>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+          const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
+          const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
+          const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
+          *(uint32_t*)(region + mrow * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * half) * 2) = v;
+        });
+        epilogue_flush<32, TN / 2>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base / 2, a.N / 2);
+      }
+    } else if constexpr (WITH_ACT) {
+      if (a.out1 != nullptr) {
+        static_for<FN * 4>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+          u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
+                     pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
+          *(u32x2*)(region + mrow * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * half) * 2) = v;
+        });
+        epilogue_flush<32, TN>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base, a.N);
+      }
+    }
+  });
 }
 
 // ---- launch helper -------------------------------------------------------------------------------------------------

@@ -320,6 +320,245 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   }
 }
 
+// ---- the same GEMM as a stream of tiles per workgroup -----------------------------------------------------------------
+// One workgroup per compute unit walks through the tiles b, b + gridDim.x, ... of the XCD-aware tile order and keeps
+// the ring running across tile boundaries (gemm_stream_loop).  ROLE_UP_FWD and ROLE_PLAIN only; needs Kdim >= 3 * BK.
+template <class C, int ROLE, int ACT>
+__global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMParams p) {
+  static_assert(ROLE == ROLE_UP_FWD || ROLE == ROLE_PLAIN, "the dz epilogue is not built as a stream");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, SLICES = C::BK / 16;
+  const uint32_t smem_base = lds_address(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % C::WM, wn = wave / C::WM;
+
+  // tile bookkeeping is read through the constant address space: uniform addresses then become scalar loads, which do
+  // not touch the vector-memory counter the ring is timed with
+  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+  const const_i32_ptr tm_header = (const_i32_ptr)p.tm.header, tm_expert = (const_i32_ptr)p.tm.expert,
+                      tm_row0 = (const_i32_ptr)p.tm.row0, off = (const_i32_ptr)p.off;
+  const int num_m_tiles = tm_header[0];
+  const int64_t total = (int64_t)num_m_tiles * p.n_tiles;
+  const int64_t per_xcd = (total + 7) >> 3;
+  struct Tile {
+    int e, row0, row_end, n0;
+    bool valid;
+  };
+  // tile of virtual workgroup vb (the XCD-aware order of the one-tile-per-workgroup kernel)
+  auto tile_at = [&](int64_t vb) {
+    Tile t = {0, 0, 1, 0, false};
+    const int64_t slot = vb >> 3;
+    const int64_t lin = (vb & 7) * per_xcd + slot;
+    if (slot < per_xcd && lin < total) {
+      constexpr int GM = 8;
+      const int64_t per_group = (int64_t)GM * p.n_tiles;
+      const int group = (int)(lin / per_group);
+      const int first_m = group * GM;
+      const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
+      const int within = (int)(lin - (int64_t)group * per_group);
+      const int mt = first_m + within % gm;
+      t.e = tm_expert[mt];
+      t.row0 = tm_row0[mt];
+      t.row_end = off[t.e + 1];
+      t.n0 = (within / gm) * BN;
+      t.valid = true;
+    }
+    return t;
+  };
+  int64_t vb = blockIdx.x;
+  Tile cur = tile_at(vb);
+  if (!cur.valid) return;
+#ifdef SMOE_PROBE_STAGGER
+  // timing probe: tiles take the same time on every compute unit, so all epilogues fall together and share the
+  // chip's store bandwidth; start the workgroups in 8 groups a few microseconds apart
+  for (int i = 0; i < (int)((blockIdx.x >> 3) & 7) * SMOE_PROBE_STAGGER; i++) __builtin_amdgcn_s_sleep(32);
+#endif
+  Tile nxt = tile_at(vb += gridDim.x);
+  bool more = nxt.valid;  // a tile follows the current one
+  if (!more) nxt = cur;   // the streams always run on: past the last tile they re-read it into slots nobody reads
+  Tile nn = tile_at(vb += gridDim.x);
+
+  // ---- global source addresses ----
+  // Everything a tile switch computes from the lane number starts from a copy of it the compiler cannot see through:
+  // otherwise the per-lane parts are hoisted out of the tile loop and occupy registers the main loop needs.
+  auto opaque_lane = [&]() {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
+  // source rows of a tile's token operand (ordinary vector loads when gathered)
+  auto token_rows = [&](const Tile& t, int(&rows)[C::P_INSTR]) {
+    const int ln = opaque_lane();
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) {
+      int m = t.row0 + (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
+      m = m < t.row_end ? m : t.row_end - 1;
+      rows[i] = p.gidx ? p.gidx[m] : m;
+    }
+  };
+  const uint16_t* p_src[C::P_INSTR];
+  const uint16_t* q_src[C::Q_INSTR];
+  const int64_t q_step = C::QMN ? (int64_t)BK * p.q_stride_row : (int64_t)BK;
+  auto point_p = [&](const int(&rows)[C::P_INSTR]) {
+    const int ln = opaque_lane();
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) {
+      const int r = (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
+      p_src[i] = p.P + (int64_t)rows[i] * p.p_stride + (((ln % C::KPR) ^ kswz<BK>(r)) << 3);
+    }
+  };
+  auto point_q = [&](const Tile& t) {
+    const int ln = opaque_lane();
+    const uint16_t* qe = p.Q + (int64_t)t.e * p.q_stride_e;
+#pragma unroll
+    for (int i = 0; i < C::Q_INSTR; i++) {
+      if constexpr (!C::QMN) {
+        const int r = (wave * C::Q_INSTR + i) * C::KRPI + ln / C::KPR;
+        int n = t.n0 + r;
+        n = n < p.N ? n : p.N - 1;
+        q_src[i] = qe + (int64_t)n * p.q_stride_row + (((ln % C::KPR) ^ kswz<BK>(r)) << 3);
+      } else {
+        const int kl = (wave * C::Q_INSTR + i) * C::RPI + ln / C::LPR;
+        const int phys16 = ln % C::LPR;
+        const int log32 = (phys16 >> 1) ^ mnswz(kl);
+        int n = t.n0 + ((log32 << 1) | (phys16 & 1)) * 8;
+        n = n <= p.N - 8 ? n : p.N - 8;
+        q_src[i] = qe + (int64_t)kl * p.q_stride_row + n;
+      }
+    }
+  };
+  int rows_next[C::P_INSTR];  // token rows of nxt: loaded at the start of a tile, picked up behind its first stage
+  {
+    int rows_cur[C::P_INSTR];
+    token_rows(cur, rows_cur);
+    point_p(rows_cur);
+    point_q(cur);
+    token_rows(nxt, rows_next);
+  }
+
+  const int S_total = p.Kdim / BK;
+
+  // ---- per-lane LDS fragment offsets (bytes inside a stage) ----
+  int p_off[SLICES];
+  {
+    const int row = wm * C::TM + (lane & 31);
+    const int sw = kswz<BK>(row);
+#pragma unroll
+    for (int ks = 0; ks < SLICES; ks++) p_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+  }
+  int q_off[C::QMN ? 2 * FN : SLICES];
+  if constexpr (!C::QMN) {
+    const int row = wn * C::TN + (lane & 31);
+    const int sw = kswz<BK>(row);
+#pragma unroll
+    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+  } else {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int kk = 8 * (grp >> 1) + (i16 >> 2);
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+      const int c32 = (wn * C::TN) / 16 + fn * 2 + (grp & 1);
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int k = kk + 4 * h;
+        q_off[fn * 2 + h] = k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+      }
+    }
+  }
+
+  f32x16 acc[FN][FM];
+  auto clear_acc = [&]() {
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++)
+#pragma unroll
+      for (int fm = 0; fm < FM; fm++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
+  };
+  clear_acc();
+
+  constexpr int Q_RING = C::P_SLOTS * C::P_STAGE;
+  int p_stage = 0, q_stage = 0;  // stages issued to each stream for the tile it is on
+  auto issue_p = [&](int slot, auto i_c) {
+    constexpr int i = decltype(i_c)::value;
+    load16_to_lds(p_src[i], smem_base + slot * C::P_STAGE + (wave * C::P_INSTR + i) * 1024);
+    p_src[i] += BK;
+  };
+  auto issue_q = [&](int slot, auto j_c) {
+    constexpr int j = decltype(j_c)::value;
+    load16_to_lds(q_src[j], smem_base + Q_RING + slot * C::Q_STAGE + (wave * C::Q_INSTR + j) * 1024);
+    q_src[j] += q_step;
+  };
+  auto issued_p = [&]() {
+    if (++p_stage == S_total) {
+      p_stage = 0;
+      point_p(rows_next);
+    }
+  };
+  auto issued_q = [&]() {
+    if (++q_stage == S_total) {
+      q_stage = 0;
+      point_q(nxt);
+    }
+  };
+  auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
+    const char* sp = smem + p_slot * C::P_STAGE;
+    const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
+#pragma unroll
+    for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(sp + p_off[ks] + fm * 32 * C::KROW);
+#pragma unroll
+    for (int fn = 0; fn < FN; fn++) {
+      if constexpr (!C::QMN) {
+        qf[fn] = lds_read_b128(sq + q_off[ks] + fn * 32 * C::KROW);
+      } else {
+        qf[fn] = lds_read_tr2(sq + q_off[fn * 2] + ks * 16 * C::ROWB, sq + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
+      }
+    }
+  };
+  // the rows loaded in tile_end are complete here; naming them in an asm statement makes this the place where the
+  // compiler waits for them
+  auto first_boundary = [&]() {
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) asm volatile("" : "+v"(rows_next[i]));
+  };
+  constexpr int PARK = 32 * EpiLayout<C::TN>::ROW_BYTES;  // one wave's parked fragment row
+  static_assert((C::NW / 2) * PARK <= C::P_STAGE && (C::NW / 2) * PARK <= C::Q_STAGE, "parking must fit into a ring slot");
+  auto tile_end = [&](int p_slot, int q_slot) {
+    FwdEpilogueArgs ea;
+    ea.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
+    ea.out0 = p.out0;
+    ea.out0_stride = p.out0_stride;
+    ea.out1 = p.out1;
+    ea.out1_stride = p.out1_stride;
+    ea.m_base = cur.row0 + wm * C::TM;
+    ea.row_end = cur.row_end;
+    ea.n_base = cur.n0 + wn * C::TN;
+    ea.N = p.N;
+    // waves 0..NW/2-1 park in the vacated P slot, the others in the vacated Q slot
+    char* region = wave < C::NW / 2 ? smem + p_slot * C::P_STAGE + wave * PARK
+                                    : smem + Q_RING + q_slot * C::Q_STAGE + (wave - C::NW / 2) * PARK;
+#ifdef SMOE_PROBE_PHASES
+    const unsigned long long t0_ = wall_clock64();
+#endif
+    forward_epilogue_rows<C::TN, FM, FN, ROLE == ROLE_UP_FWD, ACT>(acc, region, opaque_lane(), ea);
+#ifdef SMOE_PROBE_PHASES
+    if (threadIdx.x == 0) atomicAdd(&smoe_phase_ticks[6], wall_clock64() - t0_);
+#endif
+    if (!more) return false;
+    clear_acc();
+    cur = nxt;
+    nxt = nn;
+    more = nxt.valid;
+    if (!more) nxt = cur;
+    nn = tile_at(vb += gridDim.x);
+    token_rows(nxt, rows_next);
+    return true;
+  };
+  gemm_stream_loop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR, C::Q_INSTR, SLICES>(
+      S_total, acc, issue_p, issue_q, load, issued_p, issued_q, first_boundary, tile_end);
+}
+
 template <class C, int ROLE, int ACT>
 static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
   static LdsLimitOnce lds_limit;
@@ -336,6 +575,28 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
+  if constexpr (ROLE != ROLE_DZ) {
+    // SMOE_GEMM_STREAM=0 (environment, read once) keeps the one-tile-per-workgroup kernel
+    static const bool stream = !(getenv("SMOE_GEMM_STREAM") && atoi(getenv("SMOE_GEMM_STREAM")) == 0);
+    if (stream && p.Kdim >= 3 * C::BK) {
+      static LdsLimitOnce lds_limit_stream;
+      auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
+      const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
+      if (rc_s) return rc_s;
+      int dev = 0, cus = 0;
+      SMOE_HIP_CHECK(hipGetDevice(&dev));
+      SMOE_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+      int64_t sgrid = ((int64_t)cus / 8) * 8;  // one resident workgroup per compute unit, the same number on every XCD
+      // SMOE_GEMM_STREAM_GRID (environment, read at every launch) overrides the number of workgroups: small values
+      // make small problems run several tiles per workgroup (used by the tests)
+      if (const char* g = getenv("SMOE_GEMM_STREAM_GRID")) sgrid = ((int64_t)atoi(g) + 7) / 8 * 8;
+      if (sgrid < 8) sgrid = 8;
+      if (sgrid > grid) sgrid = grid;
+      hipLaunchKernelGGL(skern, dim3((unsigned)sgrid), dim3(C::NT), C::SMEM, st, p);
+      SMOE_LAUNCH_CHECK();
+      return SMOE_OK;
+    }
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
@@ -491,3 +752,13 @@ int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_st
 }
 
 }  // namespace smoe
+
+#ifdef SMOE_PROBE_PHASES
+// timing probe: read and clear the phase counters of the tile-stream kernels
+extern "C" int smoe_probe_phases(unsigned long long* out) {
+  unsigned long long zero[8] = {};
+  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(smoe::smoe_phase_ticks), sizeof(zero)) != hipSuccess) return -1;
+  if (hipMemcpyToSymbol(HIP_SYMBOL(smoe::smoe_phase_ticks), zero, sizeof(zero)) != hipSuccess) return -1;
+  return 0;
+}
+#endif

@@ -116,6 +116,56 @@ def test_backward_ops(dev, T, H, I, E, K, skew, empty):
     assert rel_l2(dx, dx_ref) < TOL
 
 
+STREAM_SHAPES = [
+    # contraction lengths 192 = 3 stages (the shortest a tile stream takes), 256, 384, 768; ragged tails; empty experts
+    (1500, 192, 192, 16, 4, 1.2, (3, 15)),
+    (2048, 256, 128, 4, 2, 0.0, ()),
+    (4096, 768, 192, 8, 4, 0.8, (0,)),
+]
+
+
+@pytest.mark.parametrize("grid", [8, 24])
+@pytest.mark.parametrize("T,H,I,E,K,skew,empty", STREAM_SHAPES)
+def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
+    """The grouped GEMMs whose workgroups walk through several tiles each: few workgroups (8 = one per XCD, 24) force
+    long streams on small problems, so tile switches, the parked epilogue and the last tile of a stream are all hit."""
+    monkeypatch.setenv("SMOE_GEMM_STREAM_GRID", str(grid))
+    fwd, bwd = _ops()
+    _, w1, w2 = make_weights(E, H, I, dev, seed=T + 20)
+    b1 = (torch.randn(E, 2 * I, generator=torch.Generator().manual_seed(T + 23)) * 0.5).to(torch.bfloat16).to(dev)
+    idx, scores, meta, md = make_tc_routing(T, E, K, dev, seed=T + 21, skew=skew, empty=empty)
+    g = torch.Generator().manual_seed(T + 22)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    TK = T * K
+    off, gidx, sidx = (md[k] for k in ("expert_frequency_offset", "x_gather_idx", "s_scatter_idx"))
+    stream = torch.cuda.current_stream().cuda_stream
+
+    for bias in (None, b1):
+        z = torch.empty(TK, 2 * I, dtype=torch.bfloat16, device=dev)
+        y1 = torch.empty(TK, I, dtype=torch.bfloat16, device=dev)
+        fwd._up_projection_forward(x, w1.permute(1, 2, 0), z, y1, bias, off, None, gidx, stream, "swiglu", True, False)
+        z_ref, y1_ref = M.up_projection_forward(x, w1, off, gidx, b1=bias)
+        assert rel_l2(z, z_ref) < TOL
+        assert rel_l2(y1, y1_ref) < TOL
+
+    y2 = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
+    fwd._down_projection_forward(w2.permute(1, 2, 0), y1, y2, None, off, None, gidx, stream)
+    assert rel_l2(y2, M.down_projection_forward(y1, w2, off)) < TOL
+
+    dz = torch.randn(TK, 2 * I, generator=g).to(torch.bfloat16).to(dev)
+    dxe = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
+    bwd._up_projection_backward(x, w1.permute(1, 2, 0), dxe, None, dz, None, off, None, gidx, sidx, True, stream)
+    _, dxe_ref = M.up_projection_backward(x, w1, dz, off, gidx)
+    assert rel_l2(dxe, dxe_ref) < TOL
+
+    # the same results from the one-tile-per-workgroup launch order (many workgroups, one tile each)
+    monkeypatch.setenv("SMOE_GEMM_STREAM_GRID", "1000000")
+    z1 = torch.empty_like(z)
+    y11 = torch.empty_like(y1)
+    fwd._up_projection_forward(x, w1.permute(1, 2, 0), z1, y11, b1, off, None, gidx, stream, "swiglu", True, False)
+    assert torch.equal(z1, z) and torch.equal(y11, y1)
+
+
 def test_unsupported_arguments_raise(dev):
     fwd, _ = _ops()
     T, H, I, E, K = 64, 96, 64, 4, 2  # H not a multiple of 64
