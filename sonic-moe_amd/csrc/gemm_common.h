@@ -460,24 +460,29 @@ struct EpiLayout {
   static constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
 };
 
-// store rows [0, TR) of the parked tile: global row = row_base + r (valid below row_limit), col = col_base + c
+// store rows [0, TR) of the parked tile: global row = row_base + r (valid below row_limit), col = col_base + c.
+// The LDS reads of a batch are issued together ahead of its stores: one LDS round trip per batch, not per store.
 template <int TR, int TC>
 SMOE_DEV void epilogue_flush(const char* region, int lane, uint16_t* out, int64_t out_stride, int row_base,
                              int row_limit, int col_base, int col_limit) {
   using L = EpiLayout<TC>;
+  constexpr int NIT = TR / L::ROWS_PER_PASS, BATCH = NIT < 8 ? NIT : 8;
+  static_assert(NIT % BATCH == 0, "passes come in whole batches");
   const int rr = lane / L::LANES_PER_ROW, cc = lane % L::LANES_PER_ROW;
+  const int col = col_base + cc * 8;
+  uint16_t* dst = out + (int64_t)(row_base + rr) * out_stride + col;
 #pragma unroll
-  for (int it = 0; it < TR / L::ROWS_PER_PASS; it++) {
-    const int r = it * L::ROWS_PER_PASS + rr;
-    const u32x4 v = *(const u32x4*)(region + r * L::ROW_BYTES + cc * 16);
-    const int row = row_base + r, col = col_base + cc * 8;
-#ifdef SMOE_PROBE_EPI_NO_STORE
-    if (row < row_limit && col < col_limit && v[0] == 0x7fc12345u) *(u32x4*)(out + (int64_t)row * out_stride + col) = v;
-#elif defined(SMOE_PROBE_NT_STORE)
-    if (row < row_limit && col < col_limit) __builtin_nontemporal_store(v, (u32x4*)(out + (int64_t)row * out_stride + col));
-#else
-    if (row < row_limit && col < col_limit) *(u32x4*)(out + (int64_t)row * out_stride + col) = v;
-#endif
+  for (int b0 = 0; b0 < NIT; b0 += BATCH) {
+    u32x4 v[BATCH];
+#pragma unroll
+    for (int j = 0; j < BATCH; j++)
+      v[j] = *(const u32x4*)(region + ((b0 + j) * L::ROWS_PER_PASS + rr) * L::ROW_BYTES + cc * 16);
+#pragma unroll
+    for (int j = 0; j < BATCH; j++) {
+      const int r = (b0 + j) * L::ROWS_PER_PASS + rr;
+      if (row_base + r < row_limit && col < col_limit)
+        *(u32x4*)(dst + (int64_t)((b0 + j) * L::ROWS_PER_PASS) * out_stride) = v[j];
+    }
   }
 }
 
