@@ -368,10 +368,12 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
       acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
       static_for<LPS>([&](auto j_c) {
         constexpr int j = decltype(j_c)::value;
+#ifndef SMOE_PROBE_NO_REFILL
         if constexpr (j * NM / LPS == i) {
           if constexpr (j < PI) issue_p(p_slot, j_c);
           else issue_q(q_slot, std::integral_constant<int, j - PI>{});
         }
+#endif
       });
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -412,11 +414,7 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
     // stage 0: stores of the previous epilogue may still be outstanding, wait for everything
     SMOE_PHASE_MARK(5)
     inner_slices(bp, bq);
-#ifdef SMOE_PROBE_STREAM_COUNTED_WAIT
-    wait_vmem_upto<QI>();  // timing probe (unsafe: stores and loads may retire out of order)
-#else
     wait_vmem_all();
-#endif
     SMOE_PHASE_MARK(0)
     first_boundary();
     boundary();

@@ -346,7 +346,7 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     p.S = (const uint16_t*)x;
     p.s_stride = H;
     p.gidx = x_gather_idx;
-    p.off = off;
+      p.off = off;
     p.out = (uint16_t*)dw1;
     p.out_stride_e = dw1_stride_e;
     p.out_stride_row = dw1_stride_row;

@@ -197,9 +197,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
                                                                                           load);
 
   const int m_base = row0 + wm * C::TM, n_base = n0 + wn * C::TN;
-#ifdef SMOE_PROBE_NO_EPILOGUE
-  if (acc[0][0][0] != 12345.f) return;
-#endif
 
   if constexpr (ROLE == ROLE_PLAIN || ROLE == ROLE_UP_FWD) {
     FwdEpilogueArgs ea;
@@ -369,11 +366,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
   int64_t vb = blockIdx.x;
   Tile cur = tile_at(vb);
   if (!cur.valid) return;
-#ifdef SMOE_PROBE_STAGGER
-  // timing probe: tiles take the same time on every compute unit, so all epilogues fall together and share the
-  // chip's store bandwidth; start the workgroups in 8 groups a few microseconds apart
-  for (int i = 0; i < (int)((blockIdx.x >> 3) & 7) * SMOE_PROBE_STAGGER; i++) __builtin_amdgcn_s_sleep(32);
-#endif
   Tile nxt = tile_at(vb += gridDim.x);
   bool more = nxt.valid;  // a tile follows the current one
   if (!more) nxt = cur;   // the streams always run on: past the last tile they re-read it into slots nobody reads
@@ -503,6 +495,9 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     }
   };
   auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
+#ifdef SMOE_PROBE_NO_LDSREAD
+    return;
+#endif
     const char* sp = smem + p_slot * C::P_STAGE;
     const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
 #pragma unroll
@@ -602,15 +597,10 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   return SMOE_OK;
 }
 
-// 256 x 256 tile, 8 wavefronts as 2 (token) x 4 (feature), 64 of the contraction per stage, double buffer
-#ifdef SMOE_PROBE_TILE_256x128x3
-// timing probe: a 256 x 128 tile leaves room for a third 64-deep stage (two in flight)
-template <bool QMN>
-using TileCfg = Cfg<256, 128, 2, 4, QMN, 64, 3>;
-#else
+// 256 x 256 tile, 8 wavefronts as 2 (token) x 4 (feature), 64 of the contraction per stage; the ring is 2 token-operand
+// slots + 3 weight-operand slots (the last template argument is not used by these kernels)
 template <bool QMN>
 using TileCfg = Cfg<256, 256, 2, 4, QMN, 64, 2>;
-#endif
 
 // one kernel per activation: the epilogue math and (gated or not) the tile geometry of z / y1 depend on it
 template <bool QMN, int ROLE>

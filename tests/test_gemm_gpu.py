@@ -154,9 +154,26 @@ def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
 
     dz = torch.randn(TK, 2 * I, generator=g).to(torch.bfloat16).to(dev)
     dxe = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
-    bwd._up_projection_backward(x, w1.permute(1, 2, 0), dxe, None, dz, None, off, None, gidx, sidx, True, stream)
-    _, dxe_ref = M.up_projection_backward(x, w1, dz, off, gidx)
+    dw1 = torch.full((E, 2 * I, H), 3.0, dtype=torch.bfloat16, device=dev).permute(1, 2, 0)
+    bwd._up_projection_backward(x, w1.permute(1, 2, 0), dxe, dw1, dz, None, off, None, gidx, sidx, True, stream)
+    dw1_ref, dxe_ref = M.up_projection_backward(x, w1, dz, off, gidx)
     assert rel_l2(dxe, dxe_ref) < TOL
+    assert rel_l2(dw1.permute(2, 0, 1), dw1_ref) < TOL
+    for e in empty:
+        assert bool((dw1[..., e] == 0).all()), "experts without tokens get zero weight gradients"
+
+    dout = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    s_flat = torch.from_numpy(scores).to(dev).view(-1)
+    zb = z_ref.to(torch.bfloat16)
+    dw2 = torch.full((E, H, I), 3.0, dtype=torch.bfloat16, device=dev).permute(1, 2, 0)
+    dz2 = torch.empty(TK, 2 * I, dtype=torch.bfloat16, device=dev)
+    ds = torch.empty(TK, dtype=torch.float32, device=dev)
+    bwd._down_projection_backward(dout, zb, w2.permute(1, 2, 0), dw2, dz2, ds, None, None, s_flat, off, None, gidx, sidx,
+                                  stream, True, "swiglu")
+    _, _, _, dw2_ref = M.down_projection_backward(dout, zb, w2, s_flat, off, gidx, sidx, round_dtype=torch.bfloat16)
+    assert rel_l2(dw2.permute(2, 0, 1), dw2_ref) < TOL
+    for e in empty:
+        assert bool((dw2[..., e] == 0).all())
 
     # the same results from the one-tile-per-workgroup launch order (many workgroups, one tile each)
     monkeypatch.setenv("SMOE_GEMM_STREAM_GRID", "1000000")
