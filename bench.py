@@ -159,11 +159,11 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
 
 # operators that are one grouped-GEMM kernel launch (plus a ~5 us tile-map builder), and the kernel they launch
 SINGLE_KERNEL_OPS = {
-    "up_projection_forward": "varlen_m_kernel<up-projection forward>",
-    "down_projection_forward": "varlen_m_kernel<down-projection forward>",
+    "up_projection_forward": "varlen_m_stream_kernel<up-projection forward>",
+    "down_projection_forward": "varlen_m_stream_kernel<down-projection forward>",
     "down_projection_backward(dz only)": "varlen_m_kernel<dz>",
     "up_projection_backward(dW1 only)": "varlen_k_kernel<dW1>",
-    "up_projection_backward(dx only)": "varlen_m_kernel<dx_expanded>",
+    "up_projection_backward(dx only)": "varlen_m_stream_kernel<dx_expanded>",
 }
 
 

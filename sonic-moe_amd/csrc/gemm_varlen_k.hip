@@ -24,7 +24,7 @@ struct VarlenKParams {
   int NA, NB;  // output rows / cols
   int tiles_a, tiles_b;
   int E;
-  int xcd_chunked;  // 1: contiguous tile range per XCD (probe), 0: round-robin
+  int xcd_chunked;  // tile order: 2 blocked, 1 contiguous tile range per XCD (probe: unbalanced on skewed experts), 0 round-robin
 };
 
 template <int BA_, int BB_, int WA_, int WB_, bool R_GATHER_, bool S_GATHER_, int BK_, int NSTAGE_>
@@ -54,15 +54,34 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave % C::WA, wb = wave / C::WA;
 
-  // Tiles of one expert are dealt round-robin over the XCDs (workgroup b runs on XCD b % 8): an expert's cost is its
-  // token count, so giving every XCD a slice of every expert balances skewed loads, and the tiles an XCD gets from one
-  // expert (every 8th) still share their S-operand columns in its L2.
+  // Tile order.  Workgroup b runs on XCD b % 8 and every XCD runs 32 workgroups side by side.  An expert's cost is its
+  // token count, so every expert is spread over several XCDs (skewed loads stay balanced), in blocks that share operand
+  // panels in the XCD's L2 (see the blocked order below); order 0 deals single tiles round-robin instead.
   const int64_t per_e = (int64_t)p.tiles_a * p.tiles_b;
-  const int64_t lin = p.xcd_chunked ? xcd_linear_tile(per_e * p.E) : (blockIdx.x < per_e * p.E ? (int64_t)blockIdx.x : -1);
-  if (lin < 0) return;
-  const int e = (int)(lin / per_e);
-  const int within = (int)(lin - (int64_t)e * per_e);
-  const int ta = within / p.tiles_b, tb = within % p.tiles_b;
+  int e, ta, tb;
+  if (p.xcd_chunked == 2) {
+    // Blocked order: the 32 tiles an XCD runs side by side are one ba x bb block of ONE expert's output (8 blocks of
+    // 32 consecutive workgroup slots per round of 256 workgroups), so per stage they fetch ba + bb operand panels
+    // instead of one or two panels each.  Block B runs on XCD (B + B/8) % 8: an expert's blocks go to neighbouring
+    // XCDs, and the rotation keeps any XCD from always getting the same experts.
+    const int bb = p.tiles_b < 8 ? p.tiles_b : 8, ba = 32 / bb;
+    const int nbj = p.tiles_b / bb, nb = (p.tiles_a / ba) * nbj;  // blocks per expert
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int seq = j >> 5, in = j & 31;
+    const int64_t B = (int64_t)seq * 8 + ((xcd + 8 - (seq & 7)) & 7);
+    if (B >= (int64_t)nb * p.E) return;
+    e = (int)(B / nb);
+    const int blk = (int)(B - (int64_t)e * nb);
+    ta = (blk / nbj) * ba + in / bb;
+    tb = (blk % nbj) * bb + in % bb;
+  } else {
+    const int64_t lin = p.xcd_chunked ? xcd_linear_tile(per_e * p.E) : (blockIdx.x < per_e * p.E ? (int64_t)blockIdx.x : -1);
+    if (lin < 0) return;
+    e = (int)(lin / per_e);
+    const int within = (int)(lin - (int64_t)e * per_e);
+    ta = within / p.tiles_b;
+    tb = within % p.tiles_b;
+  }
   const int a0 = ta * C::BA, b0 = tb * C::BB;
   const int row_begin = p.off[e], row_end = p.off[e + 1];
   const int cnt = row_end - row_begin;
@@ -167,6 +186,9 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       if (s + 1 < S) fetch(s + 1);  // stages are issued in order: have the next one's rows ready
   };
   auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
+#ifdef SMOE_PROBE_NO_LDSREAD
+    return;
+#endif
     const char* st = smem + buf * C::STAGE;
 #pragma unroll
     for (int f = 0; f < FA; f++)
@@ -210,11 +232,21 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   p.tiles_a = (int)ceil_div(p.NA, C::BA);
   p.tiles_b = (int)ceil_div(p.NB, C::BB);
   {
-    static const int chunked = getenv("SMOE_VARLEN_K_XCD_CHUNKED") ? atoi(getenv("SMOE_VARLEN_K_XCD_CHUNKED")) : 0;
-    p.xcd_chunked = chunked;
+    // SMOE_VARLEN_K_TILE_ORDER (environment, read once): 2 = blocked (default), 0 = round-robin, 1 = whole experts per XCD
+    static const int order = getenv("SMOE_VARLEN_K_TILE_ORDER") ? atoi(getenv("SMOE_VARLEN_K_TILE_ORDER")) : 2;
+    p.xcd_chunked = order;
   }
   const int64_t total = (int64_t)p.tiles_a * p.tiles_b * p.E;
-  const int64_t grid = ((total + 7) / 8) * 8;
+  int64_t grid = ((total + 7) / 8) * 8;
+  if (p.xcd_chunked == 2) {
+    const int bb = p.tiles_b < 8 ? p.tiles_b : 8, ba = 32 / bb;
+    if (32 % bb == 0 && p.tiles_b % bb == 0 && p.tiles_a % ba == 0) {
+      const int64_t blocks = total / 32;
+      grid = ((blocks + 7) / 8) * 256;
+    } else {
+      p.xcd_chunked = 0;  // the output does not split into whole blocks
+    }
+  }
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "weight-grad gemm: too many tiles");
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
   SMOE_LAUNCH_CHECK();
