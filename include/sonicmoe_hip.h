@@ -156,6 +156,14 @@ int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride
                                 int64_t TK, int H, int I, int E, int activation, void* workspace,
                                 size_t workspace_bytes, void* stream);
 
+/* Weight gradient of the router's linear layer, dWr = dlogits^T x, split over the tokens: partial[c] (E, H) bf16 is the
+ * product over tokens [c * ceil(T / chunks), ...) and the caller sums the `chunks` partials.  The reference leaves this
+ * GEMM to torch (router_logits = F.linear(x, router_w), sonicmoe/functional/__init__.py:438); with E rows of output and
+ * T = tens of thousands of contraction elements a library GEMM without a split fills an eighth of the chip.
+ * dlogits (T, E) and x (T, H) contiguous bf16; E and H multiples of 8. */
+int smoe_router_weight_grad(const void* dlogits, const void* x, void* partial, int64_t T, int E, int H, int chunks,
+                            void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------
  * Token-rounding router (benchmarks/moe-token-rounding.py:139-191 of the reference, there a chain of torch ops
  * with a dense (T, E) argsort).  Chain: smoe_tr_softmax -> smoe_topk_softmax_fwd(probs, softmax = 0) ->

@@ -24,6 +24,8 @@ struct VarlenKParams {
   int NA, NB;  // output rows / cols
   int tiles_a, tiles_b;
   int E;
+  int uniform_rows;  // off == nullptr: group e is rows [e * uniform_rows, min((e + 1) * uniform_rows, total_rows))
+  int64_t total_rows;
   int xcd_chunked;  // tile order: 2 blocked, 1 contiguous tile range per XCD (probe: unbalanced on skewed experts), 0 round-robin
 };
 
@@ -83,7 +85,15 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     tb = within % p.tiles_b;
   }
   const int a0 = ta * C::BA, b0 = tb * C::BB;
-  const int row_begin = p.off[e], row_end = p.off[e + 1];
+  int row_begin, row_end;
+  if (p.off != nullptr) {
+    row_begin = p.off[e];
+    row_end = p.off[e + 1];
+  } else {
+    row_begin = e * p.uniform_rows;
+    const int64_t end = (int64_t)(e + 1) * p.uniform_rows;
+    row_end = (int)(end < p.total_rows ? end : p.total_rows);
+  }
   const int cnt = row_end - row_begin;
   const int S = (cnt + BK - 1) / BK;
 
@@ -393,4 +403,29 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     if (rc) return rc;
   }
   return SMOE_OK;
+}
+
+extern "C" int smoe_router_weight_grad(const void* dlogits, const void* x, void* partial, int64_t T, int E, int H,
+                                       int chunks, void* stream) {
+  SMOE_REQUIRE(T > 0 && T < (1ll << 31), SMOE_ERR_INVALID, "router_weight_grad: T out of range");
+  SMOE_REQUIRE(E >= 8 && E % 8 == 0, SMOE_ERR_UNSUPPORTED, "router_weight_grad: E=%d must be a multiple of 8", E);
+  SMOE_REQUIRE(H >= 8 && H % 8 == 0, SMOE_ERR_UNSUPPORTED, "router_weight_grad: H=%d must be a multiple of 8", H);
+  SMOE_REQUIRE(chunks >= 1, SMOE_ERR_INVALID, "router_weight_grad: chunks must be positive");
+  SMOE_REQUIRE(dlogits && x && partial, SMOE_ERR_INVALID, "router_weight_grad: null pointer");
+  VarlenKParams p = {};
+  p.R = (const uint16_t*)dlogits;
+  p.r_stride = E;
+  p.S = (const uint16_t*)x;
+  p.s_stride = H;
+  p.gidx = nullptr;
+  p.off = nullptr;
+  p.uniform_rows = (int)((T + chunks - 1) / chunks);
+  p.total_rows = T;
+  p.out = (uint16_t*)partial;
+  p.out_stride_e = (int64_t)E * H;
+  p.out_stride_row = H;
+  p.NA = E;
+  p.NB = H;
+  p.E = chunks;
+  return launch_varlen_k_variant<false, false>(p, (hipStream_t)stream);
 }

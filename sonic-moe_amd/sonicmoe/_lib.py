@@ -40,6 +40,7 @@ _SIGNATURES = {
         c_int,
         [_P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
+    "smoe_router_weight_grad": (c_int, [_P, _P, _P, _L, _I, _I, _I, _P]),
     "smoe_tr_softmax": (c_int, [_P, _I, _L, _I, _L, _P, _P]),
     "smoe_tr_rank": (c_int, [_P, _P, _I, _P, _P, _L, _I, _I, _P]),
     "smoe_tr_select": (c_int, [_P, _I, _P, _P, _L, _I, _P]),

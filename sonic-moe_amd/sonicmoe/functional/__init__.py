@@ -10,13 +10,22 @@ inside the weight-gradient kernels.
 
 from __future__ import annotations
 
+import os
+
 import torch
 import torch.nn.functional as F
 
 from .. import _lib
 from ..count_cumsum import count_cumsum
 from ..enums import LIBRARY_NAME, ActivationType, is_glu
-from .backward import _down_projection_backward, _softmax_topk_bwd, _token_broadcast_backward, _up_projection_backward
+from .backward import (
+    _down_projection_backward,
+    _router_weight_grad,
+    _softmax_topk_bwd,
+    _token_broadcast_backward,
+    _up_projection_backward,
+    router_weight_grad_chunks,
+)
 from .forward import _down_projection_forward, _router_forward, _softmax_topk_fwd, _up_projection_forward
 from .fp8 import (
     _down_projection_forward_fp8,
@@ -121,6 +130,23 @@ def general_routing_router_metadata(
 # ---------------------------------------------------------------------------------------------------------------
 
 
+class _RouterLinearFunction(torch.autograd.Function):
+    """router_logits = F.linear(x, router_w) (sonicmoe/functional/__init__.py:438 of the reference) with the weight
+    gradient as a token-split GEMM (_router_wgrad)."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, router_w: torch.Tensor):
+        ctx.save_for_backward(x, router_w)
+        return F.linear(x, router_w)
+
+    @staticmethod
+    def backward(ctx, dlogits: torch.Tensor):
+        x, router_w = ctx.saved_tensors
+        dx = dlogits @ router_w if ctx.needs_input_grad[0] else None
+        dw = _router_wgrad(dlogits, x, router_w) if ctx.needs_input_grad[1] else None
+        return dx, dw
+
+
 class TC_Softmax_Topk_Router_Function(torch.autograd.Function):
     """(scores fp32 (T, K), indices int32 (T, K)) = softmax(top-K(logits)); backward scatters into a zero (T, E)."""
 
@@ -141,6 +167,65 @@ class TC_Softmax_Topk_Router_Function(torch.autograd.Function):
         dlogits = torch.zeros(scores.size(0), ctx.E, dtype=ctx.logits_dtype, device=scores.device)
         _softmax_topk_bwd(dlogits, None, dscores, scores, indices, ctx.K)
         return dlogits, None, None
+
+
+def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
+                     stream_id, inference):
+    """o = combine(down(act(up(gather(x))))); returns (o, z) with z = None in inference mode."""
+    T, H = x.shape
+    N1, _, E = w1.shape
+    glu = is_glu(activation_type)
+    I = N1 // 2 if glu else N1
+    TK = gidx.numel()
+
+    z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
+    y1 = None if is_using_fp8_forward() else torch.empty(TK, I, dtype=x.dtype, device=x.device)
+    y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
+    if is_using_fp8_forward():
+        xq, xs = mx_quantize(x)
+        w1q, w1s = quantize_expert_weight(w1)
+        # y1 leaves the up-projection already quantised (from the fp32 accumulator); its bf16 form is not stored
+        y1q = torch.empty(TK, I, dtype=torch.uint8, device=x.device)
+        y1s = torch.empty(I // 128, TK, dtype=torch.int32, device=x.device)
+        _up_projection_forward_fp8(
+            xq, xs, w1q, w1s, z, None, b1, off, gidx, E, stream_id, activation_type.value, glu, y1q, y1s
+        )
+        del xq, xs, w1q, w1s
+        w2q, w2s = quantize_expert_weight(w2)
+        _down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, b2, off, E, stream_id)
+        del y1q, y1s, w2q, w2s
+    else:
+        _up_projection_forward(x, w1, z, y1, b1, off, None, gidx, stream_id, activation_type.value, glu, inference)
+        _down_projection_forward(w2, y1, y2, b2, off, None, gidx, stream_id)
+    del y1
+    o = torch.empty(T, H, dtype=x.dtype, device=x.device)
+    _router_forward(y2, o, scores_flat, ridx, tok_off, K_or_maxK, H, is_varlen_K)
+    return o, z
+
+
+def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
+                      activation_type, stream_id):
+    """Returns (dx, dw1, db1, dw2, db2, ds) of _experts_forward."""
+    T, H = x.shape
+    TK = gidx.numel()
+    glu = is_glu(activation_type)
+    dout = dout.contiguous()
+
+    dw2 = torch.empty_like(w2)  # keeps the (E, H, I)-contiguous layout of the parameter view
+    db2 = None if b2 is None else torch.empty_like(b2)
+    dz = torch.empty_like(z)
+    ds = torch.empty(TK, dtype=torch.float32, device=x.device)
+    _down_projection_backward(
+        dout, z, w2, dw2, dz, ds, b2, db2, scores_flat, off, None, gidx, sidx, stream_id, glu, activation_type.value
+    )
+    dw1 = torch.empty_like(w1)
+    db1 = None if b2 is None else torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device)
+    dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
+    _up_projection_backward(x, w1, dx_expanded, dw1, dz, db1, off, None, gidx, sidx, glu, stream_id)
+    del dz
+    dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
+    _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
+    return dx, dw1, db1, dw2, db2, ds
 
 
 class _ExpertsFunction(torch.autograd.Function):
@@ -170,38 +255,10 @@ class _ExpertsFunction(torch.autograd.Function):
         stream_id: int,
         inference: bool,
     ):
-        T, H = x.shape
-        N1, _, E = w1.shape
-        glu = is_glu(activation_type)
-        I = N1 // 2 if glu else N1
-        TK = gidx.numel()
         x = x.contiguous()
         scores_flat = scores_flat.contiguous()
-
-        z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
-        y1 = None if is_using_fp8_forward() else torch.empty(TK, I, dtype=x.dtype, device=x.device)
-        y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
-        if is_using_fp8_forward():
-            xq, xs = mx_quantize(x)
-            w1q, w1s = quantize_expert_weight(w1)
-            # y1 leaves the up-projection already quantised (from the fp32 accumulator); its bf16 form is not stored
-            y1q = torch.empty(TK, I, dtype=torch.uint8, device=x.device)
-            y1s = torch.empty(I // 128, TK, dtype=torch.int32, device=x.device)
-            _up_projection_forward_fp8(
-                xq, xs, w1q, w1s, z, None, b1, off, gidx, E, stream_id, activation_type.value, glu, y1q, y1s
-            )
-            del xq, xs, w1q, w1s
-            w2q, w2s = quantize_expert_weight(w2)
-            _down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, b2, off, E, stream_id)
-            del y1q, y1s, w2q, w2s
-        else:
-            _up_projection_forward(x, w1, z, y1, b1, off, None, gidx, stream_id, activation_type.value, glu, inference)
-            _down_projection_forward(w2, y1, y2, b2, off, None, gidx, stream_id)
-        del y1
-        o = torch.empty(T, H, dtype=x.dtype, device=x.device)
-        _router_forward(y2, o, scores_flat, ridx, tok_off, K_or_maxK, H, is_varlen_K)
-        del y2
-
+        o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K,
+                                activation_type, stream_id, inference)
         if not inference:
             ctx.save_for_backward(x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference)
@@ -213,27 +270,72 @@ class _ExpertsFunction(torch.autograd.Function):
         if inference:
             raise RuntimeError("backward through an inference-mode MoE forward: z was not stored")
         x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
-        T, H = x.shape
-        TK = gidx.numel()
-        glu = is_glu(activation_type)
-        dout = dout.contiguous()
-
-        dw2 = torch.empty_like(w2)  # keeps the (E, H, I)-contiguous layout of the parameter view
-        db2 = None if b2 is None else torch.empty_like(b2)
-        dz = torch.empty_like(z)
-        ds = torch.empty(TK, dtype=torch.float32, device=x.device)
-        _down_projection_backward(
-            dout, z, w2, dw2, dz, ds, b2, db2, scores_flat, off, None, gidx, sidx, stream_id, glu,
-            activation_type.value,
+        dx, dw1, db1, dw2, db2, ds = _experts_backward(
+            dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
+            stream_id,
         )
-        dw1 = torch.empty_like(w1)
-        db1 = None if b2 is None else torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device)
-        dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
-        _up_projection_backward(x, w1, dx_expanded, dw1, dz, db1, off, None, gidx, sidx, glu, stream_id)
-        del dz
-        dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
-        _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
         return dx, dw1, db1, dw2, db2, ds, None, None, None, None, None, None, None, None, None, None
+
+
+def _router_wgrad(dlogits: torch.Tensor, x: torch.Tensor, like: torch.Tensor) -> torch.Tensor:
+    """dWr = dlogits^T x: a token-split GEMM where the kernel supports the shape (it has only E output rows and T
+    contraction elements, which a library GEMM without a split runs on an eighth of the chip), torch otherwise."""
+    T, E = dlogits.shape
+    H = x.size(1)
+    fast = x.is_cuda and x.dtype == torch.bfloat16 and dlogits.dtype == torch.bfloat16 and E % 8 == 0 and H % 8 == 0
+    if fast and T >= 256 and os.environ.get("SMOE_ROUTER_WGRAD", "1") != "0":
+        partial = torch.empty(router_weight_grad_chunks(T, E, H), E, H, dtype=x.dtype, device=x.device)
+        _router_weight_grad(dlogits.contiguous(), x.contiguous(), partial)
+        return partial.sum(0, dtype=torch.float32).to(like.dtype) if partial.size(0) > 1 else partial[0]
+    return dlogits.t() @ x
+
+
+class _TCLayerFunction(torch.autograd.Function):
+    """The whole token-choice layer as one autograd node: router GEMM -> top-K softmax -> metadata -> experts.
+
+    One node instead of three lets the backward pass form dx = dx_experts + dlogits Wr inside the router GEMM
+    (`addmm_` on the experts' dx) instead of leaving the sum of the two paths to autograd's elementwise add, and
+    adds a gradient arriving at router_logits from outside (an auxiliary loss) before the router GEMMs."""
+
+    @staticmethod
+    def forward(ctx, x, router_w, w1, b1, w2, b2, K: int, activation_type: ActivationType, stream_id: int,
+                inference: bool):
+        T, E = x.size(0), router_w.size(0)
+        x = x.contiguous()
+        router_logits = F.linear(x, router_w)
+        scores = torch.empty(T, K, dtype=torch.float32, device=x.device)
+        indices = torch.empty(T, K, dtype=torch.int32, device=x.device)
+        _softmax_topk_fwd(router_logits, scores, indices, E, K)
+        freq, off, gidx, sidx, ridx, tok_off = _build_metadata(indices.view(-1), None, T, E, K)
+        scores_flat = scores.view(-1)
+        o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K, False, activation_type,
+                                stream_id, inference)
+        if not inference:
+            ctx.save_for_backward(x, router_w, w1, w2, b2, z, scores, indices, off, gidx, sidx, ridx, tok_off)
+        ctx.cfg = (K, activation_type, stream_id, inference, router_logits.dtype)
+        ctx.mark_non_differentiable(freq)
+        return o, router_logits, freq
+
+    @staticmethod
+    def backward(ctx, dout, dlogits_outside, _dfreq):
+        K, activation_type, stream_id, inference, logits_dtype = ctx.cfg
+        if inference:
+            raise RuntimeError("backward through an inference-mode MoE forward: z was not stored")
+        x, router_w, w1, w2, b2, z, scores, indices, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
+        T, E = x.size(0), router_w.size(0)
+        dx, dw1, db1, dw2, db2, ds = _experts_backward(
+            dout, x, w1, w2, b2, z, scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id
+        )
+        dlogits = torch.zeros(T, E, dtype=logits_dtype, device=x.device)
+        _softmax_topk_bwd(dlogits, None, ds.view(T, K), scores, indices, K)
+        if dlogits_outside is not None:
+            dlogits = dlogits + dlogits_outside
+        dwr = _router_wgrad(dlogits, x, router_w) if ctx.needs_input_grad[1] else None
+        if ctx.needs_input_grad[0]:
+            dx.addmm_(dlogits, router_w)  # dx_experts + dlogits Wr in the GEMM's epilogue
+        else:
+            dx = None
+        return dx, dwr, dw1, db1, dw2, db2, None, None, None, None
 
 
 def _check_bias(b1, b2):
@@ -271,15 +373,19 @@ def moe_TC_softmax_topk_layer(
     """
     b1, b2 = _check_bias(b1, b2)
     activation_type = _as_activation(activation_type)
-    T, E = x.size(0), router_w.size(0)
-    router_logits = F.linear(x, router_w)
-    topk_scores, topk_indices = TC_Softmax_Topk_Router_Function.apply(router_logits, E, K)
-    freq, off, gidx, sidx, ridx, tok_off = _build_metadata(topk_indices.view(-1), None, T, E, K)
-    o = _ExpertsFunction.apply(
-        x, w1, b1, w2, b2, topk_scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id,
-        is_inference_mode_enabled,
+    if os.environ.get("SMOE_FUSED_TC_LAYER", "1") == "0":  # the layer as three autograd nodes, as the reference builds it
+        T, E = x.size(0), router_w.size(0)
+        router_logits = _RouterLinearFunction.apply(x, router_w)
+        topk_scores, topk_indices = TC_Softmax_Topk_Router_Function.apply(router_logits, E, K)
+        freq, off, gidx, sidx, ridx, tok_off = _build_metadata(topk_indices.view(-1), None, T, E, K)
+        o = _ExpertsFunction.apply(
+            x, w1, b1, w2, b2, topk_scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type,
+            stream_id, is_inference_mode_enabled,
+        )
+        return o, router_logits, freq
+    return _TCLayerFunction.apply(
+        x, router_w, w1, b1, w2, b2, K, activation_type, stream_id, is_inference_mode_enabled
     )
-    return o, router_logits, freq
 
 
 def moe_general_routing_inputs(

@@ -193,3 +193,27 @@ def _softmax_topk_bwd(
         _lib.current_stream_handle(),
     )
     _lib.check(rc, "_softmax_topk_bwd")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_router_weight_grad", mutates_args={"partial"})
+def _router_weight_grad(dlogits: torch.Tensor, x: torch.Tensor, partial: torch.Tensor) -> None:
+    """partial[c] (E, H) = dlogits[rows of chunk c]^T x[rows of chunk c]; the chunks are partial.size(0) equal token
+    ranges.  Their sum is the weight gradient of router_logits = F.linear(x, router_w)."""
+    _lib.require_device(dlogits, x, partial)
+    if dlogits.dtype != torch.bfloat16 or x.dtype != torch.bfloat16 or partial.dtype != torch.bfloat16:
+        raise NotImplementedError("_router_weight_grad: bf16 only")
+    T, E = dlogits.shape
+    H = x.size(1)
+    assert dlogits.is_contiguous() and x.is_contiguous() and partial.is_contiguous()
+    assert x.size(0) == T and partial.shape[1:] == (E, H)
+    rc = _lib.lib().smoe_router_weight_grad(
+        _lib.ptr(dlogits), _lib.ptr(x), _lib.ptr(partial), T, E, H, partial.size(0), _lib.current_stream_handle()
+    )
+    _lib.check(rc, "_router_weight_grad")
+
+
+def router_weight_grad_chunks(T: int, E: int, H: int) -> int:
+    """Token chunks that give the split GEMM at least one 256 x 256 output tile per compute unit, each chunk at least
+    256 tokens long."""
+    tiles = -(-E // 256) * -(-H // 256)
+    return max(1, min(64, -(-256 // tiles), T // 256))

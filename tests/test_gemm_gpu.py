@@ -183,6 +183,32 @@ def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
     assert torch.equal(z1, z) and torch.equal(y11, y1)
 
 
+@pytest.mark.parametrize("T,E,H", [(4096, 64, 512), (300, 128, 256), (1000, 8, 64), (8192, 128, 1024), (5000, 264, 320)])
+def test_router_weight_grad(dev, T, E, H):
+    """dWr = dlogits^T x as a token-split GEMM (partials summed by the caller) against the fp32 product; ragged last
+    chunk, E below and above one 256-row tile, a single chunk."""
+    from sonicmoe.functional.backward import _router_weight_grad, router_weight_grad_chunks
+
+    g = torch.Generator().manual_seed(T + E)
+    dl = (torch.randn(T, E, generator=g) * 0.1).to(torch.bfloat16).to(dev)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    chunks = router_weight_grad_chunks(T, E, H)
+    partial = torch.full((chunks, E, H), 7.0, dtype=torch.bfloat16, device=dev)
+    _router_weight_grad(dl, x, partial)
+    ref = dl.float().t() @ x.float()
+    assert rel_l2(partial.float().sum(0), ref) < TOL
+    # through autograd: the layer's router linear
+    from sonicmoe.functional import _RouterLinearFunction
+
+    w = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16).to(dev).requires_grad_()
+    xr = x.clone().requires_grad_()
+    logits = _RouterLinearFunction.apply(xr, w)
+    gx, gw = torch.autograd.grad(logits, (xr, w), dl)
+    assert rel_l2(gw, ref) < TOL
+    assert rel_l2(gx, dl.float() @ w.detach().float()) < TOL
+    assert rel_l2(logits, x.float() @ w.detach().float().t()) < TOL
+
+
 def test_unsupported_arguments_raise(dev):
     fwd, _ = _ops()
     T, H, I, E, K = 64, 96, 64, 4, 2  # H not a multiple of 64

@@ -68,6 +68,37 @@ def test_moe_forward_backward(dev, T, H, I, E, K):
     assert abs(float(aux) - float(aux_ref)) < 1e-3 * abs(float(aux_ref))
 
 
+def test_fused_layer_node_matches_three_nodes(dev, monkeypatch):
+    """The token-choice layer as one autograd node (dx formed inside the router GEMM, the outside gradient of the
+    logits added before the router GEMMs) against the same layer as three nodes whose dx contributions autograd adds;
+    the loss also reads router_logits directly, as an auxiliary loss does."""
+    from sonicmoe.functional import moe_TC_softmax_topk_layer
+    from helpers import make_weights
+
+    T, H, I, E, K = 2048, 768, 256, 32, 4
+    wr, w1, w2 = make_weights(E, H, I, dev, seed=7)
+    g = torch.Generator().manual_seed(8)
+    x0 = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    dl = (torch.randn(T, E, generator=g) * 0.01).to(torch.bfloat16).to(dev)
+
+    def run(fused):
+        monkeypatch.setenv("SMOE_FUSED_TC_LAYER", "1" if fused else "0")
+        x = x0.clone().requires_grad_()
+        ps = [p.detach().clone().requires_grad_() for p in (wr, w1, w2)]
+        o, logits, freq = moe_TC_softmax_topk_layer(x, ps[0], ps[1].permute(1, 2, 0), None, ps[2].permute(1, 2, 0), None,
+                                                    K, 0)
+        loss = (o.float() * dy.float()).sum() + (logits.float() * dl.float()).sum()
+        return o, logits, freq, torch.autograd.grad(loss, [x] + ps)
+
+    o1, l1, f1, g1 = run(True)
+    o0, l0, f0, g0 = run(False)
+    assert torch.equal(o1, o0) and torch.equal(l1, l0) and torch.equal(f1, f0)
+    for name, a, b in zip(["dx", "d_router_w", "d_w1", "d_w2"], g1, g0):
+        assert rel_l2(a, b) < 5e-3, name  # dx and d_router_w: one rounding less in the fused node
+    assert torch.equal(g1[2], g0[2]) and torch.equal(g1[3], g0[3])
+
+
 def test_inference_mode_matches_training_forward(dev):
     from sonicmoe import KernelBackendMoE
 
