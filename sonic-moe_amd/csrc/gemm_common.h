@@ -328,8 +328,9 @@ static __device__ unsigned long long smoe_phase_ticks[8];
 //                              operation of the wave is outstanding: the place to pick up ordinary loads issued in
 //                              tile_end (a wait for them anywhere else would also wait for the ring)
 //   tile_end(p_slot, q_slot)   epilogue of the finished tile; may use the two slots as scratch (every wave is past the
-//                              barrier behind the last stage); clears the accumulators, advances the caller's tile
-//                              state and returns false if the tile was the workgroup's last
+//                              barrier behind the last stage); advances the caller's tile state and returns false if
+//                              the tile was the workgroup's last.  The accumulators need no clearing: the first slice
+//                              of every tile starts them from zero
 // Needs S >= 3 (stage 0 of the next tile is requested at the latest behind stage S-3 of the current one).  Stores and
 // loads share one counter and may retire out of order with respect to each other, so the first wait of a tile is for
 // everything; from then on only loads are outstanding and the counted waits are exact again.
@@ -348,12 +349,16 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
     static_for<QI>([&](auto j_c) { issue_q(slot, j_c); });
     issued_q();
   };
-  auto slice_mfma = [&](auto cur_c) {
+  // fresh: the first slice of a tile starts the accumulators from the constant 0 operand instead of reading them, so
+  // nobody has to clear 128 registers per lane between tiles
+  auto slice_mfma = [&](auto cur_c, auto fresh_c) {
     constexpr int cur = decltype(cur_c)::value;
+    constexpr bool fresh = decltype(fresh_c)::value;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int q = 0; q < NQ; q++)
 #pragma unroll
-      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
+      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], fresh ? zero : acc[q][pp]);
     constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
 #pragma unroll
     for (int i = 0; i < NR; i++) {
@@ -380,13 +385,16 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
     issued_p();
     issued_q();
   };
-  auto inner_slices = [&](int bp, int bq) {
+  auto inner_slices = [&](int bp, int bq, auto first_stage_c) {
     static_for<SLICES - 1>([&](auto ks_c) {
       constexpr int ks = decltype(ks_c)::value;
       load(bp, bq, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
-      slice_mfma(std::integral_constant<int, (ks & 1)>{});
+      slice_mfma(std::integral_constant<int, (ks & 1)>{},
+                 std::integral_constant<bool, decltype(first_stage_c)::value && ks == 0>{});
     });
   };
+  constexpr std::false_type later{};
+  constexpr std::true_type first{};
 
   all_p(0);
   all_q(0);
@@ -413,22 +421,22 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
   for (;;) {
     // stage 0: stores of the previous epilogue may still be outstanding, wait for everything
     SMOE_PHASE_MARK(5)
-    inner_slices(bp, bq);
+    inner_slices(bp, bq, first);
     wait_vmem_all();
     SMOE_PHASE_MARK(0)
     first_boundary();
     boundary();
     for (int s = 1; s + 1 < S; s++) {
-      inner_slices(bp, bq);
+      inner_slices(bp, bq, later);
       wait_vmem_upto<QI>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
       boundary();
     }
     // last stage: the stages of the next tile that are due are already requested; its own slots become scratch
     SMOE_PHASE_MARK(1)
-    inner_slices(bp, bq);
+    inner_slices(bp, bq, later);
     wait_vmem_upto<QI>();
     lds_barrier();
-    slice_mfma(std::integral_constant<int, 1>{});
+    slice_mfma(std::integral_constant<int, 1>{}, later);
     SMOE_PHASE_MARK(2)
     if (!tile_end(bp, bq)) break;
     SMOE_PHASE_MARK(3)

@@ -459,16 +459,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     }
   }
 
-  f32x16 acc[FN][FM];
-  auto clear_acc = [&]() {
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-      for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
-  };
-  clear_acc();
+  f32x16 acc[FN][FM];  // started from zero by the first slice of every tile
 
   constexpr int Q_RING = C::P_SLOTS * C::P_STAGE;
   int p_stage = 0, q_stage = 0;  // stages issued to each stream for the tile it is on
@@ -541,7 +532,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     if (threadIdx.x == 0) atomicAdd(&smoe_phase_ticks[6], wall_clock64() - t0_);
 #endif
     if (!more) return false;
-    clear_acc();
     cur = nxt;
     nxt = nn;
     more = nxt.valid;
