@@ -6,7 +6,7 @@ namespace smoe {
 
 // One workgroup per token; thread c owns the 8-column chunks c, c+blockDim, ...  UNROLL slots are in flight.
 template <int UNROLL>
-__global__ __launch_bounds__(256) void gather_sum_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ out,
+__global__ __launch_bounds__(512) void gather_sum_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ out,
                                                          const float* __restrict__ w, const int32_t* __restrict__ ridx,
                                                          const int32_t* __restrict__ tok_off, int K, int H) {
   const int64_t t = blockIdx.x;
@@ -188,8 +188,8 @@ extern "C" int smoe_gather_sum(const void* src, void* out, const float* w, const
   SMOE_REQUIRE(tok_off != nullptr || K >= 1, SMOE_ERR_INVALID, "gather_sum: K must be >= 1 without tok_off");
   SMOE_REQUIRE(T < (1ll << 31), SMOE_ERR_UNSUPPORTED, "gather_sum: T too large");
   hipStream_t st = (hipStream_t)stream;
-  int threads = H / 8;
-  if (threads > 256) threads = 256;
+  int threads = H / 8;  // 512 threads (one 16-byte chunk each at H = 4096) measured 4-7 % faster than 256 or 1024 at C2
+  if (threads > 512) threads = 512;
   if (threads < 64) threads = 64;
   hipLaunchKernelGGL(gather_sum_kernel<8>, dim3((unsigned)T), dim3(threads), 0, st, (const uint16_t*)src,
                      (uint16_t*)out, w, ridx, tok_off, K, H);
