@@ -242,9 +242,11 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   p.tiles_a = (int)ceil_div(p.NA, C::BA);
   p.tiles_b = (int)ceil_div(p.NB, C::BB);
   {
-    // SMOE_VARLEN_K_TILE_ORDER (environment, read once): 2 = blocked (default), 0 = round-robin, 1 = whole experts per XCD
-    static const int order = getenv("SMOE_VARLEN_K_TILE_ORDER") ? atoi(getenv("SMOE_VARLEN_K_TILE_ORDER")) : 2;
-    p.xcd_chunked = order;
+    // SMOE_VARLEN_K_TILE_ORDER (environment, read at every launch): 2 = blocked (default), 0 = round-robin,
+    // 1 = whole experts per XCD
+    const char* order = getenv("SMOE_VARLEN_K_TILE_ORDER");
+    p.xcd_chunked = order ? atoi(order) : 2;
+    if (p.xcd_chunked < 0 || p.xcd_chunked > 2) p.xcd_chunked = 2;
   }
   const int64_t total = (int64_t)p.tiles_a * p.tiles_b * p.E;
   int64_t grid = ((total + 7) / 8) * 8;

@@ -561,8 +561,9 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
   if constexpr (ROLE != ROLE_DZ) {
-    // SMOE_GEMM_STREAM=0 (environment, read once) keeps the one-tile-per-workgroup kernel
-    static const bool stream = !(getenv("SMOE_GEMM_STREAM") && atoi(getenv("SMOE_GEMM_STREAM")) == 0);
+    // SMOE_GEMM_STREAM=0 (environment, read at every launch) keeps the one-tile-per-workgroup kernel
+    const char* stream_env = getenv("SMOE_GEMM_STREAM");
+    const bool stream = !(stream_env && atoi(stream_env) == 0);
     if (stream && p.Kdim >= 3 * C::BK) {
       static LdsLimitOnce lds_limit_stream;
       auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;

@@ -183,6 +183,40 @@ def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
     assert torch.equal(z1, z) and torch.equal(y11, y1)
 
 
+@pytest.mark.parametrize("knob,value", [("SMOE_GEMM_STREAM", "0"), ("SMOE_VARLEN_K_TILE_ORDER", "0"),
+                                        ("SMOE_VARLEN_K_TILE_ORDER", "1")])
+def test_kernel_selection_knobs(dev, monkeypatch, knob, value):
+    """The alternative kernels / tile orders an environment variable selects give the same results as the defaults
+    (bit-identical: the arithmetic of a tile does not depend on who computes it or when)."""
+    fwd, bwd = _ops()
+    T, H, I, E, K = 4096, 1024, 512, 32, 8
+    _, w1, w2 = make_weights(E, H, I, dev, seed=31)
+    idx, scores, meta, md = make_tc_routing(T, E, K, dev, seed=32, skew=0.8, empty=(0,))
+    g = torch.Generator().manual_seed(33)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    TK = T * K
+    off, gidx, sidx = (md[k] for k in ("expert_frequency_offset", "x_gather_idx", "s_scatter_idx"))
+    stream = torch.cuda.current_stream().cuda_stream
+    dz = torch.randn(TK, 2 * I, generator=g).to(torch.bfloat16).to(dev)
+
+    def run():
+        z = torch.empty(TK, 2 * I, dtype=torch.bfloat16, device=dev)
+        y1 = torch.empty(TK, I, dtype=torch.bfloat16, device=dev)
+        fwd._up_projection_forward(x, w1.permute(1, 2, 0), z, y1, None, off, None, gidx, stream, "swiglu", True, False)
+        y2 = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
+        fwd._down_projection_forward(w2.permute(1, 2, 0), y1, y2, None, off, None, gidx, stream)
+        dw1 = torch.empty(E, 2 * I, H, dtype=torch.bfloat16, device=dev).permute(1, 2, 0)
+        dxe = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
+        bwd._up_projection_backward(x, w1.permute(1, 2, 0), dxe, dw1, dz, None, off, None, gidx, sidx, True, stream)
+        return z, y1, y2, dw1, dxe
+
+    base = run()
+    monkeypatch.setenv(knob, value)
+    other = run()
+    for name, a, b in zip(["z", "y1", "y2", "dw1", "dx_expanded"], base, other):
+        assert torch.equal(a, b), name
+
+
 @pytest.mark.parametrize("T,E,H", [(4096, 64, 512), (300, 128, 256), (1000, 8, 64), (8192, 128, 1024), (5000, 264, 320)])
 def test_router_weight_grad(dev, T, E, H):
     """dWr = dlogits^T x as a token-split GEMM (partials summed by the caller) against the fp32 product; ragged last
