@@ -62,6 +62,38 @@ struct Cfg {
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
+// Per-lane LDS fragment offsets (bytes inside a ring slot) of wave (wm, wn): p_off[ks] / q_off[ks] for K-major stages
+// (one 16-byte piece per slice), q_off[2 * fn + h] for an MN-major weight stage (two transpose loads per fragment).
+template <class C>
+SMOE_DEV void fragment_offsets(int wm, int wn, int lane, int (&p_off)[C::BK / 16],
+                               int (&q_off)[C::QMN ? 2 * C::FN : C::BK / 16]) {
+  constexpr int SLICES = C::BK / 16;
+  {
+    const int row = wm * C::TM + (lane & 31);
+    const int sw = kswz<C::BK>(row);
+#pragma unroll
+    for (int ks = 0; ks < SLICES; ks++) p_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+  }
+  if constexpr (!C::QMN) {
+    const int row = wn * C::TN + (lane & 31);
+    const int sw = kswz<C::BK>(row);
+#pragma unroll
+    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+  } else {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int kk = 8 * (grp >> 1) + (i16 >> 2);
+#pragma unroll
+    for (int fn = 0; fn < C::FN; fn++) {
+      const int c32 = (wn * C::TN) / 16 + fn * 2 + (grp & 1);
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int k = kk + 4 * h;
+        q_off[fn * 2 + h] = k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+      }
+    }
+  }
+}
+
 // ACT (an smoe_activation) matters to ROLE_UP_FWD and ROLE_DZ only.  p.N counts accumulator columns: the z columns
 // (2I gated, I otherwise) for ROLE_UP_FWD, the y1 columns I for ROLE_DZ.
 template <class C, int ROLE, int ACT>
@@ -129,33 +161,10 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 
   const int S_total = p.Kdim / BK;
 
-  // ---- per-lane LDS fragment offsets (bytes inside a stage) ----
+  // ---- per-lane LDS fragment offsets (bytes inside a ring slot) ----
   int p_off[SLICES];
-  {
-    const int row = wm * C::TM + (lane & 31);
-    const int sw = kswz<BK>(row);
-#pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) p_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
-  }
   int q_off[C::QMN ? 2 * FN : SLICES];
-  if constexpr (!C::QMN) {
-    const int row = wn * C::TN + (lane & 31);
-    const int sw = kswz<BK>(row);
-#pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
-  } else {
-    const int grp = lane >> 4, i16 = lane & 15;
-    const int kk = 8 * (grp >> 1) + (i16 >> 2);
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
-      const int c32 = (wn * C::TN) / 16 + fn * 2 + (grp & 1);
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const int k = kk + 4 * h;
-        q_off[fn * 2 + h] = k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
-      }
-    }
-  }
+  fragment_offsets<C>(wm, wn, lane, p_off, q_off);
 
   f32x16 acc[FN][FM];
 #pragma unroll
@@ -431,33 +440,10 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
 
   const int S_total = p.Kdim / BK;
 
-  // ---- per-lane LDS fragment offsets (bytes inside a stage) ----
+  // ---- per-lane LDS fragment offsets (bytes inside a ring slot) ----
   int p_off[SLICES];
-  {
-    const int row = wm * C::TM + (lane & 31);
-    const int sw = kswz<BK>(row);
-#pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) p_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
-  }
   int q_off[C::QMN ? 2 * FN : SLICES];
-  if constexpr (!C::QMN) {
-    const int row = wn * C::TN + (lane & 31);
-    const int sw = kswz<BK>(row);
-#pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
-  } else {
-    const int grp = lane >> 4, i16 = lane & 15;
-    const int kk = 8 * (grp >> 1) + (i16 >> 2);
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
-      const int c32 = (wn * C::TN) / 16 + fn * 2 + (grp & 1);
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const int k = kk + 4 * h;
-        q_off[fn * 2 + h] = k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
-      }
-    }
-  }
+  fragment_offsets<C>(wm, wn, lane, p_off, q_off);
 
   f32x16 acc[FN][FM];  // started from zero by the first slice of every tile
 
