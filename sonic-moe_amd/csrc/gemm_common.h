@@ -632,28 +632,20 @@ SMOE_DEV void forward_epilogue_rows(f32x16 (&acc)[FN][FM], char* region, int lan
   constexpr int PW = act_pointwise(ACT);
   using LZ = EpiLayout<TN>;
   using LY = EpiLayout<TN / 2>;
-  float bias[FN * 4][4];
   const bool with_bias = a.bias != nullptr;
-  if (with_bias) {
-    static_for<FN * 4>([&](auto q_c) {
-      constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-      int n = a.n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
-      n = n <= a.N - 4 ? n : a.N - 4;
-      const u32x2 b = *(const u32x2*)(a.bias + n);
-      bias[fn * 4 + rg][0] = bf16_lo(b[0]);
-      bias[fn * 4 + rg][1] = bf16_hi(b[0]);
-      bias[fn * 4 + rg][2] = bf16_lo(b[1]);
-      bias[fn * 4 + rg][3] = bf16_hi(b[1]);
-    });
-  }
   const int mrow = lane & 31, half = lane >> 5;
   static_for<FM>([&](auto fm_c) {
     constexpr int fm = decltype(fm_c)::value;
-    if (with_bias) {
+    if (with_bias) {  // re-read per fragment row (a few cached words) rather than held in registers across the rows
       static_for<FN * 4>([&](auto q_c) {
         constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-#pragma unroll
-        for (int q = 0; q < 4; q++) acc[fn][fm][4 * rg + q] += bias[fn * 4 + rg][q];
+        int n = a.n_base + fn * 32 + 8 * rg + 4 * half;
+        n = n <= a.N - 4 ? n : a.N - 4;
+        const u32x2 b = *(const u32x2*)(a.bias + n);
+        acc[fn][fm][4 * rg + 0] += bf16_lo(b[0]);
+        acc[fn][fm][4 * rg + 1] += bf16_hi(b[0]);
+        acc[fn][fm][4 * rg + 2] += bf16_lo(b[1]);
+        acc[fn][fm][4 * rg + 3] += bf16_hi(b[1]);
       });
     }
     const int m0 = a.m_base + fm * 32;
