@@ -161,14 +161,33 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
   const const_i32_ptr gidx = (const_i32_ptr)p.gidx;
   int tok[RPW];  // source row of token (stage base + wave*RPW + j); -1 past the expert's end
-  auto fetch = [&](int s) {
+  // A wave's rows of a stage are consecutive, so their indices come with ONE wide scalar load whenever the whole run
+  // lies inside the expert; element-wise loads (each one waited for before the next is issued, as the compiler
+  // arranges them) are left to the expert's last, ragged stage.
+  typedef int32_t __attribute__((ext_vector_type(RPW), aligned(4))) idx_run;
+  typedef const __attribute__((address_space(4))) idx_run* const_run_ptr;
+  // The run for the following stage is requested when a stage's FIRST load is issued and taken over after its last:
+  // scalar loads return out of order, so the first wait on LDS data behind the request waits for it as well.
+  int tok_next[RPW];
+  auto fetch = [&](int s, int(&dst)[RPW]) {
     const int m0 = row_begin + s * BK + wave * RPW;
+    if (m0 + RPW <= row_end) {
+      if constexpr (C::R_GATHER || C::S_GATHER) {
+        const idx_run run = *(const_run_ptr)(gidx + m0);
+#pragma unroll
+        for (int j = 0; j < RPW; j++) dst[j] = run[j];
+      } else {
+#pragma unroll
+        for (int j = 0; j < RPW; j++) dst[j] = m0 + j;
+      }
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < RPW; j++) {
       const int m = m0 + j;
       const int mc = m < row_end ? m : row_end - 1;
       const int g = (C::R_GATHER || C::S_GATHER) ? gidx[mc] : mc;
-      tok[j] = m < row_end ? g : -1;
+      dst[j] = m < row_end ? g : -1;
     }
   };
   // branch-free: pick this lane's token row among the RPI rows of instruction i, then its global address
@@ -184,6 +203,8 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   auto issue = [&](int buf, int s, auto i_c) {
     constexpr int i = decltype(i_c)::value;
     const uint32_t base = smem_base + buf * C::STAGE;
+    if constexpr (i == 0)
+      if (s + 1 < S) fetch(s + 1, tok_next);  // stages are issued in order
     if constexpr (i < C::R_INSTR) {
       load16_to_lds(piece(p.R, p.r_stride, C::R_GATHER, C::R_RPI, C::R_LPR, s, i, r_col[i]),
                     base + (wave * C::R_INSTR + i) * 1024);
@@ -192,8 +213,10 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       load16_to_lds(piece(p.S, p.s_stride, C::S_GATHER, C::S_RPI, C::S_LPR, s, j, s_col[j]),
                     base + C::R_STAGE + (wave * C::S_INSTR + j) * 1024);
     }
-    if constexpr (i == C::R_INSTR + C::S_INSTR - 1)
-      if (s + 1 < S) fetch(s + 1);  // stages are issued in order: have the next one's rows ready
+    if constexpr (i == C::R_INSTR + C::S_INSTR - 1) {
+#pragma unroll
+      for (int j = 0; j < RPW; j++) tok[j] = tok_next[j];
+    }
   };
   auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
 #ifdef SMOE_PROBE_NO_LDSREAD
@@ -207,7 +230,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     for (int f = 0; f < FB; f++)
       sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
   };
-  if (S > 0) fetch(0);
+  if (S > 0) fetch(0, tok);
   // MFMA as D[b][a] += S[b][k] R[k][a]: lane owns output row a = l%32, register quads hold 4 consecutive columns b
   // two transpose loads per fragment: 12 reads for the 8 MFMAs of a slice, issued two per MFMA
   gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE, Bf16Mma, 2>(S, acc, issue, load);
