@@ -156,7 +156,8 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   // vector loads would share the in-order vmcnt counter with the direct-to-LDS loads and serialise the ring.
   static_assert(C::R_INSTR * C::R_RPI == C::S_INSTR * C::S_RPI, "both operands cover the same token rows per wave");
   constexpr int RPW = C::R_INSTR * C::R_RPI;  // token rows per wave and stage
-  const uint16_t* zero = (const uint16_t*)smoe_zero_page;
+  uint64_t zero = (uint64_t)smoe_zero_page;
+  asm volatile("" : "+s"(zero));  // held in a scalar register pair instead of being re-derived from the pc per load
   // constant address space: a uniform address then becomes a scalar load (the indices are read-only here)
   typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
   const const_i32_ptr gidx = (const_i32_ptr)p.gidx;
@@ -190,15 +191,31 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       dst[j] = m < row_end ? g : -1;
     }
   };
-  // branch-free: pick this lane's token row among the RPI rows of instruction i, then its global address
-  auto piece = [&](const uint16_t* base, int64_t stride, bool gather, int rpi, int lpr, int s, int i, int col) {
+  // Address of this lane's 16-byte piece of load instruction i: ONE 32x32+64-bit multiply-add onto a per-lane pointer.
+  // A gathered operand multiplies the lane's token row (picked among the instruction's RPI rows) onto its column
+  // pointer; an operand read in place has the lane's row inside the expert folded into the pointer and multiplies
+  // the stage's first row.  Rows past the expert's end read the zero page: a select, not a branch.
+  const char* r_ptr[C::R_INSTR];
+  const char* s_ptr[C::S_INSTR];
+  const uint32_t r_row_bytes = (uint32_t)p.r_stride * 2u, s_row_bytes = (uint32_t)p.s_stride * 2u;
+#pragma unroll
+  for (int i = 0; i < C::R_INSTR; i++) {
+    const int64_t row = C::R_GATHER ? 0 : row_begin + wave * RPW + i * C::R_RPI + lane / C::R_LPR;
+    r_ptr[i] = (const char*)(p.R + row * p.r_stride + r_col[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < C::S_INSTR; i++) {
+    const int64_t row = C::S_GATHER ? 0 : row_begin + wave * RPW + i * C::S_RPI + lane / C::S_LPR;
+    s_ptr[i] = (const char*)(p.S + row * p.s_stride + s_col[i]);
+  }
+  auto piece = [&](const char* lane_ptr, uint32_t row_bytes, bool gather, int rpi, int lpr, int s, int i) {
     const int sel = lane / lpr;
     int t = tok[i * rpi];
 #pragma unroll
     for (int j = 1; j < rpi; j++) t = sel == j ? tok[i * rpi + j] : t;
-    const int64_t row = gather ? (int64_t)t : (int64_t)(row_begin + s * BK + wave * RPW + i * rpi + sel);
-    const uint16_t* src = base + row * stride + col;
-    return t < 0 ? zero : src;
+    const uint32_t row = gather ? (uint32_t)t : (uint32_t)(s * BK);
+    const uint64_t src = (uint64_t)row * row_bytes + (uint64_t)lane_ptr;
+    return (const uint16_t*)(t < 0 ? zero : src);
   };
   auto issue = [&](int buf, int s, auto i_c) {
     constexpr int i = decltype(i_c)::value;
@@ -206,11 +223,11 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     if constexpr (i == 0)
       if (s + 1 < S) fetch(s + 1, tok_next);  // stages are issued in order
     if constexpr (i < C::R_INSTR) {
-      load16_to_lds(piece(p.R, p.r_stride, C::R_GATHER, C::R_RPI, C::R_LPR, s, i, r_col[i]),
+      load16_to_lds(piece(r_ptr[i], r_row_bytes, C::R_GATHER, C::R_RPI, C::R_LPR, s, i),
                     base + (wave * C::R_INSTR + i) * 1024);
     } else {
       constexpr int j = i - C::R_INSTR;
-      load16_to_lds(piece(p.S, p.s_stride, C::S_GATHER, C::S_RPI, C::S_LPR, s, j, s_col[j]),
+      load16_to_lds(piece(s_ptr[j], s_row_bytes, C::S_GATHER, C::S_RPI, C::S_LPR, s, j),
                     base + C::R_STAGE + (wave * C::S_INSTR + j) * 1024);
     }
     if constexpr (i == C::R_INSTR + C::S_INSTR - 1) {
@@ -283,6 +300,9 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
     }
   }
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "weight-grad gemm: too many tiles");
+  // the kernel forms source addresses as row * (row stride in bytes, 32 bits) + column pointer
+  SMOE_REQUIRE(p.r_stride > 0 && p.r_stride < (1ll << 31) && p.s_stride > 0 && p.s_stride < (1ll << 31),
+               SMOE_ERR_UNSUPPORTED, "weight-grad gemm: operand row stride out of range");
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
