@@ -99,6 +99,9 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
         dxe = torch.empty(TK, H, dtype=bf, device=dev)
         dx = torch.empty(T, H, dtype=bf, device=dev)
         dlog = torch.zeros(T, E, dtype=bf, device=dev)
+        sl_acc = torch.empty(E, dtype=torch.float32, device=dev)
+        sl_aux = torch.empty(1, dtype=torch.float32, device=dev)
+        sl_g = torch.ones(1, dtype=torch.float32, device=dev)
         w1v, w2v = w1.detach().permute(1, 2, 0), w2.detach().permute(1, 2, 0)
         xd = x.detach()
         sflat = scores.view(-1)
@@ -116,6 +119,9 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
             ("up_projection_backward(dx only)", lambda: backward._up_projection_backward(xd, w1v, dxe, None, dz, None, off, None, gidx, sidx, True, stream), 2 * gemm, None),
             ("token_broadcast_backward", lambda: backward._token_broadcast_backward(dx, dxe, ridx, tok_off, K, H, False), None, TK * H * 2 + T * H * 2 + TK * 4),
             ("softmax_topk_bwd", lambda: backward._softmax_topk_bwd(dlog, None, ds.view(T, K), scores, idx, K), None, T * K * 12 + T * E * 2),
+            # auxiliary (switch) loss of MoE.forward: not part of the timed layer step, listed for completeness
+            ("switch_loss_fwd", lambda: forward._switch_loss_fwd(logits, freq, sl_acc, sl_aux), None, T * E * 2),
+            ("switch_loss_bwd", lambda: backward._switch_loss_bwd(logits, freq, sl_acc, sl_g, dlog), None, T * E * 4),
         ]
         if H % 128 == 0 and I % 128 == 0 and only is None:
             # fp8 forward (config 5 = this shape with block-scaled e4m3 operands): quantisers and the two fp8 GEMMs

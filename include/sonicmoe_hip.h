@@ -164,6 +164,21 @@ int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride
 int smoe_router_weight_grad(const void* dlogits, const void* x, void* partial, int64_t T, int E, int H, int chunks,
                             void* stream);
 
+/* Load-balancing auxiliary loss of MoE.forward (sonicmoe/moe.py:247-274: softmax of the (T, E) logits in fp32, column
+ * sums, two L1 normalisations, a dot product -- six torch kernels and a (T, E) fp32 tensor there):
+ *   acc[e] = sum_t softmax(logits[t, :])[e],   aux[0] = E * <acc / max(|acc|_1, 1e-12), freq / max(|freq|_1, 1e-12)>.
+ * logits (T, E) of `dtype` (smoe_dtype), rows `row_stride` elements apart; freq (E) int32; acc (E) and aux (1) fp32
+ * out.  workspace: smoe_switch_loss_workspace_bytes(T, E).  1 <= E <= 4096.  Deterministic (no atomics). */
+size_t smoe_switch_loss_workspace_bytes(int64_t T, int E);
+int smoe_switch_loss_fwd(const void* logits, int dtype, int64_t row_stride, int64_t T, int E, const int32_t* freq,
+                         float* acc, float* aux, void* workspace, size_t workspace_bytes, void* stream);
+/* Backward of the above (the reference leaves it to autograd through the six torch ops): dlogits (T, E), same dtype as
+ * the logits, = grad_aux[0] * d aux / d logits; acc as written by smoe_switch_loss_fwd; grad_aux (1) fp32 on the
+ * device.  Every element of the (T, E) block is written. */
+int smoe_switch_loss_bwd(const void* logits, int dtype, int64_t row_stride, int64_t T, int E, const int32_t* freq,
+                         const float* acc, const float* grad_aux, void* dlogits, int64_t dlogits_row_stride,
+                         void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------
  * Token-rounding router (benchmarks/moe-token-rounding.py:139-191 of the reference, there a chain of torch ops
  * with a dense (T, E) argsort).  Chain: smoe_tr_softmax -> smoe_topk_softmax_fwd(probs, softmax = 0) ->

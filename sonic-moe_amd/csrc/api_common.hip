@@ -59,5 +59,5 @@ int launch_build_tile_map(const int32_t* off, int E, int BM, TileMap tm, hipStre
 
 }  // namespace smoe
 
-extern "C" int smoe_version(void) { return 210; }
+extern "C" int smoe_version(void) { return 220; }
 extern "C" const char* smoe_last_error(void) { return smoe::g_error; }

@@ -41,6 +41,9 @@ _SIGNATURES = {
         [_P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
     "smoe_router_weight_grad": (c_int, [_P, _P, _P, _L, _I, _I, _I, _P]),
+    "smoe_switch_loss_workspace_bytes": (c_size_t, [_L, _I]),
+    "smoe_switch_loss_fwd": (c_int, [_P, _I, _L, _L, _I, _P, _P, _P, _P, _Z, _P]),
+    "smoe_switch_loss_bwd": (c_int, [_P, _I, _L, _L, _I, _P, _P, _P, _P, _L, _P]),
     "smoe_tr_softmax": (c_int, [_P, _I, _L, _I, _L, _P, _P]),
     "smoe_tr_rank": (c_int, [_P, _P, _I, _P, _P, _L, _I, _I, _P]),
     "smoe_tr_select": (c_int, [_P, _I, _P, _P, _L, _I, _P]),

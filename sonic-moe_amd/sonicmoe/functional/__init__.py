@@ -22,11 +22,18 @@ from .backward import (
     _down_projection_backward,
     _router_weight_grad,
     _softmax_topk_bwd,
+    _switch_loss_bwd,
     _token_broadcast_backward,
     _up_projection_backward,
     router_weight_grad_chunks,
 )
-from .forward import _down_projection_forward, _router_forward, _softmax_topk_fwd, _up_projection_forward
+from .forward import (
+    _down_projection_forward,
+    _router_forward,
+    _softmax_topk_fwd,
+    _switch_loss_fwd,
+    _up_projection_forward,
+)
 from .fp8 import (
     _down_projection_forward_fp8,
     _up_projection_forward_fp8,
@@ -338,6 +345,42 @@ class _TCLayerFunction(torch.autograd.Function):
         return dx, dwr, dw1, db1, dw2, db2, None, None, None, None
 
 
+class _SwitchLossFunction(torch.autograd.Function):
+    """aux = E * <norm_1(sum_t softmax(logits)), norm_1(freq)> (fp32 scalar); the gradient reaches the logits only."""
+
+    @staticmethod
+    def forward(ctx, router_logits: torch.Tensor, expert_frequency: torch.Tensor):
+        E = router_logits.size(-1)
+        logits = router_logits.reshape(-1, E)
+        if logits.stride(1) != 1:
+            logits = logits.contiguous()
+        freq = expert_frequency.to(torch.int32).contiguous()
+        acc = torch.empty(E, dtype=torch.float32, device=logits.device)
+        aux = torch.empty(1, dtype=torch.float32, device=logits.device)
+        _switch_loss_fwd(logits, freq, acc, aux)
+        ctx.save_for_backward(logits, freq, acc)
+        ctx.logits_shape = router_logits.shape
+        return aux.view(())
+
+    @staticmethod
+    def backward(ctx, grad_aux: torch.Tensor):
+        logits, freq, acc = ctx.saved_tensors
+        dlogits = torch.empty_like(logits, memory_format=torch.contiguous_format)
+        _switch_loss_bwd(logits, freq, acc, grad_aux.reshape(1).float().contiguous(), dlogits)
+        return dlogits.view(ctx.logits_shape), None
+
+
+def switch_loss(router_logits: torch.Tensor, expert_frequency: torch.Tensor) -> torch.Tensor:
+    """Load-balancing loss of the reference's MoE._compute_switch_loss (sonicmoe/moe.py:261-274) from the router
+    logits (..., E) and the per-expert token counts (E): the softmax, its column sums, both normalisations and the dot
+    product in two launches forward and one backward, without a (T, E) fp32 tensor."""
+    if router_logits.numel() == 0:  # no tokens: both normalisations clamp and the loss is 0, as in the reference
+        acc = F.softmax(router_logits.reshape(-1, router_logits.size(-1)), dim=-1, dtype=torch.float32).sum(0)
+        f = F.normalize(expert_frequency.float(), p=1, dim=0)
+        return router_logits.size(-1) * (F.normalize(acc, p=1, dim=0) * f).sum()
+    return _SwitchLossFunction.apply(router_logits, expert_frequency)
+
+
 def _check_bias(b1, b2):
     assert (b1 is None) == (b2 is None), "b1 and b2 has to be None or not None at the same time!"
     if b1 is not None:
@@ -428,4 +471,5 @@ __all__ = [
     "is_using_fp8_forward",
     "moe_TC_softmax_topk_layer",
     "moe_general_routing_inputs",
+    "switch_loss",
 ]

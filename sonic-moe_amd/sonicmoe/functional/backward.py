@@ -217,3 +217,22 @@ def router_weight_grad_chunks(T: int, E: int, H: int) -> int:
     256 tokens long."""
     tiles = -(-E // 256) * -(-H // 256)
     return max(1, min(64, -(-256 // tiles), T // 256))
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_switch_loss_bwd", mutates_args={"dlogits"})
+def _switch_loss_bwd(router_logits: torch.Tensor, expert_frequency: torch.Tensor, acc: torch.Tensor,
+                     grad_aux: torch.Tensor, dlogits: torch.Tensor) -> None:
+    """dlogits (T, E) = grad_aux * d aux / d router_logits for the switch loss; acc as left by _switch_loss_fwd.  The
+    reference differentiates its six torch ops with autograd (sonicmoe/moe.py:261-274)."""
+    _lib.require_device(router_logits, expert_frequency, acc, grad_aux, dlogits)
+    if router_logits.dtype not in _lib.DT_CODE or dlogits.dtype != router_logits.dtype:
+        raise NotImplementedError(f"_switch_loss_bwd: unsupported dtypes {router_logits.dtype}, {dlogits.dtype}")
+    T, E = router_logits.shape
+    assert router_logits.stride(1) == 1 and dlogits.stride(1) == 1 and dlogits.shape == router_logits.shape
+    assert grad_aux.numel() == 1 and grad_aux.dtype == torch.float32 and acc.dtype == torch.float32
+    rc = _lib.lib().smoe_switch_loss_bwd(
+        _lib.ptr(router_logits), _lib.DT_CODE[router_logits.dtype], router_logits.stride(0), T, E,
+        _lib.ptr(expert_frequency), _lib.ptr(acc), _lib.ptr(grad_aux), _lib.ptr(dlogits), dlogits.stride(0),
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_switch_loss_bwd")

@@ -197,3 +197,26 @@ def _router_forward(
         is_varlen_K,
         "_router_forward",
     )
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_switch_loss_fwd", mutates_args={"acc", "aux"})
+def _switch_loss_fwd(router_logits: torch.Tensor, expert_frequency: torch.Tensor, acc: torch.Tensor,
+                     aux: torch.Tensor) -> None:
+    """acc (E) fp32 = column sums of softmax(router_logits) in fp32; aux (1) fp32 = E * <acc / |acc|_1, freq / |freq|_1>:
+    the switch loss of the reference's MoE._compute_switch_loss (sonicmoe/moe.py:261-274) in one pass over the
+    logits."""
+    _lib.require_device(router_logits, expert_frequency, acc, aux)
+    if router_logits.dtype not in _lib.DT_CODE:
+        raise NotImplementedError(f"_switch_loss_fwd: unsupported dtype {router_logits.dtype}")
+    T, E = router_logits.shape
+    assert router_logits.stride(1) == 1 and expert_frequency.dtype == torch.int32 and expert_frequency.is_contiguous()
+    assert expert_frequency.numel() == E and acc.numel() == E and acc.dtype == torch.float32 and acc.is_contiguous()
+    assert aux.numel() == 1 and aux.dtype == torch.float32
+    ws_bytes = _lib.lib().smoe_switch_loss_workspace_bytes(T, E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=router_logits.device)
+    rc = _lib.lib().smoe_switch_loss_fwd(
+        _lib.ptr(router_logits), _lib.DT_CODE[router_logits.dtype], router_logits.stride(0), T, E,
+        _lib.ptr(expert_frequency), _lib.ptr(acc), _lib.ptr(aux), _lib.ptr(ws), ws_bytes,
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_switch_loss_fwd")

@@ -15,7 +15,7 @@ import torch.nn.functional as F
 
 from .count_cumsum import count_cumsum
 from .enums import ActivationType, KernelBackendMoE, is_glu
-from .functional import moe_TC_softmax_topk_layer
+from .functional import moe_TC_softmax_topk_layer, switch_loss
 
 
 def _split_gate_up(h: torch.Tensor):
@@ -129,11 +129,15 @@ class MoE(nn.Module):
             raise ValueError(f"unexpected kernel_backend_moe ({kernel_backend_moe})")
 
         out = out.view(shape)
-        aux_loss = self._compute_switch_loss(
-            logits=router_logits,
-            probs=F.softmax(router_logits, dim=-1, dtype=torch.float32),
-            expert_frequency=expert_frequency,
-        )
+        if kernel_backend_moe == KernelBackendMoE.sonicmoe:
+            # same value as _compute_switch_loss below, one pass over the logits instead of six torch kernels
+            aux_loss = switch_loss(router_logits, expert_frequency)
+        else:
+            aux_loss = self._compute_switch_loss(
+                logits=router_logits,
+                probs=F.softmax(router_logits, dim=-1, dtype=torch.float32),
+                expert_frequency=expert_frequency,
+            )
         return out, aux_loss
 
     def _compute_switch_loss(

@@ -99,6 +99,29 @@ def test_fused_layer_node_matches_three_nodes(dev, monkeypatch):
     assert torch.equal(g1[2], g0[2]) and torch.equal(g1[3], g0[3])
 
 
+def test_module_aux_loss_value_and_gradient(dev):
+    """MoE.forward's auxiliary loss on the HIP path (fused switch-loss kernels) against the oracle's formula on the
+    same router logits and expert counts, differentiated by autograd: the value, and the gradients a loss of
+    10 * aux sends to the router weight and the input."""
+    from sonicmoe import KernelBackendMoE
+
+    moe, x, dy = _build(dev, 2048, 512, 256, 32, 4, seed=5, x_scale=1.0)
+    out, aux = moe(x, kernel_backend_moe=KernelBackendMoE.sonicmoe)
+    grads = torch.autograd.grad(10.0 * aux, [x, moe.router.weight])
+    assert aux.dtype == torch.float32
+
+    xr = x.detach().clone().requires_grad_()
+    wr = moe.router.weight.detach().clone().requires_grad_()
+    logits = torch.nn.functional.linear(xr, wr)
+    s_ref, i_ref = R.topk_softmax(logits.detach().float().cpu().numpy(), 4)
+    freq = torch.bincount(torch.from_numpy(i_ref).flatten().long(), minlength=32).to(dev)
+    aux_ref = M.switch_aux_loss(logits, freq)
+    grads_ref = torch.autograd.grad(10.0 * aux_ref, [xr, wr])
+    assert abs(float(aux.detach()) - float(aux_ref.detach())) < 1e-5 * abs(float(aux_ref.detach()))
+    for n, g, gr in zip(["dx", "d_router_w"], grads, grads_ref):
+        assert g.shape == gr.shape and rel_l2(g, gr) < TOL, n
+
+
 def test_inference_mode_matches_training_forward(dev):
     from sonicmoe import KernelBackendMoE
 

@@ -180,3 +180,56 @@ def test_token_rounding_router_on_device(dev, mode, T, E, K, tile, dtype):
     counts = np.bincount(exp.cpu().numpy(), minlength=E)
     assert counts.tolist() == target.tolist()
     assert bool((torch.diff(tok) >= 0).all())
+
+
+@pytest.mark.parametrize("T,E", [(1000, 128), (37, 8), (4096, 256), (300, 100), (65, 1000), (9, 4096), (1, 64), (32768, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32, torch.float16])
+def test_switch_loss_matches_oracle(dev, T, E, dtype):
+    """Fused switch loss (forward value and gradient with respect to the logits) against the oracle's torch formula
+    differentiated by autograd in fp32.  Tolerances: value 1e-5 relative (fp32 sums in another order); gradient
+    rel-L2 1e-5 for fp32 logits, 1e-2 for 16-bit logits (the gradient is rounded to the logits' dtype)."""
+    from oracle import moe_math as M
+    from sonicmoe.functional import switch_loss
+
+    g = torch.Generator().manual_seed(T * 7 + E)
+    logits = (torch.randn(T, E, generator=g) * 1.5).to(dtype)
+    freq = torch.randint(0, 50, (E,), generator=g, dtype=torch.int32)
+    freq[0] += 1  # not all zero
+    ref_in = logits.float().requires_grad_(True)
+    aux_ref = M.switch_aux_loss(ref_in, freq)
+    scale = float(T)  # keeps the gradient's elements (order 1/T per unit of loss) inside fp16's normal range
+    (dref,) = torch.autograd.grad(aux_ref * scale, ref_in)
+
+    x = logits.to(dev).requires_grad_(True)
+    aux = switch_loss(x, freq.to(dev))
+    assert aux.dtype == torch.float32 and aux.dim() == 0
+    (dx,) = torch.autograd.grad(aux * scale, x)
+    torch.cuda.synchronize()
+    assert abs(float(aux.detach()) - float(aux_ref.detach())) <= 1e-5 * abs(float(aux_ref.detach())) + 1e-7
+    assert dx.dtype == dtype and dx.shape == logits.shape
+    err = float((dx.float().cpu() - dref).norm() / dref.norm().clamp_min(1e-30))
+    assert err < (1e-5 if dtype == torch.float32 else 1e-2), err
+
+
+def test_switch_loss_closed_forms(dev):
+    """Uniform router and uniform load give exactly 1; all probability mass and all load on one expert give E; the
+    gradient of a row sums to zero (softmax) and vanishes for a uniform load (the loss is then constant = 1)."""
+    from sonicmoe.functional import switch_loss
+
+    E = 64
+    aux = switch_loss(torch.zeros(128, E, device=dev), torch.full((E,), 16, dtype=torch.int32, device=dev))
+    assert abs(float(aux) - 1.0) < 1e-6
+    logits = torch.full((32, E), -30.0, device=dev)
+    logits[:, 5] = 30.0
+    f = torch.zeros(E, dtype=torch.int32, device=dev)
+    f[5] = 100
+    assert abs(float(switch_loss(logits, f)) - E) < 1e-4
+    x = torch.randn(200, E, device=dev, requires_grad=True)
+    (d,) = torch.autograd.grad(switch_loss(x, torch.randint(1, 9, (E,), dtype=torch.int32, device=dev)), x)
+    assert float(d.sum(1).abs().max()) < 1e-7
+    (d,) = torch.autograd.grad(switch_loss(x, torch.full((E,), 3, dtype=torch.int32, device=dev)), x)
+    assert float(d.abs().max()) < 1e-8
+    # a strided view of a wider tensor is read in place
+    wide = torch.randn(50, 2 * E, device=dev)
+    fr = torch.randint(1, 9, (E,), dtype=torch.int32, device=dev)
+    assert abs(float(switch_loss(wide[:, :E], fr)) - float(switch_loss(wide[:, :E].contiguous(), fr))) < 1e-7
