@@ -63,6 +63,12 @@ def test_argument_checks_return_status_codes(lib):
     # a backward call with every output null has nothing to do
     assert lib.smoe_up_projection_backward(p, p, 0, 0, p, None, 0, 0, None, None, p, p, 4, 8, 64, 64, 2, 0, p, 1 << 20,
                                            None) == 1
+    # switch loss: E outside [1, 4096] -> unsupported; workspace too small -> SMOE_ERR_WORKSPACE
+    assert lib.smoe_switch_loss_fwd(p, 0, 8192, 16, 8192, p, p, p, p, 1 << 20, None) == 2
+    assert b"E=8192" in lib.smoe_last_error()
+    assert lib.smoe_switch_loss_fwd(p, 0, 128, 1024, 128, p, p, p, p, 16, None) == 4
+    assert lib.smoe_switch_loss_bwd(p, 0, 64, 16, 128, p, p, p, p, 128, None) == 1  # row stride below E
+    assert lib.smoe_switch_loss_workspace_bytes(32768, 128) == 256 * 128 * 4
     # workspace size queries are pure host functions
     assert lib.smoe_gemm_workspace_bytes(262144, 128) > 0
     assert lib.smoe_routing_metadata_workspace_bytes(262144, 128) == 2 * 128 * 256 * 4
