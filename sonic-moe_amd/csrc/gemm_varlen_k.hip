@@ -47,8 +47,26 @@ struct KCfg {
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
+#ifdef SMOE_PROBE_PHASES
+// timing probe: ticks (100 MHz) wave 0 of every workgroup spends in set-up, main loop and epilogue, summed over the
+// launch; [3] counts the workgroups, [4] / [5] are the earliest start and the latest end
+static __device__ unsigned long long smoe_kphase_ticks[8];
+#define SMOE_KPHASE(k)                              \
+  {                                                 \
+    const unsigned long long now_ = wall_clock64(); \
+    kphase_[k] += now_ - klast_;                    \
+    klast_ = now_;                                  \
+  }
+#else
+#define SMOE_KPHASE(k)
+#endif
+
 template <class C>
 __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) {
+#ifdef SMOE_PROBE_PHASES
+  unsigned long long kphase_[4] = {}, klast_ = wall_clock64();
+  const unsigned long long kstart_ = klast_;
+#endif
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
   const uint32_t smem_base = lds_address(smem);
@@ -248,10 +266,12 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
   };
   if (S > 0) fetch(0, tok);
+  SMOE_KPHASE(0)
   // MFMA as D[b][a] += S[b][k] R[k][a]: lane owns output row a = l%32, register quads hold 4 consecutive columns b
   // two transpose loads per fragment: 12 reads for the 8 MFMAs of a slice, issued two per MFMA
   gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE, Bf16Mma, 2>(S, acc, issue, load);
 
+  SMOE_KPHASE(1)
   // epilogue through LDS (also writes the zeros of experts without tokens)
   using L = EpiLayout<C::TB>;
   char* region = smem + wave * (C::TA * L::ROW_BYTES);
@@ -268,6 +288,15 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   });
   epilogue_flush<C::TA, C::TB>(region, lane, p.out + (int64_t)e * p.out_stride_e, p.out_stride_row, a0 + wa * C::TA,
                                p.NA, b0 + wb * C::TB, p.NB);
+#ifdef SMOE_PROBE_PHASES
+  SMOE_KPHASE(2)
+  if (threadIdx.x == 0) {
+    for (int k = 0; k < 3; k++) atomicAdd(&smoe_kphase_ticks[k], kphase_[k]);
+    atomicAdd(&smoe_kphase_ticks[3], 1ull);
+    atomicMin(&smoe_kphase_ticks[4], kstart_);
+    atomicMax(&smoe_kphase_ticks[5], klast_);
+  }
+#endif
 }
 
 template <class C>
@@ -474,3 +503,13 @@ extern "C" int smoe_router_weight_grad(const void* dlogits, const void* x, void*
   p.E = chunks;
   return launch_varlen_k_variant<false, false>(p, (hipStream_t)stream);
 }
+
+#ifdef SMOE_PROBE_PHASES
+// timing probe: read and reset the phase counters of the weight-gradient kernel
+extern "C" int smoe_probe_kphases(unsigned long long* out) {
+  unsigned long long init[8] = {0, 0, 0, 0, ~0ull, 0, 0, 0};
+  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(smoe::smoe_kphase_ticks), sizeof(init)) != hipSuccess) return -1;
+  if (hipMemcpyToSymbol(HIP_SYMBOL(smoe::smoe_kphase_ticks), init, sizeof(init)) != hipSuccess) return -1;
+  return 0;
+}
+#endif
