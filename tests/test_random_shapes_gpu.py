@@ -1,0 +1,71 @@
+"""Seeded random layer configurations (ragged H / I / T, every activation, with and without bias, balanced and heavily
+unbalanced routing with empty experts): module forward + backward on the HIP path against the oracle's restatement of
+the reference's torch backend, driven with the oracle's own top-K choice.  Tolerance: rel-L2 <= 1e-2 (bf16 bar)."""
+
+import random
+
+import pytest
+import torch
+
+from oracle import moe_math as M
+from oracle import routing as R
+from helpers import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+ACTS = ["swiglu", "geglu", "reglu", "relu_sq", "relu", "gelu", "silu"]
+
+
+def _config(seed):
+    rng = random.Random(1000 + seed)
+    H = 64 * rng.randint(1, 32)
+    I = 64 * rng.randint(1, 20)
+    E = rng.choice([4, 8, 12, 16, 32, 64, 128, 256])
+    K = rng.randint(1, min(E // 4 if E >= 8 else E, 12))
+    T = rng.choice([64, 255, 300, 1000, 2048, 4097])
+    return T, H, I, E, K, ACTS[seed % len(ACTS)], seed % 3 == 0, seed % 4 == 1
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_layer_configuration(dev, seed):
+    from sonicmoe import MoE, KernelBackendMoE
+    from sonicmoe.enums import ActivationType
+
+    T, H, I, E, K, act, bias, unbalanced = _config(seed)
+    torch.manual_seed(seed)
+    moe = MoE(E, K, H, I, ActivationType(act), bias, 0.02).to(device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():
+        moe.router.weight.normal_(0, 0.02)
+        if bias:
+            moe.c_fc.bias.normal_(0, 0.01)
+            moe.c_proj.bias.normal_(0, 0.01)
+        if unbalanced and E >= 8:
+            # a quarter of the experts share one router row four times the others' scale: their logits tie, about half
+            # of the tokens (those with a negative coordinate sum) pick the lowest-numbered of them, the rest of the
+            # quarter stays empty.  (A larger row, e.g. -0.5, makes the router path dominate dx and its error the
+            # bf16 rounding of dlogits: 1.4e-2, above the bar, in the reference's arithmetic as well.)
+            moe.router.weight[: E // 4] = -0.08
+    x = torch.randn(T, H, device=dev).to(torch.bfloat16).requires_grad_()
+    dy = torch.randn(T, H, device=dev).to(torch.bfloat16)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_proj.weight] + ([moe.c_fc.bias, moe.c_proj.bias] if bias else [])
+
+    out, _ = moe(x, kernel_backend_moe=KernelBackendMoE.sonicmoe)
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+
+    with torch.no_grad():
+        logits = torch.nn.functional.linear(x, moe.router.weight)
+    _, i_ref = R.topk_softmax(logits.float().cpu().numpy(), K)
+    sel = torch.from_numpy(i_ref).to(dev)
+    xr = x.detach().clone().requires_grad_()
+    pr = [p.detach().clone().requires_grad_() for p in params]
+    out_ref, _, freq_ref = M.moe_torch_backend(xr, pr[0], pr[1], pr[2], K, b1=pr[3] if bias else None,
+                                               b2=pr[4] if bias else None, selected_experts=sel, activation=act)
+    grads_ref = torch.autograd.grad(out_ref, [xr] + pr, grad_outputs=dy.float())
+    if unbalanced and E // 4 > K:
+        assert int((freq_ref == 0).sum()) > 0  # the case really has experts without tokens
+
+    assert rel_l2(out, out_ref) < TOL
+    for n, g, gr in zip(["dx", "d_router_w", "d_w1", "d_w2", "d_b1", "d_b2"], grads, grads_ref):
+        assert g.shape == gr.shape
+        assert rel_l2(g, gr) < TOL, n
