@@ -124,7 +124,19 @@ struct Bf16Mma {
 };
 
 // RPM: LDS reads slotted in behind each of the first MFMAs of a slice
-template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Mma = Bf16Mma, int RPM = 1, class Issue, class Load>
+// The first stages of a main loop, issued on their own: a kernel that works through several tiles starts the next
+// tile's loads before the finished tile's epilogue and enters gemm_mainloop<..., PROLOGUE = false> behind it.
+template <int LPS, int NSTAGE, class Issue>
+SMOE_DEV void gemm_mainloop_prologue(const int S, Issue&& issue) {
+  const int pre = S < NSTAGE ? S : NSTAGE;
+  for (int s = 0; s < pre; s++) static_for<LPS>([&](auto i_c) { issue(s, s, i_c); });
+}
+
+// PROLOGUE = false: the first min(S, NSTAGE) stages have been issued by gemm_mainloop_prologue, possibly with other
+// vector-memory operations (an epilogue's stores) behind them: the first wait is then for everything, because loads
+// and stores may retire out of order and a counted wait could not tell which are left.
+template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Mma = Bf16Mma, int RPM = 1,
+          bool PROLOGUE = true, class Issue, class Load>
 SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, Load&& load) {
   if (S <= 0) return;
   static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
@@ -133,7 +145,8 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
   constexpr int NM = NQ * NP;
   auto issue_all = [&](int buf, int s) { static_for<LPS>([&](auto i_c) { issue(buf, s, i_c); }); };
   const int pre = S < NSTAGE ? S : NSTAGE;
-  for (int s = 0; s < pre; s++) issue_all(s, s);
+  if constexpr (PROLOGUE)
+    for (int s = 0; s < pre; s++) issue_all(s, s);
 
   auto wait_next_stage = [&](int younger) {  // `younger` stages were issued after the one we need
     if constexpr (NSTAGE >= 6) if (younger >= 4) { wait_vmem_upto<4 * LPS>(); return; }
@@ -184,7 +197,8 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
     });
   };
 
-  wait_next_stage(pre - 1);
+  if constexpr (PROLOGUE) wait_next_stage(pre - 1);
+  else wait_vmem_all();
   lds_barrier();
   load(0, 0, 0, qf[0], pf[0]);
   int buf = 0;
@@ -729,14 +743,14 @@ int launch_build_tile_map(const int32_t* off, int E, int BM, TileMap tm, hipStre
 
 // XCD-aware linear tile id: workgroups are dealt round-robin to the 8 XCDs, so workgroup b runs on XCD b % 8;
 // give every XCD one contiguous range of the tile space so that tiles sharing operands share an L2.
-SMOE_DEV int64_t xcd_linear_tile(int64_t total) {
-  const int64_t b = blockIdx.x;
+SMOE_DEV int64_t xcd_linear_tile_of(int64_t b, int64_t total) {
   const int64_t per = (total + 7) >> 3;
   const int64_t slot = b >> 3;
   if (slot >= per) return -1;
   const int64_t lin = (b & 7) * per + slot;
   return lin < total ? lin : -1;
 }
+SMOE_DEV int64_t xcd_linear_tile(int64_t total) { return xcd_linear_tile_of(blockIdx.x, total); }
 
 int launch_ds_finalize(const float* ds_partial, int ncols, const int32_t* sidx, float* ds, int64_t TK, hipStream_t st);
 

@@ -184,7 +184,8 @@ def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
 
 
 @pytest.mark.parametrize("knob,value", [("SMOE_GEMM_STREAM", "0"), ("SMOE_VARLEN_K_TILE_ORDER", "0"),
-                                        ("SMOE_VARLEN_K_TILE_ORDER", "1")])
+                                        ("SMOE_VARLEN_K_TILE_ORDER", "1"), ("SMOE_VARLEN_K_TILES", "1"),
+                                        ("SMOE_VARLEN_K_TILES", "2"), ("SMOE_VARLEN_K_TILES", "3")])
 def test_kernel_selection_knobs(dev, monkeypatch, knob, value):
     """The alternative kernels / tile orders an environment variable selects give the same results as the defaults
     (bit-identical: the arithmetic of a tile does not depend on who computes it or when)."""
