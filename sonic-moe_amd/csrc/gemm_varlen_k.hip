@@ -51,6 +51,39 @@ struct KCfg {
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
+// Tile order.  Workgroup slot v runs on XCD v % 8 and every XCD runs 32 slots side by side.  An expert's cost is its
+// token count, so every expert is spread over several XCDs (skewed loads stay balanced), in blocks that share operand
+// panels in the XCD's L2 (the blocked order); order 0 deals single tiles round-robin instead, order 1 gives every XCD
+// one contiguous range of tiles.  Returns false when slot v holds no tile (then no later slot does either).
+SMOE_DEV bool decode_tile(const VarlenKParams& p, int64_t v, int& e, int& ta, int& tb) {
+  const int64_t per_e = (int64_t)p.tiles_a * p.tiles_b;
+  if (p.xcd_chunked == 2) {
+    // Blocked order: the 32 tiles an XCD runs side by side are one ba x bb block of ONE expert's output (8 blocks of
+    // 32 consecutive workgroup slots per round of 256 slots), so per stage they fetch ba + bb operand panels
+    // instead of one or two panels each.  Block B runs on XCD (B + B/8) % 8: an expert's blocks go to neighbouring
+    // XCDs, and the rotation keeps any XCD from always getting the same experts.
+    const int bb = p.tiles_b < 8 ? p.tiles_b : 8, ba = 32 / bb;
+    const int nbj = p.tiles_b / bb, nb = (p.tiles_a / ba) * nbj;  // blocks per expert
+    const int xcd = (int)(v & 7);
+    const int64_t j = v >> 3, seq = j >> 5;
+    const int in = (int)(j & 31);
+    const int64_t B = seq * 8 + ((xcd + 8 - (int)(seq & 7)) & 7);
+    if (B >= (int64_t)nb * p.E) return false;
+    e = (int)(B / nb);
+    const int blk = (int)(B - (int64_t)e * nb);
+    ta = (blk / nbj) * ba + in / bb;
+    tb = (blk % nbj) * bb + in % bb;
+    return true;
+  }
+  const int64_t lin = p.xcd_chunked ? xcd_linear_tile_of(v, per_e * p.E) : (v < per_e * p.E ? v : -1);
+  if (lin < 0) return false;
+  e = (int)(lin / per_e);
+  const int within = (int)(lin - (int64_t)e * per_e);
+  ta = within / p.tiles_b;
+  tb = within % p.tiles_b;
+  return true;
+}
+
 #ifdef SMOE_PROBE_PHASES
 // timing probe: ticks (100 MHz) wave 0 of every workgroup spends in set-up, main loop and epilogue, summed over the
 // launch; [3] counts the workgroups, [4] / [5] are the earliest start and the latest end
@@ -78,34 +111,8 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave % C::WA, wb = wave / C::WA;
 
-  // Tile order.  Workgroup b runs on XCD b % 8 and every XCD runs 32 workgroups side by side.  An expert's cost is its
-  // token count, so every expert is spread over several XCDs (skewed loads stay balanced), in blocks that share operand
-  // panels in the XCD's L2 (see the blocked order below); order 0 deals single tiles round-robin instead.
-  const int64_t per_e = (int64_t)p.tiles_a * p.tiles_b;
   int e, ta, tb;
-  if (p.xcd_chunked == 2) {
-    // Blocked order: the 32 tiles an XCD runs side by side are one ba x bb block of ONE expert's output (8 blocks of
-    // 32 consecutive workgroup slots per round of 256 workgroups), so per stage they fetch ba + bb operand panels
-    // instead of one or two panels each.  Block B runs on XCD (B + B/8) % 8: an expert's blocks go to neighbouring
-    // XCDs, and the rotation keeps any XCD from always getting the same experts.
-    const int bb = p.tiles_b < 8 ? p.tiles_b : 8, ba = 32 / bb;
-    const int nbj = p.tiles_b / bb, nb = (p.tiles_a / ba) * nbj;  // blocks per expert
-    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
-    const int seq = j >> 5, in = j & 31;
-    const int64_t B = (int64_t)seq * 8 + ((xcd + 8 - (seq & 7)) & 7);
-    if (B >= (int64_t)nb * p.E) return;
-    e = (int)(B / nb);
-    const int blk = (int)(B - (int64_t)e * nb);
-    ta = (blk / nbj) * ba + in / bb;
-    tb = (blk % nbj) * bb + in % bb;
-  } else {
-    const int64_t lin = p.xcd_chunked ? xcd_linear_tile(per_e * p.E) : (blockIdx.x < per_e * p.E ? (int64_t)blockIdx.x : -1);
-    if (lin < 0) return;
-    e = (int)(lin / per_e);
-    const int within = (int)(lin - (int64_t)e * per_e);
-    ta = within / p.tiles_b;
-    tb = within % p.tiles_b;
-  }
+  if (!decode_tile(p, (int64_t)blockIdx.x, e, ta, tb)) return;
   const int a0 = ta * C::BA, b0 = tb * C::BB;
   int row_begin, row_end;
   if (p.off != nullptr) {
@@ -301,33 +308,6 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     atomicMax(&smoe_kphase_ticks[5], klast_);
   }
 #endif
-}
-
-// Tile order.  Workgroup slot v runs on XCD v % 8 and every XCD runs 32 slots side by side.  Returns false when slot v
-// holds no tile (then no later slot of the same workgroup does either).  See varlen_k_kernel for the orders.
-SMOE_DEV bool decode_tile(const VarlenKParams& p, int64_t v, int& e, int& ta, int& tb) {
-  const int64_t per_e = (int64_t)p.tiles_a * p.tiles_b;
-  if (p.xcd_chunked == 2) {
-    const int bb = p.tiles_b < 8 ? p.tiles_b : 8, ba = 32 / bb;
-    const int nbj = p.tiles_b / bb, nb = (p.tiles_a / ba) * nbj;  // blocks per expert
-    const int xcd = (int)(v & 7);
-    const int64_t j = v >> 3, seq = j >> 5;
-    const int in = (int)(j & 31);
-    const int64_t B = seq * 8 + ((xcd + 8 - (int)(seq & 7)) & 7);
-    if (B >= (int64_t)nb * p.E) return false;
-    e = (int)(B / nb);
-    const int blk = (int)(B - (int64_t)e * nb);
-    ta = (blk / nbj) * ba + in / bb;
-    tb = (blk % nbj) * bb + in % bb;
-    return true;
-  }
-  const int64_t lin = p.xcd_chunked ? xcd_linear_tile_of(v, per_e * p.E) : (v < per_e * p.E ? v : -1);
-  if (lin < 0) return false;
-  e = (int)(lin / per_e);
-  const int within = (int)(lin - (int64_t)e * per_e);
-  ta = within / p.tiles_b;
-  tb = within % p.tiles_b;
-  return true;
 }
 
 // ---- several tiles per workgroup ------------------------------------------------------------------------------------
