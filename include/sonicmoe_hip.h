@@ -93,6 +93,21 @@ int smoe_routing_metadata(const int32_t* expert_idx, const int32_t* token_idx, i
                           int32_t* s_reverse_scatter_idx, int32_t* tok_off, void* workspace, size_t workspace_bytes,
                           void* stream);
 
+/* smoe_routing_metadata for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc) and have no workspace to hand in.  No counterpart in the reference.  Same
+ * arguments, results and limits as smoe_routing_metadata minus the workspace: the two (E, ceil(TK / 1024)) int32
+ * tables of the counting sort live in an array of SMOE_ROUTING_METADATA_STATIC_BYTES that is part of the library
+ * image (each GPU the library runs on holds one copy until the process ends).  The call allocates and frees nothing.
+ *   - sizes with smoe_routing_metadata_workspace_bytes(TK, E) > SMOE_ROUTING_METADATA_STATIC_BYTES are rejected with
+ *     SMOE_ERR_WORKSPACE (e.g. TK = 262144 fits up to E = 2048, E = 128 up to TK = 4194304)
+ *   - every call on one GPU uses that GPU's one array: calls that may overlap on a GPU (different streams or
+ *     threads) race; order them.  Nothing in the array has to be cleared between calls. */
+#define SMOE_ROUTING_METADATA_STATIC_BYTES (4u << 20)
+size_t smoe_routing_metadata_static_capacity(void);
+int smoe_routing_metadata_static(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T, int E,
+                                 int K, int32_t* freq, int32_t* off, int32_t* x_gather_idx, int32_t* s_scatter_idx,
+                                 int32_t* s_reverse_scatter_idx, int32_t* tok_off, void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------
  * Grouped GEMMs (bf16 in, fp32 MFMA accumulate, bf16 out)
  * ------------------------------------------------------------------------------------------------------ */

@@ -2,6 +2,8 @@
 // metadata, router backward.  All integer outputs are deterministic (no order-dependent atomics reach an output).
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace smoe {
@@ -450,20 +452,25 @@ extern "C" size_t smoe_routing_metadata_workspace_bytes(int64_t TK, int E) {
   return (size_t)2 * (size_t)E * (size_t)meta_segments(TK) * sizeof(int32_t);
 }
 
-extern "C" int smoe_routing_metadata(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T,
-                                     int E, int K, int32_t* freq, int32_t* off, int32_t* x_gather_idx,
-                                     int32_t* s_scatter_idx, int32_t* s_reverse_scatter_idx, int32_t* tok_off,
-                                     void* workspace, size_t workspace_bytes, void* stream) {
+// argument checks shared by the two metadata entry points (everything but the scratch memory)
+static int check_routing_metadata_args(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T, int E,
+                                       int K, const int32_t* freq, const int32_t* off, const int32_t* x_gather_idx,
+                                       const int32_t* s_scatter_idx, const int32_t* s_reverse_scatter_idx) {
   SMOE_REQUIRE(TK >= 0 && T >= 0, SMOE_ERR_INVALID, "routing_metadata: negative size");
   SMOE_REQUIRE(TK < (1ll << 31), SMOE_ERR_UNSUPPORTED, "routing_metadata: TK does not fit int32");
   SMOE_REQUIRE(E >= 1 && E <= 4096, SMOE_ERR_UNSUPPORTED, "routing_metadata: E=%d outside [1, 4096]", E);
-  SMOE_REQUIRE(freq && off && workspace, SMOE_ERR_INVALID, "routing_metadata: null pointer");
+  SMOE_REQUIRE(freq && off, SMOE_ERR_INVALID, "routing_metadata: null pointer");
   SMOE_REQUIRE(TK == 0 || (expert_idx && x_gather_idx && s_scatter_idx && s_reverse_scatter_idx), SMOE_ERR_INVALID,
                "routing_metadata: null pointer");
   SMOE_REQUIRE(token_idx != nullptr || K >= 1, SMOE_ERR_INVALID, "routing_metadata: K must be >= 1 without token_idx");
-  SMOE_REQUIRE(workspace_bytes >= smoe_routing_metadata_workspace_bytes(TK, E), SMOE_ERR_WORKSPACE,
-               "routing_metadata: workspace too small");
-  hipStream_t st = (hipStream_t)stream;
+  return SMOE_OK;
+}
+
+// the three passes of the counting sort; `workspace` holds the two (E, NS) int32 tables, both written in full by
+// the first two passes before they are read (nothing in it has to start at zero)
+static int launch_routing_metadata(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T, int E,
+                                   int K, int32_t* freq, int32_t* off, int32_t* x_gather_idx, int32_t* s_scatter_idx,
+                                   int32_t* s_reverse_scatter_idx, int32_t* tok_off, void* workspace, hipStream_t st) {
   const int NS = meta_segments(TK);
   int32_t* hist_t = (int32_t*)workspace;
   int32_t* base_t = hist_t + (size_t)E * NS;
@@ -479,4 +486,68 @@ extern "C" int smoe_routing_metadata(const int32_t* expert_idx, const int32_t* t
                      freq, base_t, off, x_gather_idx, s_scatter_idx, s_reverse_scatter_idx, tok_off);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
+}
+
+extern "C" int smoe_routing_metadata(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T,
+                                     int E, int K, int32_t* freq, int32_t* off, int32_t* x_gather_idx,
+                                     int32_t* s_scatter_idx, int32_t* s_reverse_scatter_idx, int32_t* tok_off,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+  const int rc = check_routing_metadata_args(expert_idx, token_idx, TK, T, E, K, freq, off, x_gather_idx, s_scatter_idx,
+                                             s_reverse_scatter_idx);
+  if (rc) return rc;
+  SMOE_REQUIRE(workspace != nullptr, SMOE_ERR_INVALID, "routing_metadata: null pointer");
+  SMOE_REQUIRE(workspace_bytes >= smoe_routing_metadata_workspace_bytes(TK, E), SMOE_ERR_WORKSPACE,
+               "routing_metadata: workspace too small");
+  return launch_routing_metadata(expert_idx, token_idx, TK, T, E, K, freq, off, x_gather_idx, s_scatter_idx,
+                                 s_reverse_scatter_idx, tok_off, workspace, (hipStream_t)stream);
+}
+
+// ---- the same operator for callers that cannot allocate ------------------------------------------------------
+// The two tables live in a device array that is part of the library image: one copy per GPU, at an address of its
+// own on each, looked up once per device.  In host code the array's NAME is only a handle for that look-up; the
+// kernels get the looked-up pointer.
+static __device__ __align__(256) unsigned char scratch[SMOE_ROUTING_METADATA_STATIC_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[MAX_DEVICES] = {};  // device address of `scratch` on each GPU, null = not looked up yet
+}  // namespace
+
+// device address of this GPU's copy of `scratch`
+static int static_scratch(void** out) {
+  int dev = 0;
+  SMOE_HIP_CHECK(hipGetDevice(&dev));
+  SMOE_REQUIRE(dev >= 0 && dev < MAX_DEVICES, SMOE_ERR_UNSUPPORTED, "routing_metadata_static: device %d out of range",
+               dev);
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    SMOE_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SMOE_REQUIRE(p != nullptr, SMOE_ERR_HIP, "routing_metadata_static: no device address for the scratch array");
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return SMOE_OK;
+}
+
+extern "C" size_t smoe_routing_metadata_static_capacity(void) { return SMOE_ROUTING_METADATA_STATIC_BYTES; }
+
+extern "C" int smoe_routing_metadata_static(const int32_t* expert_idx, const int32_t* token_idx, int64_t TK, int64_t T,
+                                            int E, int K, int32_t* freq, int32_t* off, int32_t* x_gather_idx,
+                                            int32_t* s_scatter_idx, int32_t* s_reverse_scatter_idx, int32_t* tok_off,
+                                            void* stream) {
+  int rc = check_routing_metadata_args(expert_idx, token_idx, TK, T, E, K, freq, off, x_gather_idx, s_scatter_idx,
+                                       s_reverse_scatter_idx);
+  if (rc) return rc;
+  const size_t need = smoe_routing_metadata_workspace_bytes(TK, E);
+  SMOE_REQUIRE(need <= (size_t)SMOE_ROUTING_METADATA_STATIC_BYTES, SMOE_ERR_WORKSPACE,
+               "routing_metadata_static: TK=%lld, E=%d need %zu bytes of scratch, the built-in array holds %zu; use "
+               "smoe_routing_metadata with a workspace of your own",
+               (long long)TK, E, need, (size_t)SMOE_ROUTING_METADATA_STATIC_BYTES);
+  void* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc) return rc;
+  return launch_routing_metadata(expert_idx, token_idx, TK, T, E, K, freq, off, x_gather_idx, s_scatter_idx,
+                                 s_reverse_scatter_idx, tok_off, ws, (hipStream_t)stream);
 }

@@ -27,6 +27,8 @@ _SIGNATURES = {
     "smoe_softmax_topk_bwd": (c_int, [_P, _I, _L, _P, _P, _P, _L, _I, _P]),
     "smoe_routing_metadata_workspace_bytes": (c_size_t, [_L, _I]),
     "smoe_routing_metadata": (c_int, [_P, _P, _L, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "smoe_routing_metadata_static_capacity": (c_size_t, []),
+    "smoe_routing_metadata_static": (c_int, [_P, _P, _L, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     "smoe_gemm_workspace_bytes": (c_size_t, [_L, _I]),
     "smoe_up_projection_forward": (c_int, [_P, _P, _L, _L, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P]),
     "smoe_down_projection_forward": (c_int, [_P, _P, _L, _L, _P, _P, _P, _L, _I, _I, _I, _P, _Z, _P]),
