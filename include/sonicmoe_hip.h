@@ -52,6 +52,16 @@ typedef enum {
 int smoe_version(void);
 const char* smoe_last_error(void);
 
+/* Kernel-selection knobs.  Each is read from the environment once, at the first launch that needs it; this call
+ * overrides one afterwards (value < 0 restores the default).  Results do not depend on any of them; they exist for
+ * tuning and so that tests can walk through every kernel.  No counterpart in the reference.
+ *   "gemm_stream"          SMOE_GEMM_STREAM          1: token-grouped GEMMs run as tile streams (default); 0: one tile
+ *                                                    per workgroup
+ *   "gemm_stream_grid"     SMOE_GEMM_STREAM_GRID     workgroups of a tile-stream launch; 0 = one per compute unit
+ *   "varlen_k_tiles"       SMOE_VARLEN_K_TILES       tiles per workgroup of the weight-gradient GEMMs; 0 = by shape
+ *   "varlen_k_tile_order"  SMOE_VARLEN_K_TILE_ORDER  2 blocked (default), 0 round-robin, 1 whole experts per XCD */
+int smoe_set_tuning(const char* name, int value);
+
 /* ---------------------------------------------------------------------------------------------------------
  * Routing
  * ------------------------------------------------------------------------------------------------------ */

@@ -1,6 +1,10 @@
 // Library-wide pieces of the C ABI: version, thread-local error text, and the tile-map builder that turns the
 // expert offsets into a list of token tiles on the device (no host synchronisation anywhere on the hot path).
 #include <stdarg.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
 
 #include "gemm_common.h"
 
@@ -13,6 +17,56 @@ void set_error(const char* fmt, ...) {
   va_start(ap, fmt);
   vsnprintf(g_error, sizeof(g_error), fmt, ap);
   va_end(ap);
+}
+
+namespace {
+std::once_flag g_tuning_once;
+Tuning g_tuning = {1, 0, 0, 2, 0};
+
+struct Knob {
+  const char* name;
+  const char* env;
+  int Tuning::*field;
+  int lo, hi, def;
+};
+const Knob g_knobs[] = {
+    {"gemm_stream", "SMOE_GEMM_STREAM", &Tuning::gemm_stream, 0, 1, 1},
+    {"gemm_stream_grid", "SMOE_GEMM_STREAM_GRID", &Tuning::gemm_stream_grid, 0, 1 << 30, 0},
+    {"varlen_k_tiles", "SMOE_VARLEN_K_TILES", &Tuning::varlen_k_tiles, 0, 1 << 20, 0},
+    {"varlen_k_tile_order", "SMOE_VARLEN_K_TILE_ORDER", &Tuning::varlen_k_tile_order, 0, 2, 2},
+    {"experiment", "SMOE_EXPERIMENT", &Tuning::experiment, 0, 1 << 20, 0},
+};
+
+void read_tuning_env() {
+  for (const Knob& k : g_knobs) {
+    const char* v = getenv(k.env);
+    if (v == nullptr || *v == 0) continue;
+    const long x = strtol(v, nullptr, 10);
+    g_tuning.*(k.field) = x < k.lo || x > k.hi ? k.def : (int)x;
+  }
+}
+}  // namespace
+
+const Tuning& tuning() {
+  std::call_once(g_tuning_once, read_tuning_env);
+  return g_tuning;
+}
+
+int device_compute_units(int* out) {
+  static int cus[64] = {};
+  int dev = 0;
+  SMOE_HIP_CHECK(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64 || cus[dev] == 0) {
+    int n = 0;
+    SMOE_HIP_CHECK(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+    if (dev < 0 || dev >= 64) {
+      *out = n;
+      return SMOE_OK;
+    }
+    cus[dev] = n;
+  }
+  *out = cus[dev];
+  return SMOE_OK;
 }
 
 __global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __restrict__ off, int E, int BM,
@@ -61,3 +115,18 @@ int launch_build_tile_map(const int32_t* off, int E, int BM, TileMap tm, hipStre
 
 extern "C" int smoe_version(void) { return 220; }
 extern "C" const char* smoe_last_error(void) { return smoe::g_error; }
+
+extern "C" int smoe_set_tuning(const char* name, int value) {
+  SMOE_REQUIRE(name != nullptr, SMOE_ERR_INVALID, "set_tuning: null name");
+  smoe::tuning();  // the environment is read first, so that it cannot overwrite this call later
+  for (const smoe::Knob& k : smoe::g_knobs) {
+    if (strcmp(name, k.name) != 0) continue;
+    if (value < 0) value = k.def;
+    SMOE_REQUIRE(value >= k.lo && value <= k.hi, SMOE_ERR_INVALID, "set_tuning: %s = %d outside [%d, %d]", name, value,
+                 k.lo, k.hi);
+    smoe::g_tuning.*(k.field) = value;
+    return SMOE_OK;
+  }
+  smoe::set_error("set_tuning: unknown knob '%s'", name);
+  return SMOE_ERR_INVALID;
+}

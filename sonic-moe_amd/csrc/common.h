@@ -32,6 +32,17 @@ void set_error(const char* fmt, ...);  // thread-local message behind smoe_last_
 
 static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+// The GEMM kernels move operands in 16-byte pieces (8 bf16): base pointers must be 16-byte aligned and row / expert
+// strides multiples of 8 elements.  Null pointers (optional arguments) pass.
+static inline bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+static inline bool stride8(int64_t s) { return s % 8 == 0; }
+#define SMOE_REQUIRE_ALIGNED(who, ...)                                                                       \
+  do {                                                                                                       \
+    const void* _ptrs[] = {__VA_ARGS__};                                                                     \
+    for (const void* _p : _ptrs)                                                                             \
+      SMOE_REQUIRE(::smoe::aligned16(_p), SMOE_ERR_UNSUPPORTED, "%s: tensor pointers must be 16-byte aligned", who); \
+  } while (0)
+
 // ---- device-side types -----------------------------------------------------------------------------------
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;

@@ -75,15 +75,8 @@ SMOE_DEV void static_for(F&& f) {
   static_for_impl<0, N>(f);
 }
 
-// -DSMOE_PROBE_NO_MFMA / -DSMOE_PROBE_NO_REFILL build timing probes (wrong results) that remove the matrix
-// instructions resp. the steady-state global loads, to tell which side of the pipeline bounds a kernel.
 SMOE_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-#ifdef SMOE_PROBE_NO_MFMA
-  c[0] += (float)a[0] * (float)b[0];
-  return c;
-#else
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-#endif
 }
 
 // s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wave's vector-memory operations (oldest first) may still be
@@ -180,11 +173,7 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
       acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
       static_for<LPS>([&](auto j_c) {
         constexpr int j = decltype(j_c)::value;
-#ifdef SMOE_PROBE_HALF_REFILL
-        if constexpr (j * NM / LPS == i && j < LPS / 2) issue(buf, s_new, j_c);
-#else
         if constexpr (j * NM / LPS == i) issue(buf, s_new, j_c);
-#endif
       });
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -203,7 +192,6 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
   load(0, 0, 0, qf[0], pf[0]);
   int buf = 0;
   int s = 0;
-#ifndef SMOE_PROBE_NO_REFILL
   for (; s + NSTAGE < S; s++) {  // steady state: every stage boundary refills the slot it frees
     inner_slices(buf, s);
     wait_next_stage(NSTAGE - 2);
@@ -214,7 +202,6 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
     slice_mfma_refill(buf, s + NSTAGE);
     buf = next;
   }
-#endif
   for (; s < S - 1; s++) {  // drain: nothing left to fetch
     inner_slices(buf, s);
     const int younger = S - 2 - s < NSTAGE - 2 ? S - 2 - s : NSTAGE - 2;
@@ -321,13 +308,6 @@ SMOE_DEV void gemm_mainloop_asym(const int S, f32x16 (&acc)[NQ][NP], IssueP&& is
   slice_mfma(std::integral_constant<int, 1>{});
 }
 
-#ifdef SMOE_PROBE_PHASES
-// timing probe: ticks (100 MHz) wave 0 of every workgroup spends in the phases of a tile, summed over the launch
-static __device__ unsigned long long smoe_phase_ticks[8];
-#define SMOE_PHASE_MARK(k) { const unsigned long long now_ = wall_clock64(); phase_[k] += now_ - last_; last_ = now_; }
-#else
-#define SMOE_PHASE_MARK(k)
-#endif
 
 // ---- main loop over a STREAM of tiles ------------------------------------------------------------------------------
 // A workgroup that works through several output tiles keeps the asymmetric ring running across the tile boundary: the
@@ -387,12 +367,10 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
       acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
       static_for<LPS>([&](auto j_c) {
         constexpr int j = decltype(j_c)::value;
-#ifndef SMOE_PROBE_NO_REFILL
         if constexpr (j * NM / LPS == i) {
           if constexpr (j < PI) issue_p(p_slot, j_c);
           else issue_q(q_slot, std::integral_constant<int, j - PI>{});
         }
-#endif
       });
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -419,9 +397,6 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
   lds_barrier();
   load(0, 0, 0, qf[0], pf[0]);
   int bp = 0, bq = 0;
-#ifdef SMOE_PROBE_PHASES
-  unsigned long long phase_[8] = {}, last_ = wall_clock64();
-#endif
   // boundary behind a stage that is not the tile's last: read slice 0 of the next stage, refill the vacated slots
   auto boundary = [&]() {
     lds_barrier();
@@ -434,10 +409,8 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
   };
   for (;;) {
     // stage 0: stores of the previous epilogue may still be outstanding, wait for everything
-    SMOE_PHASE_MARK(5)
     inner_slices(bp, bq, first);
     wait_vmem_all();
-    SMOE_PHASE_MARK(0)
     first_boundary();
     boundary();
     for (int s = 1; s + 1 < S; s++) {
@@ -446,14 +419,11 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
       boundary();
     }
     // last stage: the stages of the next tile that are due are already requested; its own slots become scratch
-    SMOE_PHASE_MARK(1)
     inner_slices(bp, bq, later);
     wait_vmem_upto<QI>();
     lds_barrier();
     slice_mfma(std::integral_constant<int, 1>{}, later);
-    SMOE_PHASE_MARK(2)
     if (!tile_end(bp, bq)) break;
-    SMOE_PHASE_MARK(3)
     wait_lds_all();
     lds_barrier();  // every wave has read its parked rows back: the two slots may be refilled
     all_p(bp);
@@ -461,12 +431,7 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
     bp ^= 1;
     bq = bq == 2 ? 0 : bq + 1;
     load(bp, bq, 0, qf[0], pf[0]);
-    SMOE_PHASE_MARK(4)
   }
-#ifdef SMOE_PROBE_PHASES
-  if (threadIdx.x == 0)
-    for (int k = 0; k < 8; k++) atomicAdd(&smoe_phase_ticks[k], phase_[k]);
-#endif
   wait_vmem_all();  // the streams ran ahead into ring slots nobody reads any more: let those loads land before the end
 }
 
@@ -696,6 +661,21 @@ SMOE_DEV void forward_epilogue_rows(f32x16 (&acc)[FN][FM], char* region, int lan
     }
   });
 }
+
+// ---- tuning knobs ----------------------------------------------------------------------------------------------
+// Read from the environment ONCE, at the first launch that asks (variable = "SMOE_" + the upper-cased field name);
+// smoe_set_tuning() overrides a knob afterwards (tests walk through the alternative kernels with it).
+struct Tuning {
+  int gemm_stream;          // 1 (default): up-projection forward, down-projection forward, dz and dx run as tile streams
+  int gemm_stream_grid;     // workgroups of the tile-stream kernels; 0 (default) = one per compute unit
+  int varlen_k_tiles;       // tiles per workgroup of the weight-gradient kernels; 0 (default) = chosen from the shape
+  int varlen_k_tile_order;  // 2 blocked (default), 0 single tiles round-robin over the XCDs, 1 whole experts per XCD
+  int experiment;           // scratch knob for kernel experiments (no effect in a release build)
+};
+const Tuning& tuning();
+
+// number of compute units of the current device (looked up once per device)
+int device_compute_units(int* out);
 
 // ---- launch helper -------------------------------------------------------------------------------------------------
 // Raise a kernel's dynamic-LDS limit once per device (the attribute is per device; a repeated call is harmless, so the

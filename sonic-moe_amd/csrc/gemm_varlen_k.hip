@@ -6,8 +6,6 @@
 // materialised gathered copy.  Experts without tokens still get their zeros written.
 //   dW1[e] (2I, H): R = dz rows,              S = x rows gathered
 //   dW2[e] (H, I) : R = dout rows gathered,   S = y1s rows
-#include <stdlib.h>
-
 #include "gemm_common.h"
 
 namespace smoe {
@@ -84,26 +82,9 @@ SMOE_DEV bool decode_tile(const VarlenKParams& p, int64_t v, int& e, int& ta, in
   return true;
 }
 
-#ifdef SMOE_PROBE_PHASES
-// timing probe: ticks (100 MHz) wave 0 of every workgroup spends in set-up, main loop and epilogue, summed over the
-// launch; [3] counts the workgroups, [4] / [5] are the earliest start and the latest end
-static __device__ unsigned long long smoe_kphase_ticks[8];
-#define SMOE_KPHASE(k)                              \
-  {                                                 \
-    const unsigned long long now_ = wall_clock64(); \
-    kphase_[k] += now_ - klast_;                    \
-    klast_ = now_;                                  \
-  }
-#else
-#define SMOE_KPHASE(k)
-#endif
 
 template <class C>
 __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) {
-#ifdef SMOE_PROBE_PHASES
-  unsigned long long kphase_[4] = {}, klast_ = wall_clock64();
-  const unsigned long long kstart_ = klast_;
-#endif
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
   const uint32_t smem_base = lds_address(smem);
@@ -265,9 +246,6 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     }
   };
   auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
-#ifdef SMOE_PROBE_NO_LDSREAD
-    return;
-#endif
     const char* st = smem + buf * C::STAGE;
 #pragma unroll
     for (int f = 0; f < FA; f++)
@@ -277,12 +255,9 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
   };
   if (S > 0) fetch(0, tok);
-  SMOE_KPHASE(0)
   // MFMA as D[b][a] += S[b][k] R[k][a]: lane owns output row a = l%32, register quads hold 4 consecutive columns b
   // two transpose loads per fragment: 12 reads for the 8 MFMAs of a slice, issued two per MFMA
   gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE, Bf16Mma, 2>(S, acc, issue, load);
-
-  SMOE_KPHASE(1)
   // epilogue through LDS (also writes the zeros of experts without tokens)
   using L = EpiLayout<C::TB>;
   char* region = smem + wave * (C::TA * L::ROW_BYTES);
@@ -299,15 +274,6 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   });
   epilogue_flush<C::TA, C::TB>(region, lane, p.out + (int64_t)e * p.out_stride_e, p.out_stride_row, a0 + wa * C::TA,
                                p.NA, b0 + wb * C::TB, p.NB);
-#ifdef SMOE_PROBE_PHASES
-  SMOE_KPHASE(2)
-  if (threadIdx.x == 0) {
-    for (int k = 0; k < 3; k++) atomicAdd(&smoe_kphase_ticks[k], kphase_[k]);
-    atomicAdd(&smoe_kphase_ticks[3], 1ull);
-    atomicMin(&smoe_kphase_ticks[4], kstart_);
-    atomicMax(&smoe_kphase_ticks[5], klast_);
-  }
-#endif
 }
 
 // ---- several tiles per workgroup ------------------------------------------------------------------------------------
@@ -536,13 +502,7 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   VarlenKParams p = pin;
   p.tiles_a = (int)ceil_div(p.NA, C::BA);
   p.tiles_b = (int)ceil_div(p.NB, C::BB);
-  {
-    // SMOE_VARLEN_K_TILE_ORDER (environment, read at every launch): 2 = blocked (default), 0 = round-robin,
-    // 1 = whole experts per XCD
-    const char* order = getenv("SMOE_VARLEN_K_TILE_ORDER");
-    p.xcd_chunked = order ? atoi(order) : 2;
-    if (p.xcd_chunked < 0 || p.xcd_chunked > 2) p.xcd_chunked = 2;
-  }
+  p.xcd_chunked = tuning().varlen_k_tile_order;
   const int64_t total = (int64_t)p.tiles_a * p.tiles_b * p.E;
   int64_t grid = ((total + 7) / 8) * 8;
   if (p.xcd_chunked == 2) {
@@ -563,10 +523,10 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   if constexpr (C::NSTAGE == 2 && C::NW == 8 && C::SMEM_MULTI <= 160 * 1024) {
     // Tiles a workgroup works through: 2 when the experts average at most 1024 rows (tiles of at most 16 stages, of
     // which the turnaround between two workgroups is a quarter: 2 % of a step at 512 rows per expert, nothing at
-    // 2048), else 1; SMOE_VARLEN_K_TILES (environment, read at every launch) overrides.  The grid stays a multiple of
-    // 256 slots so that a workgroup's tiles keep its XCD and its place in the blocked order.
-    const char* tiles_env = getenv("SMOE_VARLEN_K_TILES");
-    const int want = tiles_env ? atoi(tiles_env) : (p.total_rows <= (int64_t)1024 * p.E ? 2 : 1);
+    // 2048), else 1; the varlen_k_tiles knob overrides.  The grid stays a multiple of 256 slots so that a
+    // workgroup's tiles keep its XCD and its place in the blocked order.
+    const int knob = tuning().varlen_k_tiles;
+    const int want = knob > 0 ? knob : (p.total_rows <= (int64_t)1024 * p.E ? 2 : 1);
     if (want > 1 && grid >= 512 && grid % 256 == 0) {
       const int64_t rounds = grid / 256;
       const int64_t wg_rounds = (rounds + want - 1) / want;
@@ -585,25 +545,10 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   return SMOE_OK;
 }
 
-// SMOE_GEMM_VARIANT_K (environment, read once) picks the tile configuration of the varlen-K kernels; 3 = default.
-int gemm_variant_k() {
-  static int v = -1;
-  if (v < 0) {
-    const char* e = getenv("SMOE_GEMM_VARIANT_K");
-    v = e ? atoi(e) : 3;
-    if (v < 0 || v > 3) v = 3;
-  }
-  return v;
-}
-
+// 256 x 256 output tile, 8 wavefronts as 2 x 4, 64 token rows per stage, double buffer
 template <bool RG, bool SG>
 static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st) {
-  switch (gemm_variant_k()) {
-    case 0: return launch_varlen_k<KCfg<256, 256, 2, 2, RG, SG, 32, 5>>(p, st);   // 4 waves, BK 32, ring
-    case 1: return launch_varlen_k<KCfg<256, 256, 2, 2, RG, SG, 64, 2>>(p, st);   // 4 waves, BK 64, double buffer
-    case 2: return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 32, 5>>(p, st);   // 8 waves, BK 32, ring
-    default: return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 64, 2>>(p, st);  // 8 waves, BK 64, double buffer
-  }
+  return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 64, 2>>(p, st);
 }
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
@@ -647,6 +592,9 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
   SMOE_REQUIRE(TK == 0 || !db2 || (scores && s_scatter_idx), SMOE_ERR_INVALID,
                "down_projection_backward: db2 needs scores and s_scatter_idx");
   (void)T;
+  SMOE_REQUIRE_ALIGNED("down_projection_backward", dout, z, w2, b2, dw2, db2, dz, y1s);
+  SMOE_REQUIRE(stride8(w2_stride_e) && stride8(w2_stride_row) && stride8(dw2_stride_e) && stride8(dw2_stride_row),
+               SMOE_ERR_UNSUPPORTED, "down_projection_backward: weight strides must be multiples of 8 elements");
   hipStream_t st = (hipStream_t)stream;
   if (TK > 0 && dz) {
     rc = launch_dz(dout, z, w2, w2_stride_e, w2_stride_row, dz, y1s, ds_partial, scores, off, x_gather_idx,
@@ -698,6 +646,9 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
   SMOE_REQUIRE(TK == 0 || (dz && x_gather_idx && (!dw1 || x) && (!dx_expanded || w1)), SMOE_ERR_INVALID,
                "up_projection_backward: null pointer");
   (void)T;
+  SMOE_REQUIRE_ALIGNED("up_projection_backward", x, w1, dz, dw1, db1, dx_expanded);
+  SMOE_REQUIRE(stride8(w1_stride_e) && stride8(w1_stride_row) && stride8(dw1_stride_e) && stride8(dw1_stride_row),
+               SMOE_ERR_UNSUPPORTED, "up_projection_backward: weight strides must be multiples of 8 elements");
   hipStream_t st = (hipStream_t)stream;
   const int N1 = activation <= SMOE_ACT_REGLU ? 2 * I : I;  // columns of z and dz: (gate, up) pairs when gated
   if (db1) {
@@ -736,6 +687,7 @@ extern "C" int smoe_router_weight_grad(const void* dlogits, const void* x, void*
   SMOE_REQUIRE(H >= 8 && H % 8 == 0, SMOE_ERR_UNSUPPORTED, "router_weight_grad: H=%d must be a multiple of 8", H);
   SMOE_REQUIRE(chunks >= 1, SMOE_ERR_INVALID, "router_weight_grad: chunks must be positive");
   SMOE_REQUIRE(dlogits && x && partial, SMOE_ERR_INVALID, "router_weight_grad: null pointer");
+  SMOE_REQUIRE_ALIGNED("router_weight_grad", dlogits, x, partial);
   VarlenKParams p = {};
   p.R = (const uint16_t*)dlogits;
   p.r_stride = E;
@@ -754,12 +706,3 @@ extern "C" int smoe_router_weight_grad(const void* dlogits, const void* x, void*
   return launch_varlen_k_variant<false, false>(p, (hipStream_t)stream);
 }
 
-#ifdef SMOE_PROBE_PHASES
-// timing probe: read and reset the phase counters of the weight-gradient kernel
-extern "C" int smoe_probe_kphases(unsigned long long* out) {
-  unsigned long long init[8] = {0, 0, 0, 0, ~0ull, 0, 0, 0};
-  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(smoe::smoe_kphase_ticks), sizeof(init)) != hipSuccess) return -1;
-  if (hipMemcpyToSymbol(HIP_SYMBOL(smoe::smoe_kphase_ticks), init, sizeof(init)) != hipSuccess) return -1;
-  return 0;
-}
-#endif

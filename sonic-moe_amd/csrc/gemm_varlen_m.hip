@@ -186,9 +186,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     q_src[j] += q_step;
   };
   auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
-#ifdef SMOE_PROBE_NO_LDSREAD
-    return;
-#endif
     const char* sp = smem + p_slot * C::P_STAGE;
     const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
 #pragma unroll
@@ -472,9 +469,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     }
   };
   auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
-#ifdef SMOE_PROBE_NO_LDSREAD
-    return;
-#endif
     const char* sp = smem + p_slot * C::P_STAGE;
     const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
 #pragma unroll
@@ -510,13 +504,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     // waves 0..NW/2-1 park in the vacated P slot, the others in the vacated Q slot
     char* region = wave < C::NW / 2 ? smem + p_slot * C::P_STAGE + wave * PARK
                                     : smem + Q_RING + q_slot * C::Q_STAGE + (wave - C::NW / 2) * PARK;
-#ifdef SMOE_PROBE_PHASES
-    const unsigned long long t0_ = wall_clock64();
-#endif
     forward_epilogue_rows<C::TN, FM, FN, ROLE == ROLE_UP_FWD, ACT>(acc, region, opaque_lane(), ea);
-#ifdef SMOE_PROBE_PHASES
-    if (threadIdx.x == 0) atomicAdd(&smoe_phase_ticks[6], wall_clock64() - t0_);
-#endif
     if (!more) return false;
     cur = nxt;
     nxt = nn;
@@ -547,21 +535,18 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
   if constexpr (ROLE != ROLE_DZ) {
-    // SMOE_GEMM_STREAM=0 (environment, read at every launch) keeps the one-tile-per-workgroup kernel
-    const char* stream_env = getenv("SMOE_GEMM_STREAM");
-    const bool stream = !(stream_env && atoi(stream_env) == 0);
-    if (stream && p.Kdim >= 3 * C::BK) {
+    const Tuning& tune = tuning();
+    if (tune.gemm_stream && p.Kdim >= 3 * C::BK) {
       static LdsLimitOnce lds_limit_stream;
       auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
       const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
       if (rc_s) return rc_s;
-      int dev = 0, cus = 0;
-      SMOE_HIP_CHECK(hipGetDevice(&dev));
-      SMOE_HIP_CHECK(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+      int cus = 0;
+      const int rc_cu = device_compute_units(&cus);
+      if (rc_cu) return rc_cu;
       int64_t sgrid = ((int64_t)cus / 8) * 8;  // one resident workgroup per compute unit, the same number on every XCD
-      // SMOE_GEMM_STREAM_GRID (environment, read at every launch) overrides the number of workgroups: small values
-      // make small problems run several tiles per workgroup (used by the tests)
-      if (const char* g = getenv("SMOE_GEMM_STREAM_GRID")) sgrid = ((int64_t)atoi(g) + 7) / 8 * 8;
+      // a smaller grid makes small problems run several tiles per workgroup (used by the tests)
+      if (tune.gemm_stream_grid > 0) sgrid = ((int64_t)tune.gemm_stream_grid + 7) / 8 * 8;
       if (sgrid < 8) sgrid = 8;
       if (sgrid > grid) sgrid = grid;
       hipLaunchKernelGGL(skern, dim3((unsigned)sgrid), dim3(C::NT), C::SMEM, st, p);
@@ -631,6 +616,9 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
   if (TK == 0) return SMOE_OK;
   SMOE_REQUIRE(x && w1 && y1 && off && x_gather_idx, SMOE_ERR_INVALID, "up_projection_forward: null pointer");
   SMOE_REQUIRE(T > 0, SMOE_ERR_INVALID, "up_projection_forward: T must be positive");
+  SMOE_REQUIRE_ALIGNED("up_projection_forward", x, w1, b1, z, y1);
+  SMOE_REQUIRE(stride8(w1_stride_e) && stride8(w1_stride_row), SMOE_ERR_UNSUPPORTED,
+               "up_projection_forward: weight strides must be multiples of 8 elements");
   hipStream_t st = (hipStream_t)stream;
   VarlenMParams p = {};
   p.P = (const uint16_t*)x;
@@ -657,6 +645,9 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
   if (rc) return rc;
   if (TK == 0) return SMOE_OK;
   SMOE_REQUIRE(y1 && w2 && y2 && off, SMOE_ERR_INVALID, "down_projection_forward: null pointer");
+  SMOE_REQUIRE_ALIGNED("down_projection_forward", y1, w2, b2, y2);
+  SMOE_REQUIRE(stride8(w2_stride_e) && stride8(w2_stride_row), SMOE_ERR_UNSUPPORTED,
+               "down_projection_forward: weight strides must be multiples of 8 elements");
   hipStream_t st = (hipStream_t)stream;
   VarlenMParams p = {};
   p.P = (const uint16_t*)y1;
@@ -720,12 +711,3 @@ int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_st
 
 }  // namespace smoe
 
-#ifdef SMOE_PROBE_PHASES
-// timing probe: read and clear the phase counters of the tile-stream kernels
-extern "C" int smoe_probe_phases(unsigned long long* out) {
-  unsigned long long zero[8] = {};
-  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(smoe::smoe_phase_ticks), sizeof(zero)) != hipSuccess) return -1;
-  if (hipMemcpyToSymbol(HIP_SYMBOL(smoe::smoe_phase_ticks), zero, sizeof(zero)) != hipSuccess) return -1;
-  return 0;
-}
-#endif

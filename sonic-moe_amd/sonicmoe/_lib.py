@@ -22,6 +22,7 @@ _P, _I, _L, _Z = c_void_p, c_int, c_int64, c_size_t
 _SIGNATURES = {
     "smoe_version": (c_int, []),
     "smoe_last_error": (c_char_p, []),
+    "smoe_set_tuning": (c_int, [c_char_p, _I]),
     "smoe_count_cumsum": (c_int, [_P, _I, _L, _I, _P, _P, _P]),
     "smoe_topk_softmax_fwd": (c_int, [_P, _I, _L, _I, _I, _L, _P, _P, _I, _P]),
     "smoe_softmax_topk_bwd": (c_int, [_P, _I, _L, _P, _P, _P, _L, _I, _P]),
@@ -91,6 +92,11 @@ def check(rc: int, what: str) -> None:
     if rc != 0:
         msg = lib().smoe_last_error().decode(errors="replace")
         raise RuntimeError(f"{what} failed (status {rc}): {msg}")
+
+
+def set_tuning(name: str, value: int) -> None:
+    """Override a kernel-selection knob of the library (value < 0 restores the default)."""
+    check(lib().smoe_set_tuning(name.encode(), int(value)), f"smoe_set_tuning({name}, {value})")
 
 
 def ptr(t: torch.Tensor | None):

@@ -211,8 +211,9 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
 
 
 def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
-                      activation_type, stream_id):
-    """Returns (dx, dw1, db1, dw2, db2, ds) of _experts_forward."""
+                      activation_type, stream_id, has_b1):
+    """Returns (dx, dw1, db1, dw2, db2, ds) of _experts_forward; `has_b1` says whether the forward pass had an
+    up-projection bias (b1 itself is not needed for any gradient and is not kept)."""
     T, H = x.shape
     TK = gidx.numel()
     glu = is_glu(activation_type)
@@ -226,7 +227,7 @@ def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx
         dout, z, w2, dw2, dz, ds, b2, db2, scores_flat, off, None, gidx, sidx, stream_id, glu, activation_type.value
     )
     dw1 = torch.empty_like(w1)
-    db1 = None if b2 is None else torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device)
+    db1 = torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device) if has_b1 else None
     dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
     _up_projection_backward(x, w1, dx_expanded, dw1, dz, db1, off, None, gidx, sidx, glu, stream_id)
     del dz
@@ -268,18 +269,18 @@ class _ExpertsFunction(torch.autograd.Function):
                                 activation_type, stream_id, inference)
         if not inference:
             ctx.save_for_backward(x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
-        ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference)
+        ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference, b1 is not None)
         return o
 
     @staticmethod
     def backward(ctx, dout):
-        K_or_maxK, is_varlen_K, activation_type, stream_id, inference = ctx.cfg
+        K_or_maxK, is_varlen_K, activation_type, stream_id, inference, has_b1 = ctx.cfg
         if inference:
             raise RuntimeError("backward through an inference-mode MoE forward: z was not stored")
         x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
         dx, dw1, db1, dw2, db2, ds = _experts_backward(
             dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
-            stream_id,
+            stream_id, has_b1,
         )
         return dx, dw1, db1, dw2, db2, ds, None, None, None, None, None, None, None, None, None, None
 
@@ -319,19 +320,20 @@ class _TCLayerFunction(torch.autograd.Function):
                                 stream_id, inference)
         if not inference:
             ctx.save_for_backward(x, router_w, w1, w2, b2, z, scores, indices, off, gidx, sidx, ridx, tok_off)
-        ctx.cfg = (K, activation_type, stream_id, inference, router_logits.dtype)
+        ctx.cfg = (K, activation_type, stream_id, inference, router_logits.dtype, b1 is not None)
         ctx.mark_non_differentiable(freq)
         return o, router_logits, freq
 
     @staticmethod
     def backward(ctx, dout, dlogits_outside, _dfreq):
-        K, activation_type, stream_id, inference, logits_dtype = ctx.cfg
+        K, activation_type, stream_id, inference, logits_dtype, has_b1 = ctx.cfg
         if inference:
             raise RuntimeError("backward through an inference-mode MoE forward: z was not stored")
         x, router_w, w1, w2, b2, z, scores, indices, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
         T, E = x.size(0), router_w.size(0)
         dx, dw1, db1, dw2, db2, ds = _experts_backward(
-            dout, x, w1, w2, b2, z, scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id
+            dout, x, w1, w2, b2, z, scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id,
+            has_b1,
         )
         dlogits = torch.zeros(T, E, dtype=logits_dtype, device=x.device)
         _softmax_topk_bwd(dlogits, None, ds.view(T, K), scores, indices, K)

@@ -40,7 +40,7 @@ def _up_projection_backward(
     assert dz.size(1) == N1 and (db1 is None or (db1.shape == (E, N1) and db1.is_contiguous()))
     w_se, w_sr = expert_major_strides(w1, "w1")
     d_se, d_sr = expert_major_strides(dw1, "dw1") if dw1 is not None else (0, 0)
-    ws = _gemm_workspace(TK, E, x.device)
+    ws = _gemm_workspace(TK, E, x.device, stream_id)
     rc = _lib.lib().smoe_up_projection_backward(
         _lib.ptr(x),
         _lib.ptr(w1),
@@ -107,7 +107,7 @@ def _down_projection_backward(
     y1s = torch.empty(TK, I, dtype=z.dtype, device=z.device)
     ncols = _lib.lib().smoe_dz_partial_cols(I)
     ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
-    ws = _gemm_workspace(TK, E, z.device)
+    ws = _gemm_workspace(TK, E, z.device, stream_id)
     rc = _lib.lib().smoe_down_projection_backward(
         _lib.ptr(dout),
         _lib.ptr(z),

@@ -13,7 +13,17 @@ from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
 from ..utils import expert_major_strides
 
 
-def _gemm_workspace(TK: int, E: int, device) -> torch.Tensor:
+def _gemm_workspace(TK: int, E: int, device, stream_id: int) -> torch.Tensor:
+    """Tile-map scratch of one grouped-GEMM launch.  It comes from PyTorch's caching allocator, which orders its reuse
+    on the CURRENT stream, and the routing / combine kernels around the GEMM run on the current stream as well: a
+    GEMM launched on any other stream would race with both, so that is refused."""
+    current = _lib.current_stream_handle()
+    if stream_id != current:
+        raise RuntimeError(
+            f"grouped GEMM asked to run on stream {stream_id:#x} while PyTorch's current stream is {current:#x}: pass "
+            "torch.cuda.current_stream().cuda_stream (a MoE module keeps the stream it was constructed under in "
+            "`.stream_id`; set it again when calling the module under another stream)"
+        )
     n = _lib.lib().smoe_gemm_workspace_bytes(TK, E)
     return torch.empty(max(n, 16), dtype=torch.uint8, device=device)
 
@@ -86,7 +96,7 @@ def _up_projection_forward(
     assert x.is_contiguous() and y1.is_contiguous() and (z is None or z.is_contiguous())
     assert b1 is None or (b1.shape == (E, N1) and b1.is_contiguous())
     s_e, s_row = expert_major_strides(w1, "w1")
-    ws = _gemm_workspace(TK, E, x.device)
+    ws = _gemm_workspace(TK, E, x.device, stream_id)
     rc = _lib.lib().smoe_up_projection_forward(
         _lib.ptr(x),
         _lib.ptr(w1),
@@ -131,7 +141,7 @@ def _down_projection_forward(
     assert y1.is_contiguous() and y2.is_contiguous()
     assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous())
     s_e, s_row = expert_major_strides(w2, "w2")
-    ws = _gemm_workspace(TK, E, y1.device)
+    ws = _gemm_workspace(TK, E, y1.device, stream_id)
     rc = _lib.lib().smoe_down_projection_forward(
         _lib.ptr(y1),
         _lib.ptr(w2),

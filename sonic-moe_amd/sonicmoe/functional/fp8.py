@@ -8,6 +8,7 @@ backward pass is the bf16 one.
 
 from __future__ import annotations
 
+import weakref
 from contextlib import contextmanager
 
 import torch
@@ -58,8 +59,12 @@ def mx_quantize(t: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return q, scales
 
 
-# quantised copies of expert weights, valid while the parameter has not been written to (its version counter is
-# unchanged): inference and repeated forwards quantise a weight once, a training step re-quantises after the optimizer
+# Quantised copies of expert weights, reused while the tensor that owns the storage is alive and has not been written
+# to (same object, same version counter): inference and repeated forwards quantise a weight once, a training step
+# re-quantises after the optimizer.  An entry holds only a weak reference to that tensor and is dropped with it, so a
+# new parameter that lands at a freed parameter's address never meets the old one's entry.  Weights that have to be
+# copied into (E, out, in) order first are never cached: the copy is a fresh tensor every call.  Writes that bypass
+# the version counter (`param.data.copy_()`, raw pointers) are not seen; use cache_quantized_weights(False) there.
 _WEIGHT_CACHE: dict[tuple, tuple] = {}
 _WEIGHT_CACHE_MAX = 8
 _CACHE_WEIGHTS = True
@@ -78,19 +83,21 @@ def cache_quantized_weights(enable: bool = True):
 def quantize_expert_weight(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """w_view is the (out, in, E) permuted view of an (E, out, in) parameter; quantised along `in`."""
     w = w_view.permute(2, 0, 1)
-    if not w.is_contiguous():
+    aliases_caller = w.is_contiguous()
+    if not aliases_caller:
         w = w.contiguous()
     E, N, K = w.shape
-    if not _CACHE_WEIGHTS or torch.compiler.is_compiling():
+    if not aliases_caller or not _CACHE_WEIGHTS or torch.compiler.is_compiling():
         return mx_quantize(w.detach().reshape(E * N, K))
-    key = (w.data_ptr(), tuple(w.shape), w.device.index)
+    owner = w_view._base if w_view._base is not None else w_view  # the tensor whose version counter sees every write
+    key = (id(owner), w.data_ptr(), tuple(w.shape), w.device.index)
     hit = _WEIGHT_CACHE.get(key)
-    if hit is not None and hit[0] == w._version:
-        return hit[1], hit[2]
+    if hit is not None and hit[0]() is owner and hit[1] == owner._version:
+        return hit[2], hit[3]
     q, scales = mx_quantize(w.detach().reshape(E * N, K))
     if len(_WEIGHT_CACHE) >= _WEIGHT_CACHE_MAX:
         _WEIGHT_CACHE.pop(next(iter(_WEIGHT_CACHE)))
-    _WEIGHT_CACHE[key] = (w._version, q, scales)
+    _WEIGHT_CACHE[key] = (weakref.ref(owner, lambda _ref, k=key: _WEIGHT_CACHE.pop(k, None)), owner._version, q, scales)
     return q, scales
 
 
@@ -124,7 +131,7 @@ def _up_projection_forward_fp8(
     N1 = 2 * I if is_glu_activation else I
     assert w1q.shape == (E * N1, H) and x_scales.shape == (H // 128, T) and w1_scales.shape == (H // 128, E * N1)
     assert z is None or (z.shape == (TK, N1) and z.is_contiguous())
-    ws = _gemm_workspace(TK, E, xq.device)
+    ws = _gemm_workspace(TK, E, xq.device, stream_id)
     rc = _lib.lib().smoe_up_projection_forward_fp8(
         _lib.ptr(xq),
         _lib.ptr(x_scales),
@@ -168,7 +175,7 @@ def _down_projection_forward_fp8(
     TK, I = y1q.shape
     H = y2.size(1)
     assert w2q.shape == (E * H, I) and y1_scales.shape == (I // 128, TK) and w2_scales.shape == (I // 128, E * H)
-    ws = _gemm_workspace(TK, E, y1q.device)
+    ws = _gemm_workspace(TK, E, y1q.device, stream_id)
     rc = _lib.lib().smoe_down_projection_forward_fp8(
         _lib.ptr(y1q),
         _lib.ptr(y1_scales),

@@ -20,3 +20,19 @@ def dev():
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     return torch.device("cuda:0")
+
+
+@pytest.fixture
+def tuning():
+    """Set kernel-selection knobs of the HIP library for one test: tuning(name, value); defaults are restored after."""
+    from sonicmoe import _lib
+
+    touched = []
+
+    def set_knob(name, value):
+        _lib.set_tuning(name, value)
+        touched.append(name)
+
+    yield set_knob
+    for name in touched:
+        _lib.set_tuning(name, -1)

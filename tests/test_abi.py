@@ -75,6 +75,26 @@ def test_argument_checks_return_status_codes(lib):
     assert lib.smoe_dz_partial_cols(1024) >= 4
 
 
+def test_misaligned_operands_are_rejected(lib):
+    buf = ctypes.create_string_buffer(256)
+    base = ctypes.addressof(buf)
+    base += (-base) % 16
+    p, q = ctypes.c_void_p(base), ctypes.c_void_p(base + 2)
+    # a weight pointer that is not 16-byte aligned, then a row stride that is not a multiple of 8 elements
+    assert lib.smoe_up_projection_forward(p, q, 64, 64, None, p, p, p, p, 4, 8, 64, 64, 2, 0, p, 1 << 20, None) == 2
+    assert b"16-byte aligned" in lib.smoe_last_error()
+    assert lib.smoe_down_projection_forward(p, p, 64 * 64, 68, None, p, p, 8, 64, 64, 2, p, 1 << 20, None) == 2
+    assert b"multiples of 8" in lib.smoe_last_error()
+
+
+def test_tuning_knobs(lib):
+    assert lib.smoe_set_tuning(b"no_such_knob", 1) == 1
+    assert b"unknown knob" in lib.smoe_last_error()
+    assert lib.smoe_set_tuning(b"varlen_k_tile_order", 7) == 1
+    assert lib.smoe_set_tuning(b"gemm_stream", 0) == 0
+    assert lib.smoe_set_tuning(b"gemm_stream", -1) == 0  # back to the default
+
+
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from sonicmoe import _lib
 

@@ -152,3 +152,44 @@ def test_quantised_weight_cache_follows_parameter_updates(dev):
     assert torch.equal(a, b)
     assert torch.equal(c, d)
     assert rel_l2(c, 2.0 * a.float()) < 1e-2
+
+
+def test_quantised_weight_cache_is_not_fooled_by_address_reuse(dev):
+    """A module is freed and another of the same shape is built: its parameters may land at the freed addresses with
+    the same version counter, and must not meet the first module's quantised weights."""
+    import gc
+
+    from sonicmoe import MoE, enable_fp8_forward
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional.fp8 import cache_quantized_weights
+
+    x = torch.randn(512, 256, device=dev).to(torch.bfloat16)
+    outs = []
+    for seed in (11, 12):
+        torch.manual_seed(seed)
+        moe = MoE(8, 2, 256, 128, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+        with torch.no_grad(), enable_fp8_forward():
+            cached, _ = moe(x)
+            with cache_quantized_weights(False):
+                fresh, _ = moe(x)
+        assert torch.equal(cached, fresh), seed
+        outs.append(cached)
+        del moe
+        gc.collect()
+    assert not torch.equal(outs[0], outs[1])
+
+
+def test_weights_in_another_physical_layout_are_requantised_every_call(dev):
+    """Expert weights stored physically as (out, in, E) have to be copied into (E, out, in) order before quantising:
+    the copy is a new tensor every call and must never be served from the cache after an in-place update."""
+    from sonicmoe.functional import fp8
+
+    E, N, K = 4, 128, 256
+    g = torch.Generator().manual_seed(21)
+    w_phys = torch.randn(N, K, E, generator=g).to(torch.bfloat16).to(dev)   # the (out, in, E) "view" IS the storage
+    q0, s0 = fp8.quantize_expert_weight(w_phys)
+    w_phys.mul_(3.0)
+    q1, s1 = fp8.quantize_expert_weight(w_phys)
+    q_ref, s_ref = fp8.mx_quantize(w_phys.permute(2, 0, 1).contiguous().reshape(E * N, K))
+    assert torch.equal(q1, q_ref) and torch.equal(s1, s_ref)
+    assert not (torch.equal(q0, q1) and torch.equal(s0, s1))

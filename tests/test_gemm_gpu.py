@@ -126,10 +126,10 @@ STREAM_SHAPES = [
 
 @pytest.mark.parametrize("grid", [8, 24])
 @pytest.mark.parametrize("T,H,I,E,K,skew,empty", STREAM_SHAPES)
-def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
+def test_tile_streams(dev, tuning, grid, T, H, I, E, K, skew, empty):
     """The grouped GEMMs whose workgroups walk through several tiles each: few workgroups (8 = one per XCD, 24) force
     long streams on small problems, so tile switches, the parked epilogue and the last tile of a stream are all hit."""
-    monkeypatch.setenv("SMOE_GEMM_STREAM_GRID", str(grid))
+    tuning("gemm_stream_grid", grid)
     fwd, bwd = _ops()
     _, w1, w2 = make_weights(E, H, I, dev, seed=T + 20)
     b1 = (torch.randn(E, 2 * I, generator=torch.Generator().manual_seed(T + 23)) * 0.5).to(torch.bfloat16).to(dev)
@@ -176,18 +176,17 @@ def test_tile_streams(dev, monkeypatch, grid, T, H, I, E, K, skew, empty):
         assert bool((dw2[..., e] == 0).all())
 
     # the same results from the one-tile-per-workgroup launch order (many workgroups, one tile each)
-    monkeypatch.setenv("SMOE_GEMM_STREAM_GRID", "1000000")
+    tuning("gemm_stream_grid", 1000000)
     z1 = torch.empty_like(z)
     y11 = torch.empty_like(y1)
     fwd._up_projection_forward(x, w1.permute(1, 2, 0), z1, y11, b1, off, None, gidx, stream, "swiglu", True, False)
     assert torch.equal(z1, z) and torch.equal(y11, y1)
 
 
-@pytest.mark.parametrize("knob,value", [("SMOE_GEMM_STREAM", "0"), ("SMOE_VARLEN_K_TILE_ORDER", "0"),
-                                        ("SMOE_VARLEN_K_TILE_ORDER", "1"), ("SMOE_VARLEN_K_TILES", "1"),
-                                        ("SMOE_VARLEN_K_TILES", "2"), ("SMOE_VARLEN_K_TILES", "3")])
-def test_kernel_selection_knobs(dev, monkeypatch, knob, value):
-    """The alternative kernels / tile orders an environment variable selects give the same results as the defaults
+@pytest.mark.parametrize("knob,value", [("gemm_stream", 0), ("varlen_k_tile_order", 0), ("varlen_k_tile_order", 1),
+                                        ("varlen_k_tiles", 1), ("varlen_k_tiles", 2), ("varlen_k_tiles", 3)])
+def test_kernel_selection_knobs(dev, tuning, knob, value):
+    """The alternative kernels / tile orders a tuning knob selects give the same results as the defaults
     (bit-identical: the arithmetic of a tile does not depend on who computes it or when)."""
     fwd, bwd = _ops()
     T, H, I, E, K = 4096, 1024, 512, 32, 8
@@ -212,7 +211,7 @@ def test_kernel_selection_knobs(dev, monkeypatch, knob, value):
         return z, y1, y2, dw1, dxe
 
     base = run()
-    monkeypatch.setenv(knob, value)
+    tuning(knob, value)
     other = run()
     for name, a, b in zip(["z", "y1", "y2", "dw1", "dx_expanded"], base, other):
         assert torch.equal(a, b), name

@@ -200,6 +200,27 @@ def test_torch_compile_fullgraph(dev):
         assert rel_l2(a, b) < 5e-3  # dx: the compiled graph fuses the two dx contributions before the bf16 rounding
 
 
+def test_module_on_another_stream(dev):
+    """The grouped GEMMs take an explicit stream while the routing / combine kernels and the allocator follow PyTorch's
+    current stream: a mismatch is refused instead of racing; with `.stream_id` set to the current stream the module
+    gives the same result as on the default stream."""
+    moe, x, dy = _build(dev, 1024, 512, 256, 8, 2)
+    with torch.no_grad():
+        ref, _ = moe(x)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with pytest.raises(RuntimeError, match="current stream"):
+            with torch.no_grad():
+                moe(x)
+        constructed_under, moe.stream_id = moe.stream_id, side.cuda_stream
+        with torch.no_grad():
+            out, _ = moe(x)
+        moe.stream_id = constructed_under
+    side.synchronize()
+    assert torch.equal(out, ref)
+
+
 def test_empty_batch(dev):
     """Zero tokens: every operator accepts empty tensors; the weight gradients are zeros."""
     from sonicmoe import MoE

@@ -169,3 +169,63 @@ def test_token_rounding_invariants_and_product_router(mode):
     np.testing.assert_array_equal(t2.numpy(), tok)
     np.testing.assert_array_equal(e2.numpy(), exp)
     np.testing.assert_allclose(s2.numpy(), sc, rtol=1e-6)
+
+
+@pytest.mark.parametrize("mode", ["nr", "up", "down"])
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_token_rounding_keeps_the_best_ranked_tokens(mode, seed):
+    """Independent pin of the selection inside a class (a router that dropped an expert's BEST picks instead of its
+    worst, or padded with its worst non-picks, passes every count / containment invariant above): with the ranking
+    value worked out here from its definition in plain Python (a pick ranks by its renormalised probability, a
+    non-pick by probability - 1: benchmarks/moe-token-rounding.py:158-164 of the reference), every kept token of an
+    expert outranks every dropped one, the kept set is exactly the brute-force top-`target`, picks that were dropped are
+    the expert's lowest-ranked picks, and non-picks that were added are its highest-ranked non-picks."""
+    T, E, K, tile = 40, 6, 2, 8
+    g = torch.Generator().manual_seed(100 + seed)
+    probs = torch.softmax(torch.randn(T, E, generator=g) * 1.5, dim=-1, dtype=torch.float32).numpy()
+    sc, tok, exp, target = TR.token_choice_rounding(probs, K, tile, mode)
+
+    rank = [[0.0] * E for _ in range(T)]
+    is_pick = [[False] * E for _ in range(T)]
+    for t in range(T):
+        best = sorted(range(E), key=lambda e: (-float(probs[t, e]), e))[:K]
+        total = np.float32(0)
+        for e in best:
+            total = np.float32(total + probs[t, e])
+        for e in range(E):
+            if e in best:
+                rank[t][e] = float(np.float32(probs[t, e] / total))
+                is_pick[t][e] = True
+            else:
+                rank[t][e] = float(np.float32(probs[t, e] - np.float32(1.0)))
+    kept = {e: set() for e in range(E)}
+    for t, e in zip(tok.tolist(), exp.tolist()):
+        kept[e].add(t)
+    dropped_some = added_some = False
+    for e in range(E):
+        n = int(target[e])
+        assert len(kept[e]) == n
+        brute = set(sorted(range(T), key=lambda t: (-rank[t][e], t))[:n])
+        assert kept[e] == brute
+        out = set(range(T)) - kept[e]
+        if kept[e] and out:
+            assert min(rank[t][e] for t in kept[e]) >= max(rank[t][e] for t in out)
+        picks = {t for t in range(T) if is_pick[t][e]}
+        lost, gained = picks - kept[e], kept[e] - picks
+        if lost:  # what was dropped are the lowest-ranked picks
+            dropped_some = True
+            assert max(rank[t][e] for t in lost) <= min(rank[t][e] for t in picks & kept[e]) if picks & kept[e] else True
+        if gained:  # what was added are the highest-ranked non-picks
+            added_some = True
+            others = set(range(T)) - picks - kept[e]
+            assert not others or min(rank[t][e] for t in gained) >= max(rank[t][e] for t in others)
+    if mode == "up":
+        assert added_some and not dropped_some
+    elif mode == "down":
+        assert dropped_some and not added_some
+    else:
+        assert dropped_some or added_some
+    # the scores handed on are the renormalised probabilities for picks and the plain probabilities for the rest
+    for s_, t, e in zip(sc.tolist(), tok.tolist(), exp.tolist()):
+        want = rank[t][e] if is_pick[t][e] else float(probs[t, e])
+        assert abs(s_ - want) <= 1e-6
