@@ -37,6 +37,26 @@ SMOE_DEV void load16_to_lds(const void* g, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(g), "s"(lds_wave_base) : "memory");
 }
 
+// The same through a buffer resource: source = resource base + per-lane byte offset `voff` + wave-uniform byte offset
+// `soff`.  The address arithmetic of a stage is then one scalar add (soff moves along the contraction) instead of a
+// 64-bit vector add per load, and a lane keeps one 32-bit offset per load instead of a pointer.
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+SMOE_DEV i32x4 make_buffer_resource(const void* base) {
+  const uint64_t b = (uint64_t)base;
+  i32x4 r;
+  r[0] = __builtin_amdgcn_readfirstlane((uint32_t)b);
+  r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32) & 0xffffu);  // 48-bit base, stride 0 (raw buffer)
+  r[2] = -1;                                                                // no range limit: the kernels clamp rows
+  r[3] = 0x00020000;                                                        // 32-bit untyped data
+  return r;
+}
+SMOE_DEV void buffer_load16_to_lds(i32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_wave_base)
+               : "memory");
+}
+
 // piece swizzle of a K-major stage with BK_ of the contraction per row (BK_*2/16 pieces): chosen so that the 16 lanes
 // of a ds_read_b128 quarter-wave (16 consecutive rows, same piece) hit 16 different 16-byte bank groups
 template <int BK_>

@@ -193,6 +193,17 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       }
       return;
     }
+    // the expert's last, ragged stage: rows past its end read the zero page.  The index array goes on behind the
+    // expert (the next expert's rows) up to total_rows, so the run is still ONE wide load wherever it stays inside
+    // the array; entries past the expert's end are discarded.
+    if constexpr (C::R_GATHER || C::S_GATHER) {
+      if ((int64_t)m0 + RPW <= p.total_rows) {
+        const idx_run run = *(const_run_ptr)(gidx + m0);
+#pragma unroll
+        for (int j = 0; j < RPW; j++) dst[j] = m0 + j < row_end ? run[j] : -1;
+        return;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < RPW; j++) {
       const int m = m0 + j;
@@ -351,6 +362,17 @@ __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKPara
         for (int j = 0; j < RPW; j++) dst[j] = m0 + j;
       }
       return;
+    }
+    // the expert's last, ragged stage: rows past its end read the zero page.  The index array goes on behind the
+    // expert (the next expert's rows) up to total_rows, so the run is still ONE wide load wherever it stays inside
+    // the array; entries past the expert's end are discarded.
+    if constexpr (C::R_GATHER || C::S_GATHER) {
+      if ((int64_t)m0 + RPW <= p.total_rows) {
+        const idx_run run = *(const_run_ptr)(gidx + m0);
+#pragma unroll
+        for (int j = 0; j < RPW; j++) dst[j] = m0 + j < row_end ? run[j] : -1;
+        return;
+      }
     }
 #pragma unroll
     for (int j = 0; j < RPW; j++) {

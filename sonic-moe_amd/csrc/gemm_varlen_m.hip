@@ -15,6 +15,7 @@ struct VarlenMParams {
   const uint16_t* P;
   int64_t p_stride;
   const int32_t* gidx;  // nullable: P rows are the grouped rows themselves
+  int64_t p_rows;       // rows of P when gathered (the range of gidx)
   const uint16_t* Q;
   int64_t q_stride_e, q_stride_row;
   const int32_t* off;
@@ -392,37 +393,44 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     for (int i = 0; i < C::P_INSTR; i++) {
       int m = t.row0 + (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
       m = m < t.row_end ? m : t.row_end - 1;
-      rows[i] = p.gidx ? p.gidx[m] : m;
+      rows[i] = p.gidx ? p.gidx[m] : m - t.row0;
     }
   };
-  const uint16_t* p_src[C::P_INSTR];
-  const uint16_t* q_src[C::Q_INSTR];
-  const int64_t q_step = C::QMN ? (int64_t)BK * p.q_stride_row : (int64_t)BK;
-  auto point_p = [&](const int(&rows)[C::P_INSTR]) {
+  // Operands are fetched through buffer resources: a lane keeps one 32-bit byte offset per load (fixed for a tile),
+  // the position along the contraction is a wave-uniform offset.  The token operand's resource starts at the tensor
+  // (gathered rows: row * stride has to fit 32 bits, checked on the host) or at the tile's first row (rows in place);
+  // the weight operand's resource starts at the tile's expert.
+  uint32_t p_voff[C::P_INSTR], q_voff[C::Q_INSTR];
+  i32x4 p_rsrc = make_buffer_resource(p.P), q_rsrc = make_buffer_resource(p.Q);
+  const uint32_t p_row_bytes = (uint32_t)p.p_stride * 2u, q_row_bytes = (uint32_t)p.q_stride_row * 2u;
+  const uint32_t q_step = C::QMN ? (uint32_t)BK * q_row_bytes : (uint32_t)BK * 2u;
+  // rows: token indices (gathered) or grouped rows relative to the tile's first row
+  auto point_p = [&](const int(&rows)[C::P_INSTR], const Tile& t) {
     const int ln = opaque_lane();
+    if (!p.gidx) p_rsrc = make_buffer_resource(p.P + (int64_t)t.row0 * p.p_stride);
 #pragma unroll
     for (int i = 0; i < C::P_INSTR; i++) {
       const int r = (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
-      p_src[i] = p.P + (int64_t)rows[i] * p.p_stride + (((ln % C::KPR) ^ kswz<BK>(r)) << 3);
+      p_voff[i] = (uint32_t)rows[i] * p_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK>(r)) << 4);
     }
   };
   auto point_q = [&](const Tile& t) {
     const int ln = opaque_lane();
-    const uint16_t* qe = p.Q + (int64_t)t.e * p.q_stride_e;
+    q_rsrc = make_buffer_resource(p.Q + (int64_t)t.e * p.q_stride_e);
 #pragma unroll
     for (int i = 0; i < C::Q_INSTR; i++) {
       if constexpr (!C::QMN) {
         const int r = (wave * C::Q_INSTR + i) * C::KRPI + ln / C::KPR;
         int n = t.n0 + r;
         n = n < p.N ? n : p.N - 1;
-        q_src[i] = qe + (int64_t)n * p.q_stride_row + (((ln % C::KPR) ^ kswz<BK>(r)) << 3);
+        q_voff[i] = (uint32_t)n * q_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK>(r)) << 4);
       } else {
         const int kl = (wave * C::Q_INSTR + i) * C::RPI + ln / C::LPR;
         const int phys16 = ln % C::LPR;
         const int log32 = (phys16 >> 1) ^ mnswz(kl);
         int n = t.n0 + ((log32 << 1) | (phys16 & 1)) * 8;
         n = n <= p.N - 8 ? n : p.N - 8;
-        q_src[i] = qe + (int64_t)kl * p.q_stride_row + n;
+        q_voff[i] = (uint32_t)kl * q_row_bytes + (uint32_t)n * 2u;
       }
     }
   };
@@ -430,7 +438,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
   {
     int rows_cur[C::P_INSTR];
     token_rows(cur, rows_cur);
-    point_p(rows_cur);
+    point_p(rows_cur, cur);
     point_q(cur);
     token_rows(nxt, rows_next);
   }
@@ -448,18 +456,18 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
   int p_stage = 0, q_stage = 0;  // stages issued to each stream for the tile it is on
   auto issue_p = [&](int slot, auto i_c) {
     constexpr int i = decltype(i_c)::value;
-    load16_to_lds(p_src[i], smem_base + slot * C::P_STAGE + (wave * C::P_INSTR + i) * 1024);
-    p_src[i] += BK;
+    buffer_load16_to_lds(p_rsrc, p_voff[i], (uint32_t)p_stage * (BK * 2u),
+                         smem_base + slot * C::P_STAGE + (wave * C::P_INSTR + i) * 1024);
   };
   auto issue_q = [&](int slot, auto j_c) {
     constexpr int j = decltype(j_c)::value;
-    load16_to_lds(q_src[j], smem_base + Q_RING + slot * C::Q_STAGE + (wave * C::Q_INSTR + j) * 1024);
-    q_src[j] += q_step;
+    buffer_load16_to_lds(q_rsrc, q_voff[j], (uint32_t)q_stage * q_step,
+                         smem_base + Q_RING + slot * C::Q_STAGE + (wave * C::Q_INSTR + j) * 1024);
   };
   auto issued_p = [&]() {
     if (++p_stage == S_total) {
       p_stage = 0;
-      point_p(rows_next);
+      point_p(rows_next, nxt);
     }
   };
   auto issued_q = [&]() {
@@ -536,7 +544,9 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
   if constexpr (ROLE != ROLE_DZ) {
     const Tuning& tune = tuning();
-    if (tune.gemm_stream && p.Kdim >= 3 * C::BK) {
+    // the tile-stream kernel addresses a gathered token operand with 32-bit byte offsets from the tensor's start
+    const bool offsets_fit = p.gidx == nullptr || p.p_rows * p.p_stride * 2 <= 0xffffffffll;
+    if (tune.gemm_stream && p.Kdim >= 3 * C::BK && offsets_fit) {
       static LdsLimitOnce lds_limit_stream;
       auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
       const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
@@ -624,6 +634,7 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
   p.P = (const uint16_t*)x;
   p.p_stride = H;
   p.gidx = x_gather_idx;
+  p.p_rows = T;
   p.Q = (const uint16_t*)w1;
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
@@ -675,6 +686,7 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.P = (const uint16_t*)dout;
   p.p_stride = H;
   p.gidx = gidx;
+  p.p_rows = TK;  // an upper bound of the number of dout rows
   p.Q = (const uint16_t*)w2;  // W2[e] is (H, I): k = h rows, n = i contiguous
   p.q_stride_e = w2_stride_e;
   p.q_stride_row = w2_stride_row;
@@ -690,6 +702,11 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.scores = scores;
   p.sidx = sidx;
   p.ds_partial = ds_partial;
+  if (tuning().experiment & 2) {  // EXPERIMENT: the dz GEMM alone as a tile stream (dy1 written to y1s)
+    p.out0 = (uint16_t*)y1s;
+    p.out0_stride = I;
+    return launch_varlen_m<TileCfg<true>, ROLE_PLAIN, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
+  }
   return launch_by_activation<true, ROLE_DZ>(activation, p, off, workspace, TK, E, st);
 }
 
