@@ -66,10 +66,10 @@ SMOE_DEV int kswz(int row) {
 }
 
 // 32-byte-group swizzle of an MN-major stage: group g of contraction row k sits at g ^ mnswz(k).  A transpose load
-// makes the 32 lanes of a half-wave read 4 consecutive k-rows x 2 neighbouring groups; (k & 3) << 1 moves the four rows
-// to four different even offsets and leaves bit 0 to tell the two groups apart, so the eight 32-byte pieces fall into
-// the eight different 32-byte bank groups of the 64 banks.
-SMOE_DEV int mnswz(int k) { return (k & 3) << 1; }
+// makes the 32 lanes of a half-wave read eight k-rows (k & 3 = 0..3, twice) of one or two neighbouring groups; the
+// swizzle sends the eight 32-byte pieces to the eight different 32-byte bank groups of the 64 banks for both fragment
+// shapes (32-row fragments: rows k..k+3 of two neighbouring groups; 16-row fragments: rows k..k+3 and k+8..k+11 of one).
+SMOE_DEV int mnswz(int k) { return ((k & 3) << 1) ^ ((k >> 3) & 1); }
 
 SMOE_DEV bf16x8 lds_read_b128(const char* p) { return *(const bf16x8*)p; }
 
@@ -95,10 +95,6 @@ SMOE_DEV void static_for(F&& f) {
   static_for_impl<0, N>(f);
 }
 
-SMOE_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-}
-
 // s_waitcnt vmcnt(N) lgkmcnt(0): at most N of this wave's vector-memory operations (oldest first) may still be
 // outstanding, and all of its LDS operations have completed
 template <int N>
@@ -120,23 +116,103 @@ SMOE_DEV void lds_barrier() {
   asm volatile("" ::: "memory");
 }
 
+// ---- matrix instruction policies ---------------------------------------------------------------------------------
+// A main loop works in STEPS per LDS stage.  A step issues NQ x NP matrix instructions on fragments that the previous
+// step read from LDS: two register sets of weight-side (Q) fragments and two of token-side (P) fragments alternate.
+//   Bf16Mma32  v_mfma_f32_32x32x16_bf16: a step is one k-slice of 16; it reads all of the wave's fragments.
+//   Bf16Mma16  v_mfma_f32_16x16x32_bf16: a k-slice is 32 deep and is worked through in PH = 2 steps over the two halves
+//              of the wave's token fragments; the Q fragments are read on the even step and serve both.  Same bytes
+//              from LDS per FLOP, four times the instructions, and markedly less power per FLOP on random data (a
+//              register-only loop of these instructions sustains 2.07 PFLOP/s under the chip's power limit where
+//              the 32x32x16 form sustains 1.8), which is what bounds these kernels.
+// Accumulator layout (operands are issued as D[n][m] += Q[n][k] P[k][m]): lane l owns token column m = l % FR of the
+// fragment and, per group of four registers, four consecutive features.
+struct Bf16Mma32 {
+  typedef bf16x8 Frag;
+  typedef f32x16 Acc;
+  static constexpr int FR = 32, KSTEP = 16, PH = 1, ACC_REGS = 16;
+  static constexpr int qset(int step) { return step & 1; }
+  static constexpr int phalf(int) { return 0; }
+  static constexpr bool reads_q(int) { return true; }
+  static constexpr int kslice(int step) { return step; }
+  static __device__ __forceinline__ Acc run(const Frag& q, const Frag& p, Acc c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(q, p, c, 0, 0, 0);
+  }
+};
+struct Bf16Mma16 {
+  typedef bf16x8 Frag;
+  typedef f32x4 Acc;
+  static constexpr int FR = 16, KSTEP = 32, PH = 2, ACC_REGS = 4;
+  static constexpr int qset(int step) { return (step >> 1) & 1; }
+  static constexpr int phalf(int step) { return step & 1; }
+  static constexpr bool reads_q(int step) { return (step & 1) == 0; }
+  static constexpr int kslice(int step) { return step >> 1; }
+  static __device__ __forceinline__ Acc run(const Frag& q, const Frag& p, Acc c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(q, p, c, 0, 0, 0);
+  }
+};
+// the bf16 kernels' instruction
+typedef Bf16Mma16 Bf16Mma;
+
+template <class Mma, int NQ, int NPT>
+SMOE_DEV void clear_accumulators(typename Mma::Acc (&acc)[NQ][NPT]) {
+#pragma unroll
+  for (int q = 0; q < NQ; q++)
+#pragma unroll
+    for (int pp = 0; pp < NPT; pp++)
+#pragma unroll
+      for (int r = 0; r < Mma::ACC_REGS; r++) acc[q][pp][r] = 0.f;
+}
+
+// The matrix instructions of one step, with the LDS reads issued just before them (for the NEXT step) slotted in
+// RPM per instruction, starting after the first so that the wait in front of it covers only reads of the previous step.
+template <class Mma, int NQ, int NP, int NREADS, int RPM, int STEP, bool FRESH>
+SMOE_DEV void mma_step(typename Mma::Acc (&acc)[NQ][NP * Mma::PH], typename Mma::Frag (&qf)[2][NQ],
+                       typename Mma::Frag (&pf)[2][NP]) {
+  constexpr int qs = Mma::qset(STEP), ps = STEP & 1, ph = Mma::phalf(STEP), NM = NQ * NP;
+  typename Mma::Acc zero;
+#pragma unroll
+  for (int r = 0; r < Mma::ACC_REGS; r++) zero[r] = 0.f;
+#pragma unroll
+  for (int q = 0; q < NQ; q++)
+#pragma unroll
+    for (int pp = 0; pp < NP; pp++)
+      acc[q][ph * NP + pp] = Mma::run(qf[qs][q], pf[ps][pp], FRESH ? zero : acc[q][ph * NP + pp]);
+  constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
+#pragma unroll
+  for (int i = 0; i < NR; i++) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+}
+
+// The last step of a stage whose ring slots are refilled: `deal(i)` is called behind the i-th matrix instruction and
+// issues the refill's load instructions that fall there, so they are dealt out between the matrix instructions instead
+// of standing in front of them (the matrix pipe does not idle while every wave issues its loads behind the barrier).
+template <class Mma, int NQ, int NP, int STEP, class Deal>
+SMOE_DEV void mma_step_refill(typename Mma::Acc (&acc)[NQ][NP * Mma::PH], typename Mma::Frag (&qf)[2][NQ],
+                              typename Mma::Frag (&pf)[2][NP], Deal&& deal) {
+  constexpr int qs = Mma::qset(STEP), ps = STEP & 1, ph = Mma::phalf(STEP), NM = NQ * NP;
+  static_for<NM>([&](auto i_c) {
+    constexpr int i = decltype(i_c)::value;
+    acc[i / NP][ph * NP + i % NP] = Mma::run(qf[qs][i / NP], pf[ps][i % NP], acc[i / NP][ph * NP + i % NP]);
+    deal(i_c);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+}
+
 // ---- software-pipelined main loop ------------------------------------------------------------------------------
-// LDS holds a ring of NSTAGE stages; a stage covers SLICES MFMA k-slices (16 each) of the contraction.  One stage is
-// consumed while up to NSTAGE-1 are in flight from L2/HBM.  Per stage:
-//   slices 0..SLICES-2: read the fragments of the next slice from LDS while the MFMAs of the current slice run;
-//   last slice: wait until this wave's pieces of the NEXT stage have landed (vmcnt leaves the younger stages in
+// LDS holds a ring of NSTAGE stages; a stage is worked through in STEPS steps.  One stage is consumed while up to
+// NSTAGE-1 are in flight from L2/HBM.  Per stage:
+//   steps 0..STEPS-2: read the fragments of the next step from LDS while the matrix instructions of the current run;
+//   last step: wait until this wave's pieces of the NEXT stage have landed (vmcnt leaves the younger stages in
 //            flight), workgroup barrier (everyone's pieces landed; everyone drained the current stage), refill the
-//            current stage's slot with stage s+NSTAGE, read slice 0 of the next stage while the last MFMAs run.
+//            current stage's slot with stage s+NSTAGE, read step 0 of the next stage while the last instructions run.
 //   issue(buf, s, i)              start the i-th (compile-time index, 0 <= i < LPS) of this wave's direct-to-LDS loads of
 //                                 stage s into ring slot buf; called with i ascending, stages in order
-//   load(buf, s, ks, qf, pf)      read the fragments of slice ks of stage s from ring slot buf
-// MFMA operand fragment + instruction of the bf16 kernels; the fp8 kernels bring their own pair
-struct Bf16Mma {
-  typedef bf16x8 Frag;
-  static __device__ __forceinline__ f32x16 run(const Frag& q, const Frag& p, f32x16 c) { return mfma32(q, p, c); }
-};
-
-// RPM: LDS reads slotted in behind each of the first MFMAs of a slice
+//   load(buf, s, step, qf, pf)    read the fragments step `step` (a compile-time constant) needs from ring slot buf
+//                                 into the fragment sets handed in
 // The first stages of a main loop, issued on their own: a kernel that works through several tiles starts the next
 // tile's loads before the finished tile's epilogue and enters gemm_mainloop<..., PROLOGUE = false> behind it.
 template <int LPS, int NSTAGE, class Issue>
@@ -148,14 +224,14 @@ SMOE_DEV void gemm_mainloop_prologue(const int S, Issue&& issue) {
 // PROLOGUE = false: the first min(S, NSTAGE) stages have been issued by gemm_mainloop_prologue, possibly with other
 // vector-memory operations (an epilogue's stores) behind them: the first wait is then for everything, because loads
 // and stores may retire out of order and a counted wait could not tell which are left.
-template <int NQ, int NP, int NREADS, int LPS, int SLICES, int NSTAGE, class Mma = Bf16Mma, int RPM = 1,
+template <int NQ, int NP, int NREADS, int LPS, int STEPS, int NSTAGE, class Mma = Bf16Mma, int RPM = 1,
           bool PROLOGUE = true, class Issue, class Load>
-SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, Load&& load) {
+SMOE_DEV void gemm_mainloop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::PH], Issue&& issue, Load&& load) {
   if (S <= 0) return;
   static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
-  static_assert(SLICES % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 6, "unsupported pipeline shape");
+  static_assert(STEPS % 2 == 0 && NSTAGE >= 2 && NSTAGE <= 6, "unsupported pipeline shape");
   typename Mma::Frag qf[2][NQ], pf[2][NP];
-  constexpr int NM = NQ * NP;
+  constexpr int NM = NQ * NP, LAST = STEPS - 1;
   auto issue_all = [&](int buf, int s) { static_for<LPS>([&](auto i_c) { issue(buf, s, i_c); }); };
   const int pre = S < NSTAGE ? S : NSTAGE;
   if constexpr (PROLOGUE)
@@ -168,71 +244,53 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
     if constexpr (NSTAGE >= 3) if (younger == 1) { wait_vmem_upto<LPS>(); return; }
     wait_vmem_all();
   };
-  // the MFMAs of one slice; the LDS reads issued just before them (for the NEXT slice) are slotted in one per MFMA,
-  // starting after the first MFMA so that the wait in front of it covers only reads of the previous slice
-  auto slice_mfma = [&](auto cur_c) {
-    constexpr int cur = decltype(cur_c)::value;
-#pragma unroll
-    for (int q = 0; q < NQ; q++)
-#pragma unroll
-      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
-    constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
-#pragma unroll
-    for (int i = 0; i < NR; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  auto read_step = [&](int buf, int s, auto step_c) {
+    constexpr int step = decltype(step_c)::value;
+    load(buf, s, step_c, qf[Mma::qset(step)], pf[step & 1]);
   };
-  // the last slice of a stage whose ring slot is refilled: the refill's load instructions (address arithmetic, M0
-  // set-up, the load) are dealt out between the MFMAs instead of standing in front of them, so the matrix pipe does
-  // not idle while every wave of the SIMD issues its loads right after the barrier
-  auto slice_mfma_refill = [&](int buf, int s_new) {
-    static_for<NM>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
-      static_for<LPS>([&](auto j_c) {
-        constexpr int j = decltype(j_c)::value;
-        if constexpr (j * NM / LPS == i) issue(buf, s_new, j_c);
-      });
-      __builtin_amdgcn_sched_barrier(0);
+  auto inner_steps = [&](int buf, int s) {
+    static_for<STEPS - 1>([&](auto k_c) {
+      constexpr int k = decltype(k_c)::value;
+      read_step(buf, s, std::integral_constant<int, k + 1>{});
+      mma_step<Mma, NQ, NP, NREADS, RPM, k, false>(acc, qf, pf);
     });
   };
-  auto inner_slices = [&](int buf, int s) {
-    static_for<SLICES - 1>([&](auto ks_c) {
-      constexpr int ks = decltype(ks_c)::value;
-      load(buf, s, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
-      slice_mfma(std::integral_constant<int, (ks & 1)>{});
-    });
-  };
+  constexpr std::integral_constant<int, 0> step0{};
 
   if constexpr (PROLOGUE) wait_next_stage(pre - 1);
   else wait_vmem_all();
   lds_barrier();
-  load(0, 0, 0, qf[0], pf[0]);
+  read_step(0, 0, step0);
   int buf = 0;
   int s = 0;
   for (; s + NSTAGE < S; s++) {  // steady state: every stage boundary refills the slot it frees
-    inner_slices(buf, s);
+    inner_steps(buf, s);
     wait_next_stage(NSTAGE - 2);
     lds_barrier();
     const int next = buf + 1 == NSTAGE ? 0 : buf + 1;
-    load(next, s + 1, 0, qf[0], pf[0]);
+    read_step(next, s + 1, step0);
     __builtin_amdgcn_sched_barrier(0);
-    slice_mfma_refill(buf, s + NSTAGE);
+    const int s_new = s + NSTAGE;
+    mma_step_refill<Mma, NQ, NP, LAST>(acc, qf, pf, [&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      static_for<LPS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        if constexpr (j * NM / LPS == i) issue(buf, s_new, j_c);
+      });
+    });
     buf = next;
   }
   for (; s < S - 1; s++) {  // drain: nothing left to fetch
-    inner_slices(buf, s);
+    inner_steps(buf, s);
     const int younger = S - 2 - s < NSTAGE - 2 ? S - 2 - s : NSTAGE - 2;
     wait_next_stage(younger);
     lds_barrier();
     buf = buf + 1 == NSTAGE ? 0 : buf + 1;
-    load(buf, s + 1, 0, qf[0], pf[0]);
-    slice_mfma(std::integral_constant<int, 1>{});
+    read_step(buf, s + 1, step0);
+    mma_step<Mma, NQ, NP, NREADS, RPM, LAST, false>(acc, qf, pf);
   }
-  inner_slices(buf, S - 1);
-  slice_mfma(std::integral_constant<int, 1>{});
+  inner_steps(buf, S - 1);
+  mma_step<Mma, NQ, NP, NREADS, RPM, LAST, false>(acc, qf, pf);
 }
 
 // ---- main loop with an asymmetric ring -------------------------------------------------------------------------------
@@ -243,14 +301,15 @@ SMOE_DEV void gemm_mainloop(const int S, f32x16 (&acc)[NQ][NP], Issue&& issue, L
 // to come back within one.
 //   issue_p(slot, i) / issue_q(slot, j)   start the i-th / j-th load of this wave into that operand's ring slot; stages
 //                                          are issued in order, so the callee advances its own source pointers
-//   load(p_slot, q_slot, ks, qf, pf)      read the fragments of slice ks
-template <int NQ, int NP, int NREADS, int PI, int QI, int SLICES, class Mma = Bf16Mma, int RPM = 1, class IssueP,
+//   load(p_slot, q_slot, step, qf, pf)    read the fragments of step `step`
+template <int NQ, int NP, int NREADS, int PI, int QI, int STEPS, class Mma = Bf16Mma, int RPM = 1, class IssueP,
           class IssueQ, class Load>
-SMOE_DEV void gemm_mainloop_asym(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issue_p, IssueQ&& issue_q, Load&& load) {
+SMOE_DEV void gemm_mainloop_asym(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::PH], IssueP&& issue_p,
+                                 IssueQ&& issue_q, Load&& load) {
   if (S <= 0) return;
-  static_assert(SLICES % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
+  static_assert(STEPS % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
   typename Mma::Frag qf[2][NQ], pf[2][NP];
-  constexpr int NM = NQ * NP, LPS = PI + QI;
+  constexpr int NM = NQ * NP, LPS = PI + QI, LAST = STEPS - 1;
   auto all_p = [&](int slot) { static_for<PI>([&](auto i_c) { issue_p(slot, i_c); }); };
   auto all_q = [&](int slot) { static_for<QI>([&](auto j_c) { issue_q(slot, j_c); }); };
   all_p(0);
@@ -261,71 +320,57 @@ SMOE_DEV void gemm_mainloop_asym(const int S, f32x16 (&acc)[NQ][NP], IssueP&& is
   }
   if (S > 2) all_q(2);
 
-  auto slice_mfma = [&](auto cur_c) {
-    constexpr int cur = decltype(cur_c)::value;
-#pragma unroll
-    for (int q = 0; q < NQ; q++)
-#pragma unroll
-      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], acc[q][pp]);
-    constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
-#pragma unroll
-    for (int i = 0; i < NR; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  auto read_step = [&](int bp, int bq, auto step_c) {
+    constexpr int step = decltype(step_c)::value;
+    load(bp, bq, step_c, qf[Mma::qset(step)], pf[step & 1]);
   };
-  // last slice of a stage with the refill (P pieces first, then Q pieces) dealt out between its MFMAs
-  auto slice_mfma_refill = [&](int p_slot, int q_slot) {
-    static_for<NM>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
-      static_for<LPS>([&](auto j_c) {
-        constexpr int j = decltype(j_c)::value;
-        if constexpr (j * NM / LPS == i) {
-          if constexpr (j < PI) issue_p(p_slot, j_c);
-          else issue_q(q_slot, std::integral_constant<int, j - PI>{});
-        }
-      });
-      __builtin_amdgcn_sched_barrier(0);
+  auto inner_steps = [&](int bp, int bq) {
+    static_for<STEPS - 1>([&](auto k_c) {
+      constexpr int k = decltype(k_c)::value;
+      read_step(bp, bq, std::integral_constant<int, k + 1>{});
+      mma_step<Mma, NQ, NP, NREADS, RPM, k, false>(acc, qf, pf);
     });
   };
-  auto inner_slices = [&](int bp, int bq) {
-    static_for<SLICES - 1>([&](auto ks_c) {
-      constexpr int ks = decltype(ks_c)::value;
-      load(bp, bq, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
-      slice_mfma(std::integral_constant<int, (ks & 1)>{});
-    });
-  };
+  constexpr std::integral_constant<int, 0> step0{};
 
   if (S > 2) wait_vmem_upto<PI + 2 * QI>();  // stage 0 has landed; P1, Q1, Q2 may still be on their way
   else wait_vmem_all();
   lds_barrier();
-  load(0, 0, 0, qf[0], pf[0]);
+  read_step(0, 0, step0);
   int bp = 0, bq = 0, s = 0;
   for (; s + 3 < S; s++) {  // steady state: P(s+2) and Q(s+3) exist
-    inner_slices(bp, bq);
+    inner_steps(bp, bq);
     wait_vmem_upto<QI>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
     lds_barrier();
     const int np = bp ^ 1, nq = bq == 2 ? 0 : bq + 1;
-    load(np, nq, 0, qf[0], pf[0]);
+    read_step(np, nq, step0);
     __builtin_amdgcn_sched_barrier(0);
-    slice_mfma_refill(bp, bq);  // the slots stage s leaves behind
+    // the slots stage s leaves behind: P pieces first, then Q pieces
+    mma_step_refill<Mma, NQ, NP, LAST>(acc, qf, pf, [&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      static_for<LPS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        if constexpr (j * NM / LPS == i) {
+          if constexpr (j < PI) issue_p(bp, j_c);
+          else issue_q(bq, std::integral_constant<int, j - PI>{});
+        }
+      });
+    });
     bp = np;
     bq = nq;
   }
   for (; s < S - 1; s++) {  // drain: at most P(s+2) is left to request
-    inner_slices(bp, bq);
+    inner_steps(bp, bq);
     wait_vmem_all();
     lds_barrier();
     if (s + 2 < S) all_p(bp);
     bp ^= 1;
     bq = bq == 2 ? 0 : bq + 1;
-    load(bp, bq, 0, qf[0], pf[0]);
-    slice_mfma(std::integral_constant<int, 1>{});
+    read_step(bp, bq, step0);
+    mma_step<Mma, NQ, NP, NREADS, RPM, LAST, false>(acc, qf, pf);
   }
-  inner_slices(bp, bq);
-  slice_mfma(std::integral_constant<int, 1>{});
+  inner_steps(bp, bq);
+  mma_step<Mma, NQ, NP, NREADS, RPM, LAST, false>(acc, qf, pf);
 }
 
 
@@ -343,18 +388,20 @@ SMOE_DEV void gemm_mainloop_asym(const int S, f32x16 (&acc)[NQ][NP], IssueP&& is
 //                              tile_end (a wait for them anywhere else would also wait for the ring)
 //   tile_end(p_slot, q_slot)   epilogue of the finished tile; may use the two slots as scratch (every wave is past the
 //                              barrier behind the last stage); advances the caller's tile state and returns false if
-//                              the tile was the workgroup's last.  The accumulators need no clearing: the first slice
-//                              of every tile starts them from zero
+//                              the tile was the workgroup's last.  The accumulators need no clearing: the first
+//                              k-slice of every tile starts them from zero
 // Needs S >= 3 (stage 0 of the next tile is requested at the latest behind stage S-3 of the current one).  Stores and
 // loads share one counter and may retire out of order with respect to each other, so the first wait of a tile is for
 // everything; from then on only loads are outstanding and the counted waits are exact again.
-template <int NQ, int NP, int NREADS, int PI, int QI, int SLICES, class Mma = Bf16Mma, int RPM = 1, class IssueP,
+template <int NQ, int NP, int NREADS, int PI, int QI, int STEPS, class Mma = Bf16Mma, int RPM = 1, class IssueP,
           class IssueQ, class Load, class IssuedP, class IssuedQ, class First, class TileEnd>
-SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issue_p, IssueQ&& issue_q, Load&& load,
-                               IssuedP&& issued_p, IssuedQ&& issued_q, First&& first_boundary, TileEnd&& tile_end) {
-  static_assert(SLICES % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
+SMOE_DEV void gemm_stream_loop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::PH], IssueP&& issue_p,
+                               IssueQ&& issue_q, Load&& load, IssuedP&& issued_p, IssuedQ&& issued_q,
+                               First&& first_boundary, TileEnd&& tile_end) {
+  static_assert(STEPS % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
+  static_assert(STEPS > Mma::PH, "a stage holds more than one k-slice");
   typename Mma::Frag qf[2][NQ], pf[2][NP];
-  constexpr int NM = NQ * NP, LPS = PI + QI;
+  constexpr int NM = NQ * NP, LPS = PI + QI, LAST = STEPS - 1;
   auto all_p = [&](int slot) {
     static_for<PI>([&](auto i_c) { issue_p(slot, i_c); });
     issued_p();
@@ -363,50 +410,22 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
     static_for<QI>([&](auto j_c) { issue_q(slot, j_c); });
     issued_q();
   };
-  // fresh: the first slice of a tile starts the accumulators from the constant 0 operand instead of reading them, so
-  // nobody has to clear 128 registers per lane between tiles
-  auto slice_mfma = [&](auto cur_c, auto fresh_c) {
-    constexpr int cur = decltype(cur_c)::value;
-    constexpr bool fresh = decltype(fresh_c)::value;
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int q = 0; q < NQ; q++)
-#pragma unroll
-      for (int pp = 0; pp < NP; pp++) acc[q][pp] = Mma::run(qf[cur][q], pf[cur][pp], fresh ? zero : acc[q][pp]);
-    constexpr int NG0 = (NREADS + RPM - 1) / RPM, NR = NG0 < NM ? NG0 : NM - 1;
-#pragma unroll
-    for (int i = 0; i < NR; i++) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  auto read_step = [&](int bp, int bq, auto step_c) {
+    constexpr int step = decltype(step_c)::value;
+    load(bp, bq, step_c, qf[Mma::qset(step)], pf[step & 1]);
   };
-  auto slice_mfma_refill = [&](int p_slot, int q_slot) {
-    static_for<NM>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      acc[i / NP][i % NP] = Mma::run(qf[1][i / NP], pf[1][i % NP], acc[i / NP][i % NP]);
-      static_for<LPS>([&](auto j_c) {
-        constexpr int j = decltype(j_c)::value;
-        if constexpr (j * NM / LPS == i) {
-          if constexpr (j < PI) issue_p(p_slot, j_c);
-          else issue_q(q_slot, std::integral_constant<int, j - PI>{});
-        }
-      });
-      __builtin_amdgcn_sched_barrier(0);
-    });
-    issued_p();
-    issued_q();
-  };
-  auto inner_slices = [&](int bp, int bq, auto first_stage_c) {
-    static_for<SLICES - 1>([&](auto ks_c) {
-      constexpr int ks = decltype(ks_c)::value;
-      load(bp, bq, ks + 1, qf[(ks + 1) & 1], pf[(ks + 1) & 1]);
-      slice_mfma(std::integral_constant<int, (ks & 1)>{},
-                 std::integral_constant<bool, decltype(first_stage_c)::value && ks == 0>{});
+  // first_stage: the steps of the tile's first k-slice start the accumulators from the constant 0 operand instead of
+  // reading them, so nobody has to clear 128 registers per lane between tiles
+  auto inner_steps = [&](int bp, int bq, auto first_stage_c) {
+    static_for<STEPS - 1>([&](auto k_c) {
+      constexpr int k = decltype(k_c)::value;
+      read_step(bp, bq, std::integral_constant<int, k + 1>{});
+      mma_step<Mma, NQ, NP, NREADS, RPM, k, decltype(first_stage_c)::value && (k < Mma::PH)>(acc, qf, pf);
     });
   };
   constexpr std::false_type later{};
   constexpr std::true_type first{};
+  constexpr std::integral_constant<int, 0> step0{};
 
   all_p(0);
   all_q(0);
@@ -415,34 +434,46 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
   all_q(2);
   wait_vmem_upto<PI + 2 * QI>();
   lds_barrier();
-  load(0, 0, 0, qf[0], pf[0]);
+  read_step(0, 0, step0);
   int bp = 0, bq = 0;
-  // boundary behind a stage that is not the tile's last: read slice 0 of the next stage, refill the vacated slots
+  // boundary behind a stage that is not the tile's last: read step 0 of the next stage, refill the vacated slots
   auto boundary = [&]() {
     lds_barrier();
     const int np = bp ^ 1, nq = bq == 2 ? 0 : bq + 1;
-    load(np, nq, 0, qf[0], pf[0]);
+    read_step(np, nq, step0);
     __builtin_amdgcn_sched_barrier(0);
-    slice_mfma_refill(bp, bq);  // P(s+2), Q(s+3) into the slots stage s leaves behind
+    // P(s+2), Q(s+3) into the slots stage s leaves behind
+    mma_step_refill<Mma, NQ, NP, LAST>(acc, qf, pf, [&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      static_for<LPS>([&](auto j_c) {
+        constexpr int j = decltype(j_c)::value;
+        if constexpr (j * NM / LPS == i) {
+          if constexpr (j < PI) issue_p(bp, j_c);
+          else issue_q(bq, std::integral_constant<int, j - PI>{});
+        }
+      });
+    });
+    issued_p();
+    issued_q();
     bp = np;
     bq = nq;
   };
   for (;;) {
     // stage 0: stores of the previous epilogue may still be outstanding, wait for everything
-    inner_slices(bp, bq, first);
+    inner_steps(bp, bq, first);
     wait_vmem_all();
     first_boundary();
     boundary();
     for (int s = 1; s + 1 < S; s++) {
-      inner_slices(bp, bq, later);
+      inner_steps(bp, bq, later);
       wait_vmem_upto<QI>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
       boundary();
     }
     // last stage: the stages of the next tile that are due are already requested; its own slots become scratch
-    inner_slices(bp, bq, later);
+    inner_steps(bp, bq, later);
     wait_vmem_upto<QI>();
     lds_barrier();
-    slice_mfma(std::integral_constant<int, 1>{}, later);
+    mma_step<Mma, NQ, NP, NREADS, RPM, LAST, false>(acc, qf, pf);
     if (!tile_end(bp, bq)) break;
     wait_lds_all();
     lds_barrier();  // every wave has read its parked rows back: the two slots may be refilled
@@ -450,7 +481,7 @@ SMOE_DEV void gemm_stream_loop(const int S, f32x16 (&acc)[NQ][NP], IssueP&& issu
     all_q(bq);
     bp ^= 1;
     bq = bq == 2 ? 0 : bq + 1;
-    load(bp, bq, 0, qf[0], pf[0]);
+    read_step(bp, bq, step0);
   }
   wait_vmem_all();  // the streams ran ahead into ring slots nobody reads any more: let those loads land before the end
 }
@@ -554,18 +585,30 @@ struct FwdEpilogueArgs {
   int n_base, N;         // first accumulator column of this wave's tile, number of accumulator columns
 };
 
-// acc[fn][fm] is the wave's TM x TN tile (lane = token row l%32 of fragment row fm; register quad rg of fragment column
-// fn = columns fn*32 + 8*rg + 4*(l/32) + 0..3).  Adds the bias, stores out0, and with WITH_ACT evaluates activation ACT
-// from the un-rounded accumulator into out1 (TN/2 columns for the gated activations, TN otherwise).  The caller has
-// made sure that no wave still reads the LDS ring: every wave parks its tile in its own region of it.
-template <int TM, int TN, int FM, int FN, bool WITH_ACT, int ACT>
-SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int lane, const FwdEpilogueArgs& a) {
+// Where a lane's accumulator registers sit in the wave's TM x TN tile: acc[fn][fm] is fragment (fn, fm) of FR x FR
+// values; a lane owns token row fm * FR + l % FR and, in register group rg (QPF groups of four per fragment), the four
+// consecutive features fn * FR + rg * 4 * (64 / FR) + 4 * (l / FR) + 0..3.
+template <class Mma>
+struct AccLayout {
+  static constexpr int FR = Mma::FR, QPF = Mma::ACC_REGS / 4, NGRP = 64 / FR;
+  static __device__ __forceinline__ int row(int lane) { return lane & (FR - 1); }
+  static __device__ __forceinline__ int col(int rg, int lane) { return rg * (4 * NGRP) + 4 * (lane / FR); }
+};
+
+// acc is the wave's TM x TN tile.  Adds the bias, stores out0, and with WITH_ACT evaluates activation ACT from the
+// un-rounded accumulator into out1 (TN/2 columns for the gated activations, TN otherwise).  The caller has made sure
+// that no wave still reads the LDS ring: every wave parks its tile in its own region of it.
+template <class Mma, int TM, int TN, bool WITH_ACT, int ACT>
+SMOE_DEV void forward_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* smem, int wave, int lane,
+                               const FwdEpilogueArgs& a) {
+  using AL = AccLayout<Mma>;
+  constexpr int FR = Mma::FR, FM = TM / FR, FN = TN / FR, QPF = AL::QPF;
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
   if (a.bias != nullptr) {
-    static_for<FN * 4>([&](auto q_c) {
-      constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-      int n = a.n_base + fn * 32 + 8 * rg + 4 * (lane >> 5);
+    static_for<FN * QPF>([&](auto q_c) {
+      constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+      int n = a.n_base + fn * FR + AL::col(rg, lane);
       n = n <= a.N - 4 ? n : a.N - 4;
       const u32x2 b = *(const u32x2*)(a.bias + n);
       const float b0 = bf16_lo(b[0]), b1 = bf16_hi(b[0]), b2 = bf16_lo(b[1]), b3 = bf16_hi(b[1]);
@@ -581,100 +624,116 @@ SMOE_DEV void forward_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int 
   using LZ = EpiLayout<TN>;
   using LY = EpiLayout<TN / 2>;
   char* region = smem + wave * (TM * LZ::ROW_BYTES);
+  const int lrow = AL::row(lane);
   if (!WITH_ACT || a.out0 != nullptr) {
     static_for<FM>([&](auto fm_c) {
       constexpr int fm = decltype(fm_c)::value;
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+      static_for<FN * QPF>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
         u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
                    pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
-        *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+        *(u32x2*)(region + (fm * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
       });
     });
     epilogue_flush<TM, TN>(region, lane, a.out0, a.out0_stride, a.m_base, a.row_end, a.n_base, a.N);
   }
   if constexpr (WITH_ACT && GLU) {
     if (a.out1 != nullptr) {
-    static_for<FM>([&](auto fm_c) {
-      constexpr int fm = decltype(fm_c)::value;
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
-        const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
-        const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
-        *(uint32_t*)(region + (fm * 32 + (lane & 31)) * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * (lane >> 5)) * 2) = v;
+      static_for<FM>([&](auto fm_c) {
+        constexpr int fm = decltype(fm_c)::value;
+        static_for<FN * QPF>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+          const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
+          const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
+          const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
+          *(uint32_t*)(region + (fm * FR + lrow) * LY::ROW_BYTES + (fn * FR + AL::col(rg, lane))) = v;
+        });
       });
-    });
-    epilogue_flush<TM, TN / 2>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base / 2, a.N / 2);
+      epilogue_flush<TM, TN / 2>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base / 2, a.N / 2);
     }
   } else if constexpr (WITH_ACT) {
     if (a.out1 != nullptr) {
-    static_for<FM>([&](auto fm_c) {
-      constexpr int fm = decltype(fm_c)::value;
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
-                   pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
-        *(u32x2*)(region + (fm * 32 + (lane & 31)) * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+      static_for<FM>([&](auto fm_c) {
+        constexpr int fm = decltype(fm_c)::value;
+        static_for<FN * QPF>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+          u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
+                     pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
+          *(u32x2*)(region + (fm * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
+        });
       });
-    });
-    epilogue_flush<TM, TN>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base, a.N);
+      epilogue_flush<TM, TN>(region, lane, a.out1, a.out1_stride, a.m_base, a.row_end, a.n_base, a.N);
     }
   }
 }
 
-// The same epilogue one 32-row fragment row at a time, parked in a caller-chosen LDS region of 32 padded rows
+// The same epilogue 32 rows at a time, parked in a caller-chosen LDS region of 32 padded rows
 // (32 * EpiLayout<TN>::ROW_BYTES bytes per wave): for kernels whose ring keeps running during the epilogue.
-template <int TN, int FM, int FN, bool WITH_ACT, int ACT>
-SMOE_DEV void forward_epilogue_rows(f32x16 (&acc)[FN][FM], char* region, int lane, const FwdEpilogueArgs& a) {
+template <class Mma, int TM, int TN, bool WITH_ACT, int ACT>
+SMOE_DEV void forward_epilogue_rows(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* region, int lane,
+                                    const FwdEpilogueArgs& a) {
+  using AL = AccLayout<Mma>;
+  constexpr int FR = Mma::FR, FN = TN / FR, QPF = AL::QPF, RB = 32 / FR;  // RB fragment rows make a 32-row batch
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
   using LZ = EpiLayout<TN>;
   using LY = EpiLayout<TN / 2>;
   const bool with_bias = a.bias != nullptr;
-  const int mrow = lane & 31, half = lane >> 5;
-  static_for<FM>([&](auto fm_c) {
-    constexpr int fm = decltype(fm_c)::value;
-    if (with_bias) {  // re-read per fragment row (a few cached words) rather than held in registers across the rows
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        int n = a.n_base + fn * 32 + 8 * rg + 4 * half;
+  const int lrow = AL::row(lane);
+  static_for<TM / 32>([&](auto blk_c) {
+    constexpr int blk = decltype(blk_c)::value;
+    if (with_bias) {  // re-read per batch (a few cached words) rather than held in registers across the batches
+      static_for<FN * QPF>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+        int n = a.n_base + fn * FR + AL::col(rg, lane);
         n = n <= a.N - 4 ? n : a.N - 4;
         const u32x2 b = *(const u32x2*)(a.bias + n);
-        acc[fn][fm][4 * rg + 0] += bf16_lo(b[0]);
-        acc[fn][fm][4 * rg + 1] += bf16_hi(b[0]);
-        acc[fn][fm][4 * rg + 2] += bf16_lo(b[1]);
-        acc[fn][fm][4 * rg + 3] += bf16_hi(b[1]);
+        static_for<RB>([&](auto sub_c) {
+          constexpr int fm = blk * RB + decltype(sub_c)::value;
+          acc[fn][fm][4 * rg + 0] += bf16_lo(b[0]);
+          acc[fn][fm][4 * rg + 1] += bf16_hi(b[0]);
+          acc[fn][fm][4 * rg + 2] += bf16_lo(b[1]);
+          acc[fn][fm][4 * rg + 3] += bf16_hi(b[1]);
+        });
       });
     }
-    const int m0 = a.m_base + fm * 32;
+    const int m0 = a.m_base + blk * 32;
     if (!WITH_ACT || a.out0 != nullptr) {
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
-                   pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
-        *(u32x2*)(region + mrow * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * half) * 2) = v;
+      static_for<RB>([&](auto sub_c) {
+        constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
+        static_for<FN * QPF>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+          u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
+                     pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
+          *(u32x2*)(region + (sub * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
+        });
       });
       epilogue_flush<32, TN>(region, lane, a.out0, a.out0_stride, m0, a.row_end, a.n_base, a.N);
     }
     if constexpr (WITH_ACT && GLU) {
       if (a.out1 != nullptr) {
-        static_for<FN * 4>([&](auto q_c) {
-          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-          const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
-          const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
-          const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
-          *(uint32_t*)(region + mrow * LY::ROW_BYTES + (fn * 16 + 4 * rg + 2 * half) * 2) = v;
+        static_for<RB>([&](auto sub_c) {
+          constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
+          static_for<FN * QPF>([&](auto q_c) {
+            constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+            const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
+            const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
+            const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
+            *(uint32_t*)(region + (sub * FR + lrow) * LY::ROW_BYTES + (fn * FR + AL::col(rg, lane))) = v;
+          });
         });
         epilogue_flush<32, TN / 2>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base / 2, a.N / 2);
       }
     } else if constexpr (WITH_ACT) {
       if (a.out1 != nullptr) {
-        static_for<FN * 4>([&](auto q_c) {
-          constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-          u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
-                     pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
-          *(u32x2*)(region + mrow * LZ::ROW_BYTES + (fn * 32 + 8 * rg + 4 * half) * 2) = v;
+        static_for<RB>([&](auto sub_c) {
+          constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
+          static_for<FN * QPF>([&](auto q_c) {
+            constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+            u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
+                       pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
+            *(u32x2*)(region + (sub * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
+          });
         });
         epilogue_flush<32, TN>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base, a.N);
       }

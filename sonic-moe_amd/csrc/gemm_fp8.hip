@@ -18,7 +18,6 @@
 namespace smoe {
 
 typedef int i32x8 __attribute__((ext_vector_type(8)));
-typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 // ---- quantiser ---------------------------------------------------------------------------------------------------
 // e8m0 exponent of the smallest power of two s with amax / s <= 448 (the largest e4m3 value): no element saturates
@@ -138,6 +137,13 @@ struct Fp8Frag {
 };
 struct Fp8Mma {
   typedef Fp8Frag Frag;
+  typedef f32x16 Acc;
+  // a step is one k-slice of 64 contraction bytes and reads all of the wave's fragments (see Bf16Mma32)
+  static constexpr int FR = 32, KSTEP = 64, PH = 1, ACC_REGS = 16;
+  static constexpr int qset(int step) { return step & 1; }
+  static constexpr int phalf(int) { return 0; }
+  static constexpr bool reads_q(int) { return true; }
+  static constexpr int kslice(int step) { return step; }
   static __device__ __forceinline__ f32x16 run(const Frag& q, const Frag& p, f32x16 c) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(q.data, p.data, c, 0, 0, 0, q.scale, 0, p.scale);
   }
@@ -323,7 +329,8 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
       s_src[j] += s_step[j];
     }
   };
-  auto load = [&](int buf, int /*s*/, int ks, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[FM]) {
+  auto load = [&](int buf, int /*s*/, auto step_c, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[FM]) {
+    constexpr int ks = decltype(step_c)::value;
     const char* st = smem + buf * C::STAGE;
     const int shift = 8 * (2 * ks + half);
 #pragma unroll
@@ -355,7 +362,7 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
   ea.N = p.N;
   wait_vmem_all();
   lds_barrier();  // all waves are done reading the last stage
-  forward_epilogue<C::TM, C::TN, FM, FN, WITH_ACT, ACT>(acc, smem, wave, lane, ea);
+  forward_epilogue<Fp8Mma, C::TM, C::TN, WITH_ACT, ACT>(acc, smem, wave, lane, ea);
   if constexpr (WITH_ACT) {
     if (p.yq != nullptr)  // the parking area of forward_epilogue is read back by the same wave that wrote it: no barrier
       fp8_activation_epilogue<C::TM, C::TN, FM, FN, ACT>(acc, smem, wave, lane, p.yq, p.I, p.yq_scales, p.yq_rows,

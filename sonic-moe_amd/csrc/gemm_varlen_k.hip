@@ -34,8 +34,12 @@ struct KCfg {
   static constexpr int BA = BA_, BB = BB_, WA = WA_, WB = WB_, BK = BK_, NSTAGE = NSTAGE_;
   static constexpr bool R_GATHER = R_GATHER_, S_GATHER = S_GATHER_;
   static constexpr int NW = WA * WB, NT = NW * 64;
+  typedef Bf16Mma Mma;
   static constexpr int TA = BA / WA, TB = BB / WB;
-  static constexpr int FA = TA / 32, FB = TB / 32;
+  static constexpr int FR = Mma::FR;                   // rows / columns of a matrix-instruction fragment
+  static constexpr int FA = TA / FR, FB = TB / FR;     // fragments of the wave tile
+  static constexpr int NP = FA / Mma::PH;              // R fragments a step works on
+  static constexpr int STEPS = BK / Mma::KSTEP * Mma::PH;
   static constexpr int R_STAGE = BA * BK * 2, S_STAGE = BB * BK * 2;
   static constexpr int STAGE = R_STAGE + S_STAGE;
   static constexpr int EPI = NW * TA * (TB * 2 + 16);
@@ -86,7 +90,9 @@ SMOE_DEV bool decode_tile(const VarlenKParams& p, int64_t v, int& e, int& ta, in
 template <class C>
 __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
+  using Mma = typename C::Mma;
+  using AL = AccLayout<Mma>;
+  constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, FR = C::FR, QPF = AL::QPF;
   const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -131,35 +137,32 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   // transpose-load fragment offsets (bytes inside a stage)
   int r_off[2 * FA], s_off[2 * FB];
   {
+    // a fragment lane supplies column l % FR and the contraction elements 8 * (l / FR) + 0..7 of the k-slice; the
+    // transpose load hands lane i of a 16-lane group column i of the 4 (k) x 16 block its lanes' addresses name
     const int grp = lane >> 4, i16 = lane & 15;
-    const int kk = 8 * (grp >> 1) + (i16 >> 2);
+    const int kk = (C::FR == 32 ? 8 * (grp >> 1) : 8 * grp) + (i16 >> 2);
 #pragma unroll
     for (int f = 0; f < FA; f++) {
-      const int c32 = (wa * C::TA) / 16 + f * 2 + (grp & 1);
+      const int c16 = (wa * C::TA) / 16 + (C::FR == 32 ? f * 2 + (grp & 1) : f);
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        r_off[f * 2 + h] = k * C::R_ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        r_off[f * 2 + h] = k * C::R_ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
 #pragma unroll
     for (int f = 0; f < FB; f++) {
-      const int c32 = (wb * C::TB) / 16 + f * 2 + (grp & 1);
+      const int c16 = (wb * C::TB) / 16 + (C::FR == 32 ? f * 2 + (grp & 1) : f);
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
   }
 
-  f32x16 acc[FB][FA];
-#pragma unroll
-  for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-    for (int fa = 0; fa < FA; fa++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[fb][fa][r] = 0.f;
+  typename Mma::Acc acc[FB][FA];
+  clear_accumulators<Mma>(acc);
 
   // Token rows of a stage: wave w feeds rows [w*RPW, (w+1)*RPW) of each operand's stage, R_RPI resp. S_RPI rows per
   // load instruction.  The gather indices of those rows are wave-uniform, so they are fetched with SCALAR loads:
@@ -256,19 +259,25 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       for (int j = 0; j < RPW; j++) tok[j] = tok_next[j];
     }
   };
-  auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
+  auto load = [&](int buf, int /*s*/, auto step_c, bf16x8(&sf)[FB], bf16x8(&rf)[C::NP]) {
+    constexpr int step = decltype(step_c)::value;
+    constexpr int kofs = Mma::kslice(step) * Mma::KSTEP, ph = Mma::phalf(step);
     const char* st = smem + buf * C::STAGE;
 #pragma unroll
-    for (int f = 0; f < FA; f++)
-      rf[f] = lds_read_tr2(st + r_off[f * 2] + ks * 16 * C::R_ROWB, st + r_off[f * 2 + 1] + ks * 16 * C::R_ROWB);
+    for (int pp = 0; pp < C::NP; pp++) {
+      const int f = ph * C::NP + pp;
+      rf[pp] = lds_read_tr2(st + r_off[f * 2] + kofs * C::R_ROWB, st + r_off[f * 2 + 1] + kofs * C::R_ROWB);
+    }
+    if constexpr (Mma::reads_q(step)) {
 #pragma unroll
-    for (int f = 0; f < FB; f++)
-      sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
+      for (int f = 0; f < FB; f++)
+        sf[f] = lds_read_tr2(st + s_off[f * 2] + kofs * C::S_ROWB, st + s_off[f * 2 + 1] + kofs * C::S_ROWB);
+    }
   };
   if (S > 0) fetch(0, tok);
   // MFMA as D[b][a] += S[b][k] R[k][a]: lane owns output row a = l%32, register quads hold 4 consecutive columns b
   // two transpose loads per fragment: 12 reads for the 8 MFMAs of a slice, issued two per MFMA
-  gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE, Bf16Mma, 2>(S, acc, issue, load);
+  gemm_mainloop<FB, C::NP, 2 * (C::NP + FB), C::R_INSTR + C::S_INSTR, C::STEPS, NSTAGE, Mma, 2>(S, acc, issue, load);
   // epilogue through LDS (also writes the zeros of experts without tokens)
   using L = EpiLayout<C::TB>;
   char* region = smem + wave * (C::TA * L::ROW_BYTES);
@@ -276,11 +285,11 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
   lds_barrier();
   static_for<FA>([&](auto fa_c) {
     constexpr int fa = decltype(fa_c)::value;
-    static_for<FB * 4>([&](auto q_c) {
-      constexpr int fb = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
+    static_for<FB * QPF>([&](auto q_c) {
+      constexpr int fb = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
       u32x2 v = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
                  pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
-      *(u32x2*)(region + (fa * 32 + (lane & 31)) * L::ROW_BYTES + (fb * 32 + 8 * rg + 4 * (lane >> 5)) * 2) = v;
+      *(u32x2*)(region + (fa * FR + AL::row(lane)) * L::ROW_BYTES + (fb * FR + AL::col(rg, lane)) * 2) = v;
     });
   });
   epilogue_flush<C::TA, C::TB>(region, lane, p.out + (int64_t)e * p.out_stride_e, p.out_stride_row, a0 + wa * C::TA,
@@ -295,7 +304,9 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 template <class C>
 __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKParams p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, SLICES = C::BK / 16;
+  using Mma = typename C::Mma;
+  using AL = AccLayout<Mma>;
+  constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, FR = C::FR, QPF = AL::QPF;
   const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -304,35 +315,32 @@ __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKPara
   // transpose-load fragment offsets (bytes inside a stage)
   int r_off[2 * FA], s_off[2 * FB];
   {
+    // a fragment lane supplies column l % FR and the contraction elements 8 * (l / FR) + 0..7 of the k-slice; the
+    // transpose load hands lane i of a 16-lane group column i of the 4 (k) x 16 block its lanes' addresses name
     const int grp = lane >> 4, i16 = lane & 15;
-    const int kk = 8 * (grp >> 1) + (i16 >> 2);
+    const int kk = (C::FR == 32 ? 8 * (grp >> 1) : 8 * grp) + (i16 >> 2);
 #pragma unroll
     for (int f = 0; f < FA; f++) {
-      const int c32 = (wa * C::TA) / 16 + f * 2 + (grp & 1);
+      const int c16 = (wa * C::TA) / 16 + (C::FR == 32 ? f * 2 + (grp & 1) : f);
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        r_off[f * 2 + h] = k * C::R_ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        r_off[f * 2 + h] = k * C::R_ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
 #pragma unroll
     for (int f = 0; f < FB; f++) {
-      const int c32 = (wb * C::TB) / 16 + f * 2 + (grp & 1);
+      const int c16 = (wb * C::TB) / 16 + (C::FR == 32 ? f * 2 + (grp & 1) : f);
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
       }
     }
   }
 
-  f32x16 acc[FB][FA];
-#pragma unroll
-  for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-    for (int fa = 0; fa < FA; fa++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[fb][fa][r] = 0.f;
+  typename Mma::Acc acc[FB][FA];
+  clear_accumulators<Mma>(acc);
 
   static_assert(C::R_INSTR * C::R_RPI == C::S_INSTR * C::S_RPI, "both operands cover the same token rows per wave");
   constexpr int RPW = C::R_INSTR * C::R_RPI;  // token rows per wave and stage
@@ -449,14 +457,20 @@ __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKPara
       for (int j = 0; j < RPW; j++) tok[j] = tok_next[j];
     }
   };
-  auto load = [&](int buf, int /*s*/, int ks, bf16x8(&sf)[FB], bf16x8(&rf)[FA]) {
+  auto load = [&](int buf, int /*s*/, auto step_c, bf16x8(&sf)[FB], bf16x8(&rf)[C::NP]) {
+    constexpr int step = decltype(step_c)::value;
+    constexpr int kofs = Mma::kslice(step) * Mma::KSTEP, ph = Mma::phalf(step);
     const char* st = smem + buf * C::STAGE;
 #pragma unroll
-    for (int f = 0; f < FA; f++)
-      rf[f] = lds_read_tr2(st + r_off[f * 2] + ks * 16 * C::R_ROWB, st + r_off[f * 2 + 1] + ks * 16 * C::R_ROWB);
+    for (int pp = 0; pp < C::NP; pp++) {
+      const int f = ph * C::NP + pp;
+      rf[pp] = lds_read_tr2(st + r_off[f * 2] + kofs * C::R_ROWB, st + r_off[f * 2 + 1] + kofs * C::R_ROWB);
+    }
+    if constexpr (Mma::reads_q(step)) {
 #pragma unroll
-    for (int f = 0; f < FB; f++)
-      sf[f] = lds_read_tr2(st + s_off[f * 2] + ks * 16 * C::S_ROWB, st + s_off[f * 2 + 1] + ks * 16 * C::S_ROWB);
+      for (int f = 0; f < FB; f++)
+        sf[f] = lds_read_tr2(st + s_off[f * 2] + kofs * C::S_ROWB, st + s_off[f * 2 + 1] + kofs * C::S_ROWB);
+    }
   };
 
   int64_t v = blockIdx.x;
@@ -466,7 +480,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKPara
   static_assert(RB == 128, "the parked rows are 8 chunks of 16 bytes");
   for (int k = 1; have; k++) {
     const int cur_e = e, cur_a0 = a0, cur_b0 = b0;
-    gemm_mainloop<FB, FA, 2 * (FA + FB), C::R_INSTR + C::S_INSTR, SLICES, NSTAGE, Bf16Mma, 2, false>(S, acc, issue, load);
+    gemm_mainloop<FB, C::NP, 2 * (C::NP + FB), C::R_INSTR + C::S_INSTR, C::STEPS, NSTAGE, Mma, 2, false>(S, acc, issue, load);
     wait_lds_all();
     lds_barrier();  // every wave has read the ring's last stage: the next tile may land in it
     v += gridDim.x;
@@ -482,13 +496,16 @@ __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKPara
     const int a_base = cur_a0 + wa * C::TA, b_base = cur_b0 + wb * C::TB;
     const int rr = el >> 3, cc = el & 7;
     const int col = b_base + cc * 8;
-    static_for<FA>([&](auto fa_c) {
-      constexpr int fa = decltype(fa_c)::value;
-      static_for<FB * 4>([&](auto q_c) {
-        constexpr int fb = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        u32x2 pv = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
-                    pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
-        epi_park_y<RB>(region, el & 31, (fb * 32 + 8 * rg + 4 * (el >> 5)) * 2, pv);
+    static_for<C::TA / 32>([&](auto blk_c) {  // 32 output rows at a time
+      constexpr int blk = decltype(blk_c)::value;
+      static_for<32 / FR>([&](auto sub_c) {
+        constexpr int sub = decltype(sub_c)::value, fa = blk * (32 / FR) + sub;
+        static_for<FB * QPF>([&](auto q_c) {
+          constexpr int fb = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+          u32x2 pv = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
+                      pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
+          epi_park_y<RB>(region, sub * FR + AL::row(el), (fb * FR + AL::col(rg, el)) * 2, pv);
+        });
       });
       u32x4 rows[4];
 #pragma unroll
@@ -498,17 +515,12 @@ __global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKPara
       }
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        const int row = a_base + fa * 32 + q * 8 + rr;
+        const int row = a_base + blk * 32 + q * 8 + rr;
         if (row < p.NA && col < p.NB) *(u32x4*)(out + (int64_t)row * p.out_stride_row + col) = rows[q];
       }
-      __builtin_amdgcn_sched_barrier(0);  // fragment row by fragment row
+      __builtin_amdgcn_sched_barrier(0);  // batch by batch
     });
-#pragma unroll
-    for (int fb = 0; fb < FB; fb++)
-#pragma unroll
-      for (int fa = 0; fa < FA; fa++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[fb][fa][r] = 0.f;
+    clear_accumulators<Mma>(acc);
   }
   wait_vmem_all();
 }

@@ -39,8 +39,13 @@ struct Cfg {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, NSTAGE = NSTAGE_;
   static constexpr bool QMN = QMN_;
   static constexpr int NW = WM * WN, NT = NW * 64;
+  typedef Bf16Mma Mma;
   static constexpr int TM = BM / WM, TN = BN / WN;
-  static constexpr int FM = TM / 32, FN = TN / 32;
+  static constexpr int FR = Mma::FR;                       // rows / columns of a matrix-instruction fragment
+  static constexpr int FM = TM / FR, FN = TN / FR;         // fragments of the wave tile
+  static constexpr int NP = FM / Mma::PH;                  // token fragments a step works on
+  static constexpr int KSL = BK / Mma::KSTEP;              // k-slices per stage
+  static constexpr int STEPS = KSL * Mma::PH;              // steps per stage
   static constexpr int P_STAGE = BM * BK * 2, Q_STAGE = BN * BK * 2;  // bytes
   static constexpr int STAGE = P_STAGE + Q_STAGE;
   static constexpr int P_INSTR = P_STAGE / 1024 / NW;  // direct-to-LDS loads per wave and stage
@@ -59,37 +64,63 @@ struct Cfg {
   static constexpr int KRPI = 64 / KPR;   // rows per load instruction of a K-major stage
   static constexpr int NG = ROWB / 32;    // 32-byte groups per k-row
   static_assert(P_INSTR >= 1 && Q_INSTR >= 1, "tile too small for the wave count");
-  static_assert(TM % 32 == 0 && TN % 32 == 0, "wave tile must be a multiple of the 32x32 MFMA");
+  static_assert(TM % 32 == 0 && TN % 32 == 0 && FM % Mma::PH == 0, "wave tile must be a multiple of 32 x 32");
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
-// Per-lane LDS fragment offsets (bytes inside a ring slot) of wave (wm, wn): p_off[ks] / q_off[ks] for K-major stages
-// (one 16-byte piece per slice), q_off[2 * fn + h] for an MN-major weight stage (two transpose loads per fragment).
+// Per-lane LDS fragment offsets (bytes inside a ring slot) of wave (wm, wn): p_off[ksl] / q_off[ksl] for K-major
+// stages (one 16-byte piece per k-slice ksl; fragment f of the wave lies f * FR rows further), q_off[2 * fn + h] for an
+// MN-major weight stage (two transpose loads per fragment; k-slice ksl lies ksl * KSTEP k-rows further).
+// A fragment lane supplies row (K-major) or column (MN-major) l % FR and the 8 contraction elements 8 * (l / FR) + 0..7
+// of the k-slice.
 template <class C>
-SMOE_DEV void fragment_offsets(int wm, int wn, int lane, int (&p_off)[C::BK / 16],
-                               int (&q_off)[C::QMN ? 2 * C::FN : C::BK / 16]) {
-  constexpr int SLICES = C::BK / 16;
+SMOE_DEV void fragment_offsets(int wm, int wn, int lane, int (&p_off)[C::KSL], int (&q_off)[C::QMN ? 2 * C::FN : C::KSL]) {
+  constexpr int FR = C::FR, PPS = C::Mma::KSTEP / 8;  // 16-byte pieces per row and k-slice
   {
-    const int row = wm * C::TM + (lane & 31);
+    const int row = wm * C::TM + (lane & (FR - 1));
     const int sw = kswz<C::BK>(row);
 #pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) p_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+    for (int ks = 0; ks < C::KSL; ks++) p_off[ks] = row * C::KROW + (((PPS * ks + lane / FR) ^ sw) << 4);
   }
   if constexpr (!C::QMN) {
-    const int row = wn * C::TN + (lane & 31);
+    const int row = wn * C::TN + (lane & (FR - 1));
     const int sw = kswz<C::BK>(row);
 #pragma unroll
-    for (int ks = 0; ks < SLICES; ks++) q_off[ks] = row * C::KROW + (((2 * ks + (lane >> 5)) ^ sw) << 4);
+    for (int ks = 0; ks < C::KSL; ks++) q_off[ks] = row * C::KROW + (((PPS * ks + lane / FR) ^ sw) << 4);
   } else {
+    // the transpose load hands lane i of a 16-lane group column i of a 4 (k) x 16 (n) block; the lanes' addresses name
+    // its four k-rows, 4 lanes x 8 bytes each
     const int grp = lane >> 4, i16 = lane & 15;
-    const int kk = 8 * (grp >> 1) + (i16 >> 2);
+    const int kk = (FR == 32 ? 8 * (grp >> 1) : 8 * grp) + (i16 >> 2);
 #pragma unroll
     for (int fn = 0; fn < C::FN; fn++) {
-      const int c32 = (wn * C::TN) / 16 + fn * 2 + (grp & 1);
+      const int c16 = (wn * C::TN) / 16 + (FR == 32 ? fn * 2 + (grp & 1) : fn);  // 16-column block = 32-byte group
 #pragma unroll
       for (int h = 0; h < 2; h++) {
         const int k = kk + 4 * h;
-        q_off[fn * 2 + h] = k * C::ROWB + ((c32 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        q_off[fn * 2 + h] = k * C::ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+      }
+    }
+  }
+}
+
+// the LDS reads of one step: the step's half of the token fragments, and the weight fragments when the step starts a
+// k-slice
+template <class C, int STEP>
+SMOE_DEV void read_fragments(const char* sp, const char* sq, const int (&p_off)[C::KSL],
+                             const int (&q_off)[C::QMN ? 2 * C::FN : C::KSL], bf16x8 (&qf)[C::FN], bf16x8 (&pf)[C::NP]) {
+  using Mma = typename C::Mma;
+  constexpr int ksl = Mma::kslice(STEP), ph = Mma::phalf(STEP);
+#pragma unroll
+  for (int pp = 0; pp < C::NP; pp++) pf[pp] = lds_read_b128(sp + p_off[ksl] + (ph * C::NP + pp) * C::FR * C::KROW);
+  if constexpr (Mma::reads_q(STEP)) {
+#pragma unroll
+    for (int fn = 0; fn < C::FN; fn++) {
+      if constexpr (!C::QMN) {
+        qf[fn] = lds_read_b128(sq + q_off[ksl] + fn * C::FR * C::KROW);
+      } else {
+        qf[fn] = lds_read_tr2(sq + q_off[fn * 2] + ksl * Mma::KSTEP * C::ROWB,
+                              sq + q_off[fn * 2 + 1] + ksl * Mma::KSTEP * C::ROWB);
       }
     }
   }
@@ -102,7 +133,9 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, SLICES = C::BK / 16;
+  using Mma = typename C::Mma;
+  using AL = AccLayout<Mma>;
+  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, FR = C::FR, QPF = AL::QPF;
   const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -163,17 +196,12 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
   const int S_total = p.Kdim / BK;
 
   // ---- per-lane LDS fragment offsets (bytes inside a ring slot) ----
-  int p_off[SLICES];
-  int q_off[C::QMN ? 2 * FN : SLICES];
+  int p_off[C::KSL];
+  int q_off[C::QMN ? 2 * FN : C::KSL];
   fragment_offsets<C>(wm, wn, lane, p_off, q_off);
 
-  f32x16 acc[FN][FM];
-#pragma unroll
-  for (int fn = 0; fn < FN; fn++)
-#pragma unroll
-    for (int fm = 0; fm < FM; fm++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
+  typename Mma::Acc acc[FN][FM];
+  clear_accumulators<Mma>(acc);
 
   constexpr int Q_RING = C::P_SLOTS * C::P_STAGE;  // byte offset of the weight operand's slots
   auto issue_p = [&](int slot, auto i_c) {
@@ -186,22 +214,12 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     load16_to_lds(q_src[j], smem_base + Q_RING + slot * C::Q_STAGE + (wave * C::Q_INSTR + j) * 1024);
     q_src[j] += q_step;
   };
-  auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
-    const char* sp = smem + p_slot * C::P_STAGE;
-    const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
-#pragma unroll
-    for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(sp + p_off[ks] + fm * 32 * C::KROW);
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
-      if constexpr (!C::QMN) {
-        qf[fn] = lds_read_b128(sq + q_off[ks] + fn * 32 * C::KROW);
-      } else {
-        qf[fn] = lds_read_tr2(sq + q_off[fn * 2] + ks * 16 * C::ROWB, sq + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
-      }
-    }
+  auto load = [&](int p_slot, int q_slot, auto step_c, bf16x8(&qf)[FN], bf16x8(&pf)[C::NP]) {
+    read_fragments<C, decltype(step_c)::value>(smem + p_slot * C::P_STAGE, smem + Q_RING + q_slot * C::Q_STAGE, p_off,
+                                               q_off, qf, pf);
   };
-  gemm_mainloop_asym<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR, C::Q_INSTR, SLICES>(S_total, acc, issue_p, issue_q,
-                                                                                          load);
+  gemm_mainloop_asym<FN, C::NP, (C::QMN ? 2 * FN : FN) + C::NP, C::P_INSTR, C::Q_INSTR, C::STEPS, Mma>(
+      S_total, acc, issue_p, issue_q, load);
 
   const int m_base = row0 + wm * C::TM, n_base = n0 + wn * C::TN;
 
@@ -218,19 +236,20 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     ea.N = p.N;
     wait_vmem_all();
     lds_barrier();  // all waves are done reading the last stage
-    forward_epilogue<C::TM, C::TN, FM, FN, ROLE == ROLE_UP_FWD, ACT>(acc, smem, wave, lane, ea);
+    forward_epilogue<Mma, C::TM, C::TN, ROLE == ROLE_UP_FWD, ACT>(acc, smem, wave, lane, ea);
   } else {
     // ---- dz epilogue ----
-    // acc = dy1[i][m].  Per 32-row fragment row the wavefront stages its z sub-tile (32 rows x ZW*TN bf16; ZW = 2
+    // acc = dy1[i][m].  32 token rows at a time the wavefront stages its z sub-tile (32 rows x ZW*TN bf16; ZW = 2
     // interleaved (gate, up) columns per dy1 column for gated activations, 1 otherwise) through LDS: row-contiguous
-    // 16-byte global loads (two fragment rows in flight in registers) -> LDS -> each lane picks the z values of its four
-    // dy1 columns of its token row, computes dz in place and y1s into a second area -> both are written back
+    // 16-byte global loads (two batches in flight in registers) -> LDS -> each lane picks the z values of its four
+    // dy1 columns of its token rows, computes dz in place and y1s into a second area -> both are written back
     // row-contiguous.  All global traffic of the epilogue is full 128-byte lines.
     constexpr int ZW = GLU ? 2 : 1;
     constexpr int ZB = C::TN * 2 * ZW, YB = C::TN * 2;       // bytes per staged z/dz row, y1s row
     constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
     constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
     constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;               // row swizzle of the staged z chunks
+    constexpr int NB = C::TM / 32, RB = 32 / FR;             // 32-row batches; fragment rows per batch
     static_assert(C::NW * 32 * (ZB + YB) <= C::RING, "dz staging must fit into the idle ring");
     char* zbuf = smem + wave * (32 * (ZB + YB));
     char* ybuf = zbuf + 32 * ZB;
@@ -239,85 +258,90 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     const int zcol = ZW * n_base + zc * 8;  // first z column of this lane's 16-byte chunk
     const int zcol_c = zcol <= zlimit - 8 ? zcol : zlimit - 8;
     u32x4 zreg[2][ZN];
-    auto fetch_z = [&](int fm, u32x4(&dst)[ZN]) {
+    auto fetch_z = [&](int blk, u32x4(&dst)[ZN]) {
 #pragma unroll
       for (int it = 0; it < ZN; it++) {
-        int m = m_base + fm * 32 + it * ZR + zr;
+        int m = m_base + blk * 32 + it * ZR + zr;
         m = m < row_end ? m : row_end - 1;
         dst[it] = *(const u32x4*)(p.zin + (int64_t)m * p.zin_stride + zcol_c);
       }
     };
     fetch_z(0, zreg[0]);
-    if constexpr (FM > 1) fetch_z(1, zreg[1]);
+    if constexpr (NB > 1) fetch_z(1, zreg[1]);
     wait_lds_all();
     lds_barrier();  // every wave has finished reading the ring
-    static_for<FM>([&](auto fm_c) {
-      constexpr int fm = decltype(fm_c)::value;
+    static_for<NB>([&](auto blk_c) {
+      constexpr int blk = decltype(blk_c)::value;
 #pragma unroll
       for (int it = 0; it < ZN; it++) {
         const int r = it * ZR + zr;
-        *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4)) = zreg[fm & 1][it];
+        *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4)) = zreg[blk & 1][it];
       }
-      if constexpr (fm + 2 < FM) fetch_z(fm + 2, zreg[fm & 1]);
-      const int mrow = lane & 31;
-      const int m = m_base + fm * 32 + mrow;
-      const bool mvalid = m < row_end;
-      float sc = 0.f, dsum = 0.f;
-      if (mvalid) sc = p.scores[p.sidx[m]];
-      static_for<FN * 4>([&](auto q_c) {
-        constexpr int fn = decltype(q_c)::value / 4, rg = decltype(q_c)::value % 4;
-        const int il = fn * 32 + 8 * rg + 4 * (lane >> 5);  // first of this lane's 4 dy1 columns (wave-local)
-        const int zbyte = il * 2 * ZW;                      // their z bytes inside the staged row
-        char* zaddr = zbuf + mrow * ZB + (((zbyte >> 4) ^ (mrow & ZSW)) << 4) + (zbyte & 15);
-        float ys[4];
-        if constexpr (GLU) {
-          const u32x4 zz = *(const u32x4*)zaddr;
-          u32x4 dzv;
+      if constexpr (blk + 2 < NB) fetch_z(blk + 2, zreg[blk & 1]);
+      static_for<RB>([&](auto sub_c) {
+        constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
+        const int mrow = sub * FR + AL::row(lane);  // row inside the staged batch
+        const int m = m_base + blk * 32 + mrow;
+        const bool mvalid = m < row_end;
+        float sc = 0.f, dsum = 0.f;
+        if (mvalid) sc = p.scores[p.sidx[m]];
+        static_for<FN * QPF>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+          const int il = fn * FR + AL::col(rg, lane);  // first of this lane's 4 dy1 columns (wave-local)
+          const int zbyte = il * 2 * ZW;                // their z bytes inside the staged row
+          char* zaddr = zbuf + mrow * ZB + (((zbyte >> 4) ^ (mrow & ZSW)) << 4) + (zbyte & 15);
+          float ys[4];
+          if constexpr (GLU) {
+            const u32x4 zz = *(const u32x4*)zaddr;
+            u32x4 dzv;
 #pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const float dy = acc[fn][fm][4 * rg + q];
-            const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
-            float f, fp;
-            pointwise_grad<PW>(g, f, fp);
-            const float y1v = f * u;
-            if (n_base + il + q < p.N) dsum += dy * y1v;
-            const float sd = sc * dy;
-            dzv[q] = pack_bf16x2(sd * u * fp, sd * f);
-            ys[q] = sc * y1v;
-          }
-          *(u32x4*)zaddr = dzv;
-        } else {
-          const u32x2 zz = *(const u32x2*)zaddr;
-          float dzf[4];
+            for (int q = 0; q < 4; q++) {
+              const float dy = acc[fn][fm][4 * rg + q];
+              const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
+              float f, fp;
+              pointwise_grad<PW>(g, f, fp);
+              const float y1v = f * u;
+              if (n_base + il + q < p.N) dsum += dy * y1v;
+              const float sd = sc * dy;
+              dzv[q] = pack_bf16x2(sd * u * fp, sd * f);
+              ys[q] = sc * y1v;
+            }
+            *(u32x4*)zaddr = dzv;
+          } else {
+            const u32x2 zz = *(const u32x2*)zaddr;
+            float dzf[4];
 #pragma unroll
-          for (int q = 0; q < 4; q++) {
-            const float dy = acc[fn][fm][4 * rg + q];
-            const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
-            float f, fp;
-            pointwise_grad<PW>(t, f, fp);
-            if (n_base + il + q < p.N) dsum += dy * f;
-            dzf[q] = sc * dy * fp;
-            ys[q] = sc * f;
+            for (int q = 0; q < 4; q++) {
+              const float dy = acc[fn][fm][4 * rg + q];
+              const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
+              float f, fp;
+              pointwise_grad<PW>(t, f, fp);
+              if (n_base + il + q < p.N) dsum += dy * f;
+              dzf[q] = sc * dy * fp;
+              ys[q] = sc * f;
+            }
+            *(u32x2*)zaddr = u32x2{pack_bf16x2(dzf[0], dzf[1]), pack_bf16x2(dzf[2], dzf[3])};
           }
-          *(u32x2*)zaddr = u32x2{pack_bf16x2(dzf[0], dzf[1]), pack_bf16x2(dzf[2], dzf[3])};
-        }
-        u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
-        epi_park_y<YB>(ybuf, mrow, il * 2, yv);
+          u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
+          epi_park_y<YB>(ybuf, mrow, il * 2, yv);
+        });
+        // the 64 / FR lanes that share a token row hold disjoint columns: add their partial sums
+        dsum += __shfl_xor(dsum, 32, 64);
+        if constexpr (FR == 16) dsum += __shfl_xor(dsum, 16, 64);
+        if (mvalid && lane < FR) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
       });
-      dsum += __shfl_xor(dsum, 32, 64);
-      if (mvalid && lane < 32) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
 #pragma unroll
       for (int it = 0; it < ZN; it++) {
         const int r = it * ZR + zr;
         const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4));
-        const int mm = m_base + fm * 32 + r;
+        const int mm = m_base + blk * 32 + r;
         if (mm < row_end && zcol < zlimit) *(u32x4*)(p.out0 + (int64_t)mm * p.out0_stride + zcol) = v;
       }
 #pragma unroll
       for (int it = 0; it < YN; it++) {
         const int r = it * YR + yr;
         const u32x4 v = *(const u32x4*)(ybuf + r * YB + ((yc ^ ((r >> 1) & (YL < 8 ? YL - 1 : 7))) << 4));
-        const int mm = m_base + fm * 32 + r, col = n_base + yc * 8;
+        const int mm = m_base + blk * 32 + r, col = n_base + yc * 8;
         if (mm < row_end && col < p.N) *(u32x4*)(p.out1 + (int64_t)mm * p.out1_stride + col) = v;
       }
     });
@@ -331,7 +355,8 @@ template <class C, int ROLE, int ACT>
 __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMParams p) {
   static_assert(ROLE == ROLE_UP_FWD || ROLE == ROLE_PLAIN, "the dz epilogue is not built as a stream");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK, SLICES = C::BK / 16;
+  using Mma = typename C::Mma;
+  constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK;
   const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -446,11 +471,11 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
   const int S_total = p.Kdim / BK;
 
   // ---- per-lane LDS fragment offsets (bytes inside a ring slot) ----
-  int p_off[SLICES];
-  int q_off[C::QMN ? 2 * FN : SLICES];
+  int p_off[C::KSL];
+  int q_off[C::QMN ? 2 * FN : C::KSL];
   fragment_offsets<C>(wm, wn, lane, p_off, q_off);
 
-  f32x16 acc[FN][FM];  // started from zero by the first slice of every tile
+  typename Mma::Acc acc[FN][FM];  // started from zero by the first k-slice of every tile
 
   constexpr int Q_RING = C::P_SLOTS * C::P_STAGE;
   int p_stage = 0, q_stage = 0;  // stages issued to each stream for the tile it is on
@@ -476,19 +501,9 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
       point_q(nxt);
     }
   };
-  auto load = [&](int p_slot, int q_slot, int ks, bf16x8(&qf)[FN], bf16x8(&pf)[FM]) {
-    const char* sp = smem + p_slot * C::P_STAGE;
-    const char* sq = smem + Q_RING + q_slot * C::Q_STAGE;
-#pragma unroll
-    for (int fm = 0; fm < FM; fm++) pf[fm] = lds_read_b128(sp + p_off[ks] + fm * 32 * C::KROW);
-#pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
-      if constexpr (!C::QMN) {
-        qf[fn] = lds_read_b128(sq + q_off[ks] + fn * 32 * C::KROW);
-      } else {
-        qf[fn] = lds_read_tr2(sq + q_off[fn * 2] + ks * 16 * C::ROWB, sq + q_off[fn * 2 + 1] + ks * 16 * C::ROWB);
-      }
-    }
+  auto load = [&](int p_slot, int q_slot, auto step_c, bf16x8(&qf)[FN], bf16x8(&pf)[C::NP]) {
+    read_fragments<C, decltype(step_c)::value>(smem + p_slot * C::P_STAGE, smem + Q_RING + q_slot * C::Q_STAGE, p_off,
+                                               q_off, qf, pf);
   };
   // the rows loaded in tile_end are complete here; naming them in an asm statement makes this the place where the
   // compiler waits for them
@@ -512,7 +527,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     // waves 0..NW/2-1 park in the vacated P slot, the others in the vacated Q slot
     char* region = wave < C::NW / 2 ? smem + p_slot * C::P_STAGE + wave * PARK
                                     : smem + Q_RING + q_slot * C::Q_STAGE + (wave - C::NW / 2) * PARK;
-    forward_epilogue_rows<C::TN, FM, FN, ROLE == ROLE_UP_FWD, ACT>(acc, region, opaque_lane(), ea);
+    forward_epilogue_rows<Mma, C::TM, C::TN, ROLE == ROLE_UP_FWD, ACT>(acc, region, opaque_lane(), ea);
     if (!more) return false;
     cur = nxt;
     nxt = nn;
@@ -522,7 +537,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     token_rows(nxt, rows_next);
     return true;
   };
-  gemm_stream_loop<FN, FM, (C::QMN ? 2 * FN : FN) + FM, C::P_INSTR, C::Q_INSTR, SLICES>(
+  gemm_stream_loop<FN, C::NP, (C::QMN ? 2 * FN : FN) + C::NP, C::P_INSTR, C::Q_INSTR, C::STEPS, Mma>(
       S_total, acc, issue_p, issue_q, load, issued_p, issued_q, first_boundary, tile_end);
 }
 
