@@ -58,7 +58,6 @@ const char* smoe_last_error(void);
  *   "gemm_stream"          SMOE_GEMM_STREAM          1: token-grouped GEMMs run as tile streams (default); 0: one tile
  *                                                    per workgroup
  *   "gemm_stream_grid"     SMOE_GEMM_STREAM_GRID     workgroups of a tile-stream launch; 0 = one per compute unit
- *   "varlen_k_tiles"       SMOE_VARLEN_K_TILES       tiles per workgroup of the weight-gradient GEMMs; 0 = by shape
  *   "varlen_k_tile_order"  SMOE_VARLEN_K_TILE_ORDER  2 blocked (default), 0 round-robin, 1 whole experts per XCD */
 int smoe_set_tuning(const char* name, int value);
 

@@ -213,19 +213,8 @@ SMOE_DEV void mma_step_refill(typename Mma::Acc (&acc)[NQ][NP * Mma::PH], typena
 //                                 stage s into ring slot buf; called with i ascending, stages in order
 //   load(buf, s, step, qf, pf)    read the fragments step `step` (a compile-time constant) needs from ring slot buf
 //                                 into the fragment sets handed in
-// The first stages of a main loop, issued on their own: a kernel that works through several tiles starts the next
-// tile's loads before the finished tile's epilogue and enters gemm_mainloop<..., PROLOGUE = false> behind it.
-template <int LPS, int NSTAGE, class Issue>
-SMOE_DEV void gemm_mainloop_prologue(const int S, Issue&& issue) {
-  const int pre = S < NSTAGE ? S : NSTAGE;
-  for (int s = 0; s < pre; s++) static_for<LPS>([&](auto i_c) { issue(s, s, i_c); });
-}
-
-// PROLOGUE = false: the first min(S, NSTAGE) stages have been issued by gemm_mainloop_prologue, possibly with other
-// vector-memory operations (an epilogue's stores) behind them: the first wait is then for everything, because loads
-// and stores may retire out of order and a counted wait could not tell which are left.
-template <int NQ, int NP, int NREADS, int LPS, int STEPS, int NSTAGE, class Mma = Bf16Mma, int RPM = 1,
-          bool PROLOGUE = true, class Issue, class Load>
+template <int NQ, int NP, int NREADS, int LPS, int STEPS, int NSTAGE, class Mma = Bf16Mma, int RPM = 1, class Issue,
+          class Load>
 SMOE_DEV void gemm_mainloop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::PH], Issue&& issue, Load&& load) {
   if (S <= 0) return;
   static_assert((NSTAGE - 1) * LPS < 64, "too many loads in flight for vmcnt");
@@ -234,8 +223,7 @@ SMOE_DEV void gemm_mainloop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::
   constexpr int NM = NQ * NP, LAST = STEPS - 1;
   auto issue_all = [&](int buf, int s) { static_for<LPS>([&](auto i_c) { issue(buf, s, i_c); }); };
   const int pre = S < NSTAGE ? S : NSTAGE;
-  if constexpr (PROLOGUE)
-    for (int s = 0; s < pre; s++) issue_all(s, s);
+  for (int s = 0; s < pre; s++) issue_all(s, s);
 
   auto wait_next_stage = [&](int younger) {  // `younger` stages were issued after the one we need
     if constexpr (NSTAGE >= 6) if (younger >= 4) { wait_vmem_upto<4 * LPS>(); return; }
@@ -257,8 +245,7 @@ SMOE_DEV void gemm_mainloop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::
   };
   constexpr std::integral_constant<int, 0> step0{};
 
-  if constexpr (PROLOGUE) wait_next_stage(pre - 1);
-  else wait_vmem_all();
+  wait_next_stage(pre - 1);
   lds_barrier();
   read_step(0, 0, step0);
   int buf = 0;
@@ -747,7 +734,6 @@ SMOE_DEV void forward_epilogue_rows(typename Mma::Acc (&acc)[TN / Mma::FR][TM / 
 struct Tuning {
   int gemm_stream;          // 1 (default): up-projection forward, down-projection forward, dz and dx run as tile streams
   int gemm_stream_grid;     // workgroups of the tile-stream kernels; 0 (default) = one per compute unit
-  int varlen_k_tiles;       // tiles per workgroup of the weight-gradient kernels; 0 (default) = chosen from the shape
   int varlen_k_tile_order;  // 2 blocked (default), 0 single tiles round-robin over the XCDs, 1 whole experts per XCD
   int experiment;           // scratch knob for kernel experiments (no effect in a release build)
 };

@@ -24,8 +24,6 @@ struct VarlenKParams {
   int E;
   int uniform_rows;  // off == nullptr: group e is rows [e * uniform_rows, min((e + 1) * uniform_rows, total_rows))
   int64_t total_rows;
-  int tiles_per_wg;  // several-tiles-per-workgroup kernel: slots a workgroup works through
-  int64_t slots;    // workgroup slots of the tile order (= the grid of the one-tile-per-workgroup launch)
   int xcd_chunked;  // tile order: 2 blocked, 1 contiguous tile range per XCD (probe: unbalanced on skewed experts), 0 round-robin
 };
 
@@ -44,8 +42,6 @@ struct KCfg {
   static constexpr int STAGE = R_STAGE + S_STAGE;
   static constexpr int EPI = NW * TA * (TB * 2 + 16);
   static constexpr int SMEM = NSTAGE * STAGE > EPI ? NSTAGE * STAGE : EPI;
-  // several tiles per workgroup: the ring plus, per wavefront, 32 parked rows of the epilogue (unpadded, swizzled)
-  static constexpr int SMEM_MULTI = NSTAGE * STAGE + NW * 32 * TB * 2;
   static constexpr int R_ROWB = BA * 2, S_ROWB = BB * 2;
   static constexpr int R_LPR = R_ROWB / 16, S_LPR = S_ROWB / 16;
   static constexpr int R_RPI = 64 / R_LPR, S_RPI = 64 / S_LPR;
@@ -296,235 +292,6 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
                                p.NA, b0 + wb * C::TB, p.NB);
 }
 
-// ---- several tiles per workgroup ------------------------------------------------------------------------------------
-// Workgroup b works through the slots b, b + gridDim.x, ... (at most p.tiles_per_wg of them).  Behind a tile's main
-// loop the NEXT tile's first two stages are issued, then the finished tile's epilogue runs out of LDS of its own (not
-// the ring), so those loads fly under the epilogue and the workgroup turnaround between two tiles (release, dispatch,
-// first dependent loads: 10 us per tile for one-tile workgroups) is paid once per workgroup.
-template <class C>
-__global__ __launch_bounds__(C::NT) void varlen_k_multi_kernel(const VarlenKParams p) {
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  using Mma = typename C::Mma;
-  using AL = AccLayout<Mma>;
-  constexpr int FA = C::FA, FB = C::FB, BK = C::BK, NSTAGE = C::NSTAGE, FR = C::FR, QPF = AL::QPF;
-  const uint32_t smem_base = lds_address(smem);
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wa = wave % C::WA, wb = wave / C::WA;
-
-  // transpose-load fragment offsets (bytes inside a stage)
-  int r_off[2 * FA], s_off[2 * FB];
-  {
-    // a fragment lane supplies column l % FR and the contraction elements 8 * (l / FR) + 0..7 of the k-slice; the
-    // transpose load hands lane i of a 16-lane group column i of the 4 (k) x 16 block its lanes' addresses name
-    const int grp = lane >> 4, i16 = lane & 15;
-    const int kk = (C::FR == 32 ? 8 * (grp >> 1) : 8 * grp) + (i16 >> 2);
-#pragma unroll
-    for (int f = 0; f < FA; f++) {
-      const int c16 = (wa * C::TA) / 16 + (C::FR == 32 ? f * 2 + (grp & 1) : f);
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const int k = kk + 4 * h;
-        r_off[f * 2 + h] = k * C::R_ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
-      }
-    }
-#pragma unroll
-    for (int f = 0; f < FB; f++) {
-      const int c16 = (wb * C::TB) / 16 + (C::FR == 32 ? f * 2 + (grp & 1) : f);
-#pragma unroll
-      for (int h = 0; h < 2; h++) {
-        const int k = kk + 4 * h;
-        s_off[f * 2 + h] = C::R_STAGE + k * C::S_ROWB + ((c16 ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
-      }
-    }
-  }
-
-  typename Mma::Acc acc[FB][FA];
-  clear_accumulators<Mma>(acc);
-
-  static_assert(C::R_INSTR * C::R_RPI == C::S_INSTR * C::S_RPI, "both operands cover the same token rows per wave");
-  constexpr int RPW = C::R_INSTR * C::R_RPI;  // token rows per wave and stage
-  uint64_t zero = (uint64_t)smoe_zero_page;
-  asm volatile("" : "+s"(zero));
-  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
-  typedef int32_t __attribute__((ext_vector_type(RPW), aligned(4))) idx_run;
-  typedef const __attribute__((address_space(4))) idx_run* const_run_ptr;
-  const const_i32_ptr gidx = (const_i32_ptr)p.gidx;
-  const const_i32_ptr off = (const_i32_ptr)p.off;  // constant address space: scalar loads also behind a tile's stores
-
-  // ---- the tile whose stages are being issued ----
-  int e = 0, a0 = 0, b0 = 0, row_begin = 0, row_end = 0, S = 0;
-  const char* r_ptr[C::R_INSTR];
-  const char* s_ptr[C::S_INSTR];
-  const uint32_t r_row_bytes = (uint32_t)p.r_stride * 2u, s_row_bytes = (uint32_t)p.s_stride * 2u;
-  int tok[RPW], tok_next[RPW];
-  auto fetch = [&](int s, int(&dst)[RPW]) {
-    const int m0 = row_begin + s * BK + wave * RPW;
-    if (m0 + RPW <= row_end) {
-      if constexpr (C::R_GATHER || C::S_GATHER) {
-        const idx_run run = *(const_run_ptr)(gidx + m0);
-#pragma unroll
-        for (int j = 0; j < RPW; j++) dst[j] = run[j];
-      } else {
-#pragma unroll
-        for (int j = 0; j < RPW; j++) dst[j] = m0 + j;
-      }
-      return;
-    }
-    // the expert's last, ragged stage: rows past its end read the zero page.  The index array goes on behind the
-    // expert (the next expert's rows) up to total_rows, so the run is still ONE wide load wherever it stays inside
-    // the array; entries past the expert's end are discarded.
-    if constexpr (C::R_GATHER || C::S_GATHER) {
-      if ((int64_t)m0 + RPW <= p.total_rows) {
-        const idx_run run = *(const_run_ptr)(gidx + m0);
-#pragma unroll
-        for (int j = 0; j < RPW; j++) dst[j] = m0 + j < row_end ? run[j] : -1;
-        return;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < RPW; j++) {
-      const int m = m0 + j;
-      const int mc = m < row_end ? m : row_end - 1;
-      const int g = (C::R_GATHER || C::S_GATHER) ? gidx[mc] : mc;
-      dst[j] = m < row_end ? g : -1;
-    }
-  };
-  // decode slot v, take the expert's token range, form the per-lane pointers, request the first stage's rows
-  auto setup = [&](int64_t v) -> bool {
-    int ta, tb;
-    if (!decode_tile(p, v, e, ta, tb)) return false;
-    a0 = ta * C::BA;
-    b0 = tb * C::BB;
-    if (p.off != nullptr) {
-      row_begin = off[e];
-      row_end = off[e + 1];
-    } else {
-      row_begin = e * p.uniform_rows;
-      const int64_t end = (int64_t)(e + 1) * p.uniform_rows;
-      row_end = (int)(end < p.total_rows ? end : p.total_rows);
-    }
-    S = (row_end - row_begin + BK - 1) / BK;
-    int pl = threadIdx.x & 63;
-    asm volatile("" : "+v"(pl));  // formed here, once per tile, not carried through the main loop
-#pragma unroll
-    for (int i = 0; i < C::R_INSTR; i++) {
-      const int kl = (wave * C::R_INSTR + i) * C::R_RPI + pl / C::R_LPR;
-      const int phys16 = pl % C::R_LPR;
-      const int log32 = (phys16 >> 1) ^ mnswz(kl);
-      int a = a0 + ((log32 << 1) | (phys16 & 1)) * 8;
-      a = a <= p.NA - 8 ? a : p.NA - 8;
-      const int64_t row = C::R_GATHER ? 0 : row_begin + wave * RPW + i * C::R_RPI + pl / C::R_LPR;
-      r_ptr[i] = (const char*)(p.R + row * p.r_stride + a);
-    }
-#pragma unroll
-    for (int i = 0; i < C::S_INSTR; i++) {
-      const int kl = (wave * C::S_INSTR + i) * C::S_RPI + pl / C::S_LPR;
-      const int phys16 = pl % C::S_LPR;
-      const int log32 = (phys16 >> 1) ^ mnswz(kl);
-      int b = b0 + ((log32 << 1) | (phys16 & 1)) * 8;
-      b = b <= p.NB - 8 ? b : p.NB - 8;
-      const int64_t row = C::S_GATHER ? 0 : row_begin + wave * RPW + i * C::S_RPI + pl / C::S_LPR;
-      s_ptr[i] = (const char*)(p.S + row * p.s_stride + b);
-    }
-    if (S > 0) fetch(0, tok);
-    return true;
-  };
-  auto piece = [&](const char* lane_ptr, uint32_t row_bytes, bool gather, int rpi, int lpr, int s, int i) {
-    const int sel = lane / lpr;
-    int t = tok[i * rpi];
-#pragma unroll
-    for (int j = 1; j < rpi; j++) t = sel == j ? tok[i * rpi + j] : t;
-    const uint32_t row = gather ? (uint32_t)t : (uint32_t)(s * BK);
-    const uint64_t src = (uint64_t)row * row_bytes + (uint64_t)lane_ptr;
-    return (const uint16_t*)(t < 0 ? zero : src);
-  };
-  auto issue = [&](int buf, int s, auto i_c) {
-    constexpr int i = decltype(i_c)::value;
-    const uint32_t base = smem_base + buf * C::STAGE;
-    if constexpr (i == 0)
-      if (s + 1 < S) fetch(s + 1, tok_next);  // stages are issued in order
-    if constexpr (i < C::R_INSTR) {
-      load16_to_lds(piece(r_ptr[i], r_row_bytes, C::R_GATHER, C::R_RPI, C::R_LPR, s, i),
-                    base + (wave * C::R_INSTR + i) * 1024);
-    } else {
-      constexpr int j = i - C::R_INSTR;
-      load16_to_lds(piece(s_ptr[j], s_row_bytes, C::S_GATHER, C::S_RPI, C::S_LPR, s, j),
-                    base + C::R_STAGE + (wave * C::S_INSTR + j) * 1024);
-    }
-    if constexpr (i == C::R_INSTR + C::S_INSTR - 1) {
-#pragma unroll
-      for (int j = 0; j < RPW; j++) tok[j] = tok_next[j];
-    }
-  };
-  auto load = [&](int buf, int /*s*/, auto step_c, bf16x8(&sf)[FB], bf16x8(&rf)[C::NP]) {
-    constexpr int step = decltype(step_c)::value;
-    constexpr int kofs = Mma::kslice(step) * Mma::KSTEP, ph = Mma::phalf(step);
-    const char* st = smem + buf * C::STAGE;
-#pragma unroll
-    for (int pp = 0; pp < C::NP; pp++) {
-      const int f = ph * C::NP + pp;
-      rf[pp] = lds_read_tr2(st + r_off[f * 2] + kofs * C::R_ROWB, st + r_off[f * 2 + 1] + kofs * C::R_ROWB);
-    }
-    if constexpr (Mma::reads_q(step)) {
-#pragma unroll
-      for (int f = 0; f < FB; f++)
-        sf[f] = lds_read_tr2(st + s_off[f * 2] + kofs * C::S_ROWB, st + s_off[f * 2 + 1] + kofs * C::S_ROWB);
-    }
-  };
-
-  int64_t v = blockIdx.x;
-  bool have = setup(v);
-  if (have) gemm_mainloop_prologue<C::R_INSTR + C::S_INSTR, NSTAGE>(S, issue);
-  constexpr int RB = C::TB * 2;  // bytes of a parked row
-  static_assert(RB == 128, "the parked rows are 8 chunks of 16 bytes");
-  for (int k = 1; have; k++) {
-    const int cur_e = e, cur_a0 = a0, cur_b0 = b0;
-    gemm_mainloop<FB, C::NP, 2 * (C::NP + FB), C::R_INSTR + C::S_INSTR, C::STEPS, NSTAGE, Mma, 2, false>(S, acc, issue, load);
-    wait_lds_all();
-    lds_barrier();  // every wave has read the ring's last stage: the next tile may land in it
-    v += gridDim.x;
-    have = k < p.tiles_per_wg && setup(v);
-    if (have) gemm_mainloop_prologue<C::R_INSTR + C::S_INSTR, NSTAGE>(S, issue);
-
-    // epilogue of the finished tile (also the zeros of an expert without tokens): one 32-row fragment row at a time
-    // through this wave's own 4 KiB behind the ring; 16-byte chunk c of row r sits at c ^ ((r >> 1) & 7)
-    int el = threadIdx.x & 63;
-    asm volatile("" : "+v"(el));  // keeps the epilogue's per-lane addresses from being formed ahead of the main loop
-    char* region = smem + NSTAGE * C::STAGE + wave * (32 * RB);
-    uint16_t* out = p.out + (int64_t)cur_e * p.out_stride_e;
-    const int a_base = cur_a0 + wa * C::TA, b_base = cur_b0 + wb * C::TB;
-    const int rr = el >> 3, cc = el & 7;
-    const int col = b_base + cc * 8;
-    static_for<C::TA / 32>([&](auto blk_c) {  // 32 output rows at a time
-      constexpr int blk = decltype(blk_c)::value;
-      static_for<32 / FR>([&](auto sub_c) {
-        constexpr int sub = decltype(sub_c)::value, fa = blk * (32 / FR) + sub;
-        static_for<FB * QPF>([&](auto q_c) {
-          constexpr int fb = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-          u32x2 pv = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
-                      pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
-          epi_park_y<RB>(region, sub * FR + AL::row(el), (fb * FR + AL::col(rg, el)) * 2, pv);
-        });
-      });
-      u32x4 rows[4];
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int r = q * 8 + rr;
-        rows[q] = *(const u32x4*)(region + r * RB + ((cc ^ ((r >> 1) & 7)) << 4));
-      }
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        const int row = a_base + blk * 32 + q * 8 + rr;
-        if (row < p.NA && col < p.NB) *(u32x4*)(out + (int64_t)row * p.out_stride_row + col) = rows[q];
-      }
-      __builtin_amdgcn_sched_barrier(0);  // batch by batch
-    });
-    clear_accumulators<Mma>(acc);
-  }
-  wait_vmem_all();
-}
-
 template <class C>
 static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   static LdsLimitOnce lds_limit;
@@ -552,28 +319,6 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   // the kernel forms source addresses as row * (row stride in bytes, 32 bits) + column pointer
   SMOE_REQUIRE(p.r_stride > 0 && p.r_stride < (1ll << 31) && p.s_stride > 0 && p.s_stride < (1ll << 31),
                SMOE_ERR_UNSUPPORTED, "weight-grad gemm: operand row stride out of range");
-  p.slots = grid;
-  p.tiles_per_wg = 1;
-  if constexpr (C::NSTAGE == 2 && C::NW == 8 && C::SMEM_MULTI <= 160 * 1024) {
-    // Tiles a workgroup works through: 2 when the experts average at most 1024 rows (tiles of at most 16 stages, of
-    // which the turnaround between two workgroups is a quarter: 2 % of a step at 512 rows per expert, nothing at
-    // 2048), else 1; the varlen_k_tiles knob overrides.  The grid stays a multiple of 256 slots so that a
-    // workgroup's tiles keep its XCD and its place in the blocked order.
-    const int knob = tuning().varlen_k_tiles;
-    const int want = knob > 0 ? knob : (p.total_rows <= (int64_t)1024 * p.E ? 2 : 1);
-    if (want > 1 && grid >= 512 && grid % 256 == 0) {
-      const int64_t rounds = grid / 256;
-      const int64_t wg_rounds = (rounds + want - 1) / want;
-      static LdsLimitOnce lds_limit_multi;
-      auto mkern = varlen_k_multi_kernel<C>;
-      const int rc_attr = lds_limit_multi.ensure((const void*)mkern, C::SMEM_MULTI);
-      if (rc_attr) return rc_attr;
-      p.tiles_per_wg = (int)((rounds + wg_rounds - 1) / wg_rounds);
-      hipLaunchKernelGGL(mkern, dim3((unsigned)(wg_rounds * 256)), dim3(C::NT), C::SMEM_MULTI, st, p);
-      SMOE_LAUNCH_CHECK();
-      return SMOE_OK;
-    }
-  }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
