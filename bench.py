@@ -33,6 +33,9 @@ PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA peak
 
 CONFIGS = {
     "C2": dict(T=32768, H=4096, I=1024, E=128, K=8, zipf=False),
+    # the reference's published shapes with short down-projection contractions (its tput.png: I = 256 / 512)
+    "I256": dict(T=32768, H=4096, I=256, E=256, K=16, zipf=False),
+    "I512": dict(T=32768, H=4096, I=512, E=128, K=8, zipf=False),
     "C3": dict(T=32768, H=4096, I=1536, E=128, K=8, zipf=True),
     "C4": dict(T=16384, H=4096, I=1024, E=256, K=8, zipf=False, rounding="nr", tile=128),
 }
@@ -54,23 +57,30 @@ def make_inputs(cfg, dev, seed=0):
     return x, wr, w1, w2, dout
 
 
-def time_region(fn, steps, warmup):
-    """ms per call: `warmup` untimed calls, then `steps` calls between two events on the current stream."""
+def time_region(fn, steps, warmup, per_step=False):
+    """ms per call: `warmup` untimed calls, then `steps` calls between two events on the current stream.  With
+    per_step=True an event is recorded between the calls as well and the list of per-call times is returned too."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1 if per_step else 2)]
     t0 = time.perf_counter()
-    e0.record()
-    for _ in range(steps):
+    marks[0].record()
+    for k in range(steps):
         fn()
-    e1.record()
+        if per_step:
+            marks[k + 1].record()
+    if not per_step:
+        marks[1].record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    return e0.elapsed_time(e1) / steps, wall
+    mean = marks[0].elapsed_time(marks[-1]) / steps
+    if per_step:
+        return mean, wall, [marks[k].elapsed_time(marks[k + 1]) for k in range(steps)]
+    return mean, wall
 
 
-def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
+def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=False):
     """Time every operator of the path on its own (events on the launch stream) and return a list of dicts with
     algorithmic FLOPs / bytes.  The grouped GEMM ops launch a tile-map builder (~5 us) next to the GEMM kernel."""
     from sonicmoe.functional import _build_metadata, backward, forward
@@ -123,7 +133,9 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None):
             ("switch_loss_fwd", lambda: forward._switch_loss_fwd(logits, freq, sl_acc, sl_aux), None, T * E * 2),
             ("switch_loss_bwd", lambda: backward._switch_loss_bwd(logits, freq, sl_acc, sl_g, dlog), None, T * E * 4),
         ]
-        if H % 128 == 0 and I % 128 == 0 and only is None:
+        if gemms_only:
+            ops = [o for o in ops if o[2] and "router_gemm" not in o[0]]
+        if H % 128 == 0 and I % 128 == 0 and only is None and not gemms_only:
             # fp8 forward (config 5 = this shape with block-scaled e4m3 operands): quantisers and the two fp8 GEMMs
             from sonicmoe.functional import fp8
 
@@ -233,6 +245,30 @@ def cpu_baseline(cfg, budget_s=20.0):
         step()
         times.append(time.perf_counter() - t0)
     best = sorted(times)[len(times) // 2]
+
+    # the reference's own CPU-runnable case, whole: fp32, T=1024 H=512 I=256 E=8 K=2, loss = sum(out * g), seed 0
+    c1 = dict(T=1024, H=512, I=256, E=8, K=2)
+    torch.manual_seed(0)
+    x1 = torch.randn(c1["T"], c1["H"], requires_grad=True)
+    wr1 = (0.02 * torch.randn(c1["E"], c1["H"])).requires_grad_()
+    w11 = (0.02 * torch.randn(c1["E"], 2 * c1["I"], c1["H"])).requires_grad_()
+    w21 = (0.02 * torch.randn(c1["E"], c1["H"], c1["I"])).requires_grad_()
+    g1 = torch.randn(c1["T"], c1["H"])
+
+    def step1():
+        out, _, _ = M.moe_torch_backend(x1, wr1, w11, w21, c1["K"])
+        (out * g1).sum().backward()
+        for t in (x1, wr1, w11, w21):
+            t.grad = None
+
+    step1()
+    times1 = []
+    for _ in range(7):
+        t0 = time.perf_counter()
+        step1()
+        times1.append(time.perf_counter() - t0)
+    best1 = sorted(times1)[len(times1) // 2]
+    flops1 = 18.0 * c1["T"] * c1["K"] * c1["I"] * c1["H"]
     return dict(
         value=round(flops / best / 1e12, 4),
         unit="TFLOP/s",
@@ -240,40 +276,27 @@ def cpu_baseline(cfg, budget_s=20.0):
         kind="port",
         sample=f"oracle.moe_torch_backend fp32 fwd+bwd, T={T} tokens (1/{cfg['T'] // T} of the workload's tokens), "
         f"H={H} I={I} E={E} K={K}; median of {len(times)} passes, {best * 1e3:.0f} ms per pass",
+        config1=dict(
+            workload="C1: fp32 fwd+bwd on the host, T=1024 H=512 I=256 E=8 K=2, SwiGLU, no bias, loss = sum(out * g), seed 0",
+            ms_per_step=round(best1 * 1e3, 3),
+            tflops=round(flops1 / best1 / 1e12, 4),
+            passes=len(times1),
+        ),
     )
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-breakdown", action="store_true")
-    ap.add_argument("--pmc-target", default=None, choices=sorted(SINGLE_KERNEL_OPS),
-                    help="run only this operator (3 launches) and a 1 GiB copy: the workload of the rocprofv3 --pmc passes")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        print("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py needs a GPU", file=sys.stderr)
-        sys.exit(2)
-
+def measure_layer(cfg, name, dev, steps, warmup):
+    """Forward and forward+backward of the whole layer at one configuration.  Returns (record, tensors) where tensors are
+    the inputs, kept for the per-kernel breakdown of the headline configuration."""
     from sonicmoe.enums import ActivationType
     from sonicmoe.functional import (
         TC_Softmax_Topk_Router_Function,
         _build_metadata,
         _ExpertsFunction,
+        moe_general_routing_inputs,
         moe_TC_softmax_topk_layer,
     )
 
-    cfg = CONFIGS[a.config]
-    dev = torch.device("cuda:0")
-    if a.pmc_target:
-        pmc_target(cfg, a.pmc_target, dev)
-        return
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     x, wr, w1, w2, dout = make_inputs(cfg, dev)
     stream = torch.cuda.current_stream().cuda_stream
@@ -282,10 +305,9 @@ def main():
 
     rounding = cfg.get("rounding")
     if rounding:
-        from sonicmoe.functional import moe_general_routing_inputs
         from sonicmoe.routing import token_choice_rounding
 
-        with torch.no_grad():  # the rounding router is host-side torch and outside the timed region, as in the reference
+        with torch.no_grad():  # the rounding router is outside the timed region, as in the reference's benchmark
             r_scores, r_tok, r_exp = token_choice_rounding(torch.nn.functional.linear(x, wr), K, cfg["tile"], rounding)
         r_scores = r_scores.float().requires_grad_()
 
@@ -313,39 +335,104 @@ def main():
 
     TK = r_tok.numel() if rounding else T * K
     flops_fwd, flops_all = 6.0 * TK * I * H, 18.0 * TK * I * H
-    fwd_ms, _ = time_region(fwd_only, a.steps, a.warmup)
-    ms, wall_ms = time_region(fwd_bwd, a.steps, a.warmup)
+    fwd_ms, _ = time_region(fwd_only, steps, warmup)
+    ms, wall_ms, per_step = time_region(fwd_bwd, steps, warmup, per_step=True)
+    per_step.sort()
+    # peak memory of one step above what is resident between steps (inputs, weights): activations kept for the backward
+    # pass, transient buffers and the gradients while they are being produced
+    torch.cuda.synchronize()
+    resident = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    o = layer()
+    torch.cuda.synchronize()
+    held_for_backward = torch.cuda.memory_allocated() - resident - o.numel() * o.element_size()
+    peak_forward = torch.cuda.max_memory_allocated() - resident
+    torch.autograd.grad(o, [x, r_scores, w1, w2] if rounding else [x, wr, w1, w2], grad_outputs=dout)
+    torch.cuda.synchronize()
+    peak_step = torch.cuda.max_memory_allocated() - resident
+    del o
     tflops = flops_all / ms / 1e9
-    log(f"{a.config}: fwd {fwd_ms:.3f} ms ({flops_fwd / fwd_ms / 1e9:.1f} TFLOP/s), fwd+bwd {ms:.3f} ms "
-        f"({tflops:.1f} TFLOP/s = {100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak), host wall {wall_ms:.3f} ms/step")
+    rec = dict(
+        workload=f"{name}: MoE layer fwd+bwd, T={T} H={H} I={I} E={E} K={K}, SwiGLU, no bias, token-choice softmax "
+        f"top-k router{' with Zipf logit bias' if cfg['zipf'] else ''}"
+        f"{' then token rounding (' + rounding + ', tile 128), ' + str(TK) + ' routed pairs, general-routing entry' if rounding else ''}"
+        f"; x,dout~N(0,1), weights~N(0,0.02), seed 0",
+        flops_per_step=flops_all,
+        ms_per_step=round(ms, 4),
+        ms_per_step_median=round(per_step[len(per_step) // 2], 4),
+        ms_per_step_min=round(per_step[0], 4),
+        tflops=round(tflops, 2),
+        frac_of_peak=round(tflops / PEAK_BF16_TFLOPS, 4),
+        fwd_ms=round(fwd_ms, 4),
+        fwd_tflops=round(flops_fwd / fwd_ms / 1e9, 2),
+        host_wall_ms_per_step=round(wall_ms, 4),
+        activation_bytes_held_for_backward=int(held_for_backward),
+        peak_bytes_forward=int(peak_forward),
+        peak_bytes_step=int(peak_step),
+    )
+    log(f"{name}: fwd {fwd_ms:.3f} ms ({flops_fwd / fwd_ms / 1e9:.1f} TFLOP/s), fwd+bwd {ms:.3f} ms mean / "
+        f"{rec['ms_per_step_median']:.3f} median / {rec['ms_per_step_min']:.3f} min ({tflops:.1f} TFLOP/s = "
+        f"{100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak); kept for backward "
+        f"{held_for_backward / 2**30:.2f} GiB, peak of a step {peak_step / 2**30:.2f} GiB above the resident tensors")
+    return rec, dict(x=x, wr=wr, w1=w1, w2=w2, dout=dout, layer=layer, fwd_only=fwd_only, flops_fwd=flops_fwd)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="C2", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-breakdown", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the extra lines (C3, C4 layer times; per-kernel rows of the short-contraction shapes)")
+    ap.add_argument("--pmc-target", default=None, choices=sorted(SINGLE_KERNEL_OPS),
+                    help="run only this operator (3 launches) and a 1 GiB copy: the workload of the rocprofv3 --pmc passes")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one MI355X: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    cfg = CONFIGS[a.config]
+    dev = torch.device("cuda:0")
+    if a.pmc_target:
+        pmc_target(cfg, a.pmc_target, dev)
+        return
+    T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    rec, t = measure_layer(cfg, a.config, dev, a.steps, a.warmup)
+    rounding = cfg.get("rounding")
 
     fp8_info = None
     if not rounding and not cfg["zipf"] and H % 128 == 0 and I % 128 == 0:
         from sonicmoe import enable_fp8_forward
+        from sonicmoe.functional.fp8 import cache_quantized_weights
 
         with torch.no_grad():
-            ref_out = layer()
-            from sonicmoe.functional.fp8 import cache_quantized_weights
-
+            ref_out = t["layer"]()
             with enable_fp8_forward():
-                fp8_out = layer()
+                fp8_out = t["layer"]()
                 with cache_quantized_weights(False):
-                    fp8_ms, _ = time_region(fwd_only, a.steps, a.warmup)
-                fp8_cached_ms, _ = time_region(fwd_only, a.steps, a.warmup)
+                    fp8_ms, _ = time_region(t["fwd_only"], a.steps, a.warmup)
+                fp8_cached_ms, _ = time_region(t["fwd_only"], a.steps, a.warmup)
         rel = float((fp8_out.float() - ref_out.float()).norm() / ref_out.float().norm())
         fp8_info = dict(
             what="forward with block-scaled e4m3 operands (x, W1, y1, W2 quantised inside the timed region), bf16 outputs; "
             "fwd_ms_weights_quantised_once: W1, W2 quantised before the timed region (inference)",
             fwd_ms=round(fp8_ms, 4),
             fwd_ms_weights_quantised_once=round(fp8_cached_ms, 4),
-            fwd_tflops=round(flops_fwd / fp8_ms / 1e9, 2),
-            frac_of_fp8_peak=round(flops_fwd / fp8_ms / 1e9 / PEAK_FP8_TFLOPS, 4),
+            fwd_tflops=round(t["flops_fwd"] / fp8_ms / 1e9, 2),
+            frac_of_fp8_peak=round(t["flops_fwd"] / fp8_ms / 1e9 / PEAK_FP8_TFLOPS, 4),
             rel_l2_vs_bf16_forward=round(rel, 4),
         )
         log(f"fp8 forward: {fp8_ms:.3f} ms ({fp8_info['fwd_tflops']:.1f} TFLOP/s), rel-L2 vs bf16 forward {rel:.4f}")
         del ref_out, fp8_out
 
-    rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, x, wr, w1, w2, dout, max(5, a.steps // 2))
+    rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, t["x"], t["wr"], t["w1"], t["w2"], t["dout"],
+                                                                    max(5, a.steps // 2))
     # dominant kernel = the single grouped-GEMM launch with the largest average duration
     single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS]
     roofline = None
@@ -365,33 +452,55 @@ def main():
 
     out = dict(
         metric=f"MoE fwd+bwd TFLOP/s (% bf16 MFMA peak), T={T} H={H} I={I} E={E} K={K}",
-        value=round(tflops, 2),
+        value=rec["tflops"],
         unit="TFLOP/s",
         n_gpus=1,
         steps=a.steps,
         warmup=a.warmup,
-        ms_per_step=round(ms, 4),
+        ms_per_step=rec["ms_per_step"],
+        ms_per_step_median=rec["ms_per_step_median"],
+        ms_per_step_min=rec["ms_per_step_min"],
         higher_is_better=True,
         scaling="weak",
         vs_baseline=None,
         dtype="bf16",
         data="synthetic",
-        config=dict(
-            workload=f"{a.config}: MoE layer fwd+bwd, T={T} H={H} I={I} E={E} K={K}, SwiGLU, no bias, token-choice softmax "
-            f"top-k router{' with Zipf logit bias' if cfg['zipf'] else ''}"
-            f"{' then token rounding (' + rounding + ', tile 128), ' + str(TK) + ' routed pairs, general-routing entry' if rounding else ''}"
-            f"; x,dout~N(0,1), weights~N(0,0.02), seed 0",
-            flops_per_step=flops_all,
-        ),
-        frac_of_peak=round(tflops / PEAK_BF16_TFLOPS, 4),
-        fwd_ms=round(fwd_ms, 4),
-        fwd_tflops=round(flops_fwd / fwd_ms / 1e9, 2),
+        config=dict(workload=rec["workload"], flops_per_step=rec["flops_per_step"]),
+        frac_of_peak=rec["frac_of_peak"],
+        fwd_ms=rec["fwd_ms"],
+        fwd_tflops=rec["fwd_tflops"],
+        activation_bytes_held_for_backward=rec["activation_bytes_held_for_backward"],
+        peak_activation_bytes=rec["peak_bytes_forward"],
+        peak_bytes_step=rec["peak_bytes_step"],
         roofline=roofline,
         fp8_forward=fp8_info,
         kernels=[{k: v for k, v in r.items() if k != "flops"} for r in rows],
     )
+    del t
+    torch.cuda.empty_cache()
+
+    if not a.no_other_configs and a.config == "C2":
+        # the other benchmark configurations (whole layer) and the reference's short-contraction shapes (per kernel):
+        # extra keys, not the headline
+        others = {}
+        for name in ("C3", "C4"):
+            r, tt = measure_layer(CONFIGS[name], name, dev, max(5, a.steps // 2), 2)
+            others[name] = r
+            del tt
+            torch.cuda.empty_cache()
+        out["other_configs"] = others
+        shapes = {}
+        for name in ("I512", "I256"):
+            c = CONFIGS[name]
+            xs, wrs, w1s, w2s, ds = make_inputs(c, dev)
+            log(f"{name}: T={c['T']} H={c['H']} I={c['I']} E={c['E']} K={c['K']}")
+            shapes[name] = [{k: v for k, v in r.items() if k != "flops"}
+                            for r in kernel_breakdown(c, xs, wrs, w1s, w2s, ds, 5, gemms_only=True)]
+            del xs, wrs, w1s, w2s, ds
+            torch.cuda.empty_cache()
+        out["short_contraction_shapes"] = shapes
+
     if not a.no_cpu_baseline:
-        del x, wr, w1, w2, dout
         torch.cuda.empty_cache()
         out["cpu_baseline"] = cpu_baseline(cfg)
         log("cpu baseline:", out["cpu_baseline"])

@@ -732,10 +732,9 @@ SMOE_DEV void forward_epilogue_rows(typename Mma::Acc (&acc)[TN / Mma::FR][TM / 
 // Read from the environment ONCE, at the first launch that asks (variable = "SMOE_" + the upper-cased field name);
 // smoe_set_tuning() overrides a knob afterwards (tests walk through the alternative kernels with it).
 struct Tuning {
-  int gemm_stream;          // 1 (default): up-projection forward, down-projection forward, dz and dx run as tile streams
+  int gemm_stream;          // 1 (default): up-projection forward, down-projection forward and dx run as tile streams
   int gemm_stream_grid;     // workgroups of the tile-stream kernels; 0 (default) = one per compute unit
   int varlen_k_tile_order;  // 2 blocked (default), 0 single tiles round-robin over the XCDs, 1 whole experts per XCD
-  int experiment;           // scratch knob for kernel experiments (no effect in a release build)
 };
 const Tuning& tuning();
 

@@ -717,11 +717,6 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.scores = scores;
   p.sidx = sidx;
   p.ds_partial = ds_partial;
-  if (tuning().experiment & 2) {  // EXPERIMENT: the dz GEMM alone as a tile stream (dy1 written to y1s)
-    p.out0 = (uint16_t*)y1s;
-    p.out0_stride = I;
-    return launch_varlen_m<TileCfg<true>, ROLE_PLAIN, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
-  }
   return launch_by_activation<true, ROLE_DZ>(activation, p, off, workspace, TK, E, st);
 }
 

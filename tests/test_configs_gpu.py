@@ -203,3 +203,132 @@ def test_tensors_beyond_2_31_elements(dev):
             ref += scores[sample, j, None] * torch.einsum("ti,thi->th", y, w2.detach()[ee].float())
     assert rel_l2(o.detach()[sample], ref) < TOL
     assert bool(torch.isfinite(dx.float()).all())
+
+
+def _dense_tokens(x, w1, w2, pairs_tok, pairs_exp, pairs_score, sample):
+    """fp32 forward of the sampled tokens only: sum over a token's routed pairs of score * W2[e] swiglu(W1[e] x)."""
+    ref = torch.zeros(sample.numel(), x.size(1), device=x.device)
+    for n, t in enumerate(sample.tolist()):
+        sel = (pairs_tok == t).nonzero().flatten()
+        for j in sel.tolist():
+            e = int(pairs_exp[j])
+            h = w1.detach()[e].float() @ x.detach()[t].float()
+            y = torch.nn.functional.silu(h[0::2]) * h[1::2]
+            ref[n] += float(pairs_score[j]) * (w2.detach()[e].float() @ y)
+    return ref
+
+
+def _dense_expert_weight_grads(x, dout, w1, w2, e, tok, s):
+    """fp32 weight gradients of ONE expert from its routed tokens `tok` with scores `s` (the formulas of the layer)."""
+    xe, de = x.detach()[tok].float(), dout[tok].float()
+    z = xe @ w1.detach()[e].float().t()
+    gate, up = z[:, 0::2], z[:, 1::2]
+    sig = torch.sigmoid(gate)
+    y1 = gate * sig * up
+    dy1 = de @ w2.detach()[e].float()
+    dz = torch.empty_like(z)
+    dz[:, 0::2] = s[:, None] * dy1 * up * (gate * sig * (1 - sig) + sig)
+    dz[:, 1::2] = s[:, None] * dy1 * gate * sig
+    return dz.t() @ xe, de.t() @ (s[:, None] * y1)
+
+
+def test_config3_full_size_properties(dev):
+    """Config 3 at full size (T=32768,H=4096,I=1536,E=128,K=8, Zipf logit bias 2*log(1/(e+1))): the head experts hold
+    tens of thousands of rows, the tail ones none; I=1536 gives the weight-gradient kernels 6 column tiles.  Checked
+    without a second full implementation: routing metadata = stable sort of the router's choice, two runs bit-identical,
+    zero weight gradients for experts without tokens, sampled tokens against a dense fp32 forward, and the weight
+    gradients of one mid-sized and the largest expert against a dense fp32 evaluation of just those experts."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import TC_Softmax_Topk_Router_Function, _build_metadata, _ExpertsFunction
+
+    T, H, I, E, K = 32768, 4096, 1536, 128, 8
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16).requires_grad_()
+    wr = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    w1 = (0.02 * torch.randn(E, 2 * I, H, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    w2 = (0.02 * torch.randn(E, H, I, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    dout = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    st = torch.cuda.current_stream().cuda_stream
+    bias = _zipf_bias(E, dev).to(torch.bfloat16)
+
+    def run():
+        logits = torch.nn.functional.linear(x.detach(), wr) + bias
+        s, i = TC_Softmax_Topk_Router_Function.apply(logits, E, K)
+        freq, off, gidx, sidx, ridx, tok_off = _build_metadata(i.view(-1), None, T, E, K)
+        o = _ExpertsFunction.apply(x, w1.permute(1, 2, 0), None, w2.permute(1, 2, 0), None, s.view(-1), off, gidx, sidx,
+                                   ridx, tok_off, K, False, ActivationType.SWIGLU, st, False)
+        return o, torch.autograd.grad(o, [x, w1, w2], grad_outputs=dout), (s, i, freq, off, gidx, sidx, ridx)
+
+    o1, g1, (s, i, freq, off, gidx, sidx, ridx) = run()
+    o2, g2, _ = run()
+    assert torch.equal(o1, o2) and all(torch.equal(a, b) for a, b in zip(g1, g2)), "not deterministic"
+    flat = i.view(-1).long()
+    assert int(freq.sum()) == T * K and int(off[-1]) == T * K
+    assert torch.equal(sidx.long(), torch.sort(flat, stable=True).indices)
+    assert torch.equal(ridx[sidx.long()].long(), torch.arange(T * K, device=dev))
+    assert torch.equal(gidx, sidx // K)
+    empty = (freq == 0).nonzero().flatten()
+    assert empty.numel() > 0 and int(freq.max()) > 20000, "the Zipf bias should empty the tail and overload the head"
+    dx, dw1, dw2 = g1
+    assert bool((dw1[empty] == 0).all()) and bool((dw2[empty] == 0).all())
+    assert bool(torch.isfinite(dx.float()).all())
+
+    with torch.no_grad():
+        sample = torch.randperm(T, generator=torch.Generator().manual_seed(1))[:32].to(dev)
+        tok_of_pair = torch.arange(T, device=dev).repeat_interleave(K)
+        ref = _dense_tokens(x, w1, w2, tok_of_pair, i.view(-1), s.view(-1), sample)
+        assert rel_l2(o1.detach()[sample], ref) < TOL
+        # one mid-sized expert (its last token tile is ragged) and the largest one
+        counts = freq.tolist()
+        mid = min((e for e in range(E) if 300 <= counts[e] <= 6000), key=lambda e: counts[e], default=None)
+        for e in [e for e in (mid, int(freq.argmax())) if e is not None]:
+            a, b = int(off[e]), int(off[e + 1])
+            tok = gidx[a:b].long()
+            sc = s.view(-1)[sidx[a:b].long()]
+            dw1_ref, dw2_ref = _dense_expert_weight_grads(x, dout, w1, w2, e, tok, sc)
+            assert rel_l2(dw1[e], dw1_ref) < TOL, e
+            assert rel_l2(dw2[e], dw2_ref) < TOL, e
+
+
+def test_config4_full_size_properties(dev):
+    """Config 4 at full size (T=16384,H=4096,I=1024,E=256,K=8, token rounding "nr" to tiles of 128, general-routing
+    entry): every expert's count is a multiple of 128, the pairs are sorted by token, two runs are bit-identical,
+    sampled tokens match a dense fp32 forward over their pairs and one expert's weight gradients a dense evaluation."""
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import _build_metadata, moe_general_routing_inputs
+    from sonicmoe.routing import token_choice_rounding
+
+    T, H, I, E, K, tile = 16384, 4096, 1024, 256, 8, 128
+    g = torch.Generator(device=dev).manual_seed(0)
+    x = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16).requires_grad_()
+    wr = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(torch.bfloat16)
+    w1 = (0.02 * torch.randn(E, 2 * I, H, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    w2 = (0.02 * torch.randn(E, H, I, generator=g, device=dev)).to(torch.bfloat16).requires_grad_()
+    dout = torch.randn(T, H, generator=g, device=dev).to(torch.bfloat16)
+    st = torch.cuda.current_stream().cuda_stream
+    with torch.no_grad():
+        scores, tok, exp = token_choice_rounding(torch.nn.functional.linear(x, wr), K, tile, "nr")
+    scores = scores.float().requires_grad_()
+    assert bool((tok[1:] >= tok[:-1]).all())
+
+    def run():
+        o, freq = moe_general_routing_inputs(x, scores, tok, exp, w1.permute(1, 2, 0), None, w2.permute(1, 2, 0), None, E,
+                                             st, ActivationType.SWIGLU, False)
+        return o, freq, torch.autograd.grad(o, [x, scores, w1, w2], grad_outputs=dout)
+
+    o1, freq, g1 = run()
+    o2, _, g2 = run()
+    assert torch.equal(o1, o2) and all(torch.equal(a, b) for a, b in zip(g1, g2)), "not deterministic"
+    assert bool((freq % tile == 0).all()) and int(freq.sum()) == tok.numel()
+    assert abs(tok.numel() - T * K) <= E * tile // 2
+    with torch.no_grad():
+        sample = torch.randperm(T, generator=torch.Generator().manual_seed(2))[:32].to(dev)
+        ref = _dense_tokens(x, w1, w2, tok, exp, scores.detach(), sample)
+        assert rel_l2(o1.detach()[sample], ref) < TOL
+        _, off, gidx, sidx, _, _ = _build_metadata(exp, tok, T, E, 1)
+        e = int((freq > 0).nonzero().flatten()[7])
+        a, b = int(off[e]), int(off[e + 1])
+        dw1_ref, dw2_ref = _dense_expert_weight_grads(x, dout, w1, w2, e, gidx[a:b].long(),
+                                                      scores.detach()[sidx[a:b].long()])
+        assert rel_l2(g1[2][e], dw1_ref) < TOL
+        assert rel_l2(g1[3][e], dw2_ref) < TOL
