@@ -121,7 +121,14 @@ int smoe_routing_metadata_static(const int32_t* expert_idx, const int32_t* token
  * Grouped GEMMs (bf16 in, fp32 MFMA accumulate, bf16 out)
  * ------------------------------------------------------------------------------------------------------ */
 
-/* Workspace needed by every grouped GEMM below (tile map built from `off` on the device). */
+/* Workspace needed by every grouped GEMM below (tile map built from `off` on the device).
+ *
+ * expert_schedule_order (the reference operators' argument of that name, sonicmoe/functional/forward.py:61, :79-82;
+ * its tile scheduler's batch_idx_permute, grouped_gemm.py:819-822, :948): NULL, or E int32 on the device holding a
+ * permutation of 0 .. E-1.  The kernels then take up the experts' tiles in that order (position i of the schedule
+ * works on expert order[i]) -- e.g. largest expert first, so that the long contractions of the weight-gradient
+ * kernels do not start last.  Results do not depend on it bit for bit.  An array that is not a permutation leaves
+ * the outputs of the missing experts unwritten; the library does not check it (that would need a host round trip). */
 size_t smoe_gemm_workspace_bytes(int64_t TK, int E);
 
 /* z[m] = x[x_gather_idx[m]] W1[e]^T (+ b1[e]);  y1[m] = f(z_even) * z_odd for the gated activations (gate = even
@@ -132,16 +139,18 @@ size_t smoe_gemm_workspace_bytes(int64_t TK, int E);
  *   (inference: not stored); y1 (TK, I)
  * Limits: H % 64 == 0, I % 64 == 0. */
 int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
-                               const void* b1, void* z, void* y1, const int32_t* off, const int32_t* x_gather_idx,
-                               int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
+                               const void* b1, void* z, void* y1, const int32_t* off,
+                               const int32_t* expert_schedule_order, const int32_t* x_gather_idx, int64_t T,
+                               int64_t TK, int H, int I, int E, int activation, void* workspace,
                                size_t workspace_bytes, void* stream);
 
 /* y2[m] = y1[m] W2[e]^T (+ b2[e]).  Replaces sonicmoe::_down_projection_forward
  * (sonicmoe/functional/forward.py:132-178).
  *   y1 (TK, I); w2 (E, H, I); b2 (E, H) contiguous or NULL; y2 (TK, H) */
 int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
-                                 const void* b2, void* y2, const int32_t* off, int64_t TK, int H, int I, int E,
-                                 void* workspace, size_t workspace_bytes, void* stream);
+                                 const void* b2, void* y2, const int32_t* off, const int32_t* expert_schedule_order,
+                                 int64_t TK, int H, int I, int E, void* workspace, size_t workspace_bytes,
+                                 void* stream);
 
 /* out[t] = sum_{j in [tok_off[t], tok_off[t+1])} w[j] * src[ridx[j]]  (w == NULL: unweighted), fp32 accumulate.
  * Replaces sonicmoe::_router_forward and sonicmoe::_token_broadcast_backward
@@ -166,9 +175,9 @@ int smoe_down_projection_backward(const void* dout, const void* z, const void* w
                                   int64_t w2_stride_row, const void* b2, void* dw2, int64_t dw2_stride_e,
                                   int64_t dw2_stride_row, void* db2, void* dz, void* y1s, float* ds,
                                   float* ds_partial, const float* scores, const int32_t* off,
-                                  const int32_t* x_gather_idx, const int32_t* s_scatter_idx, int64_t T, int64_t TK,
-                                  int H, int I, int E, int activation, void* workspace, size_t workspace_bytes,
-                                  void* stream);
+                                  const int32_t* expert_schedule_order, const int32_t* x_gather_idx,
+                                  const int32_t* s_scatter_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                  int activation, void* workspace, size_t workspace_bytes, void* stream);
 
 /* dW1[e] = sum_m dz[m]^T (x) x[t_m];  db1[e] = sum_m dz[m];  dx_expanded[m] = dz[m] W1[e].
  * Replaces sonicmoe::_up_projection_backward (sonicmoe/functional/backward.py:195-283; db1 backward.py:109-168).
@@ -176,9 +185,9 @@ int smoe_down_projection_backward(const void* dout, const void* z, const void* w
  *   dw1 == NULL, db1 == NULL or dx_expanded == NULL skips that output (frozen weights / no input gradient). */
 int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
                                 const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row, void* db1,
-                                void* dx_expanded, const int32_t* off, const int32_t* x_gather_idx, int64_t T,
-                                int64_t TK, int H, int I, int E, int activation, void* workspace,
-                                size_t workspace_bytes, void* stream);
+                                void* dx_expanded, const int32_t* off, const int32_t* expert_schedule_order,
+                                const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                int activation, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Weight gradient of the router's linear layer, dWr = dlogits^T x, split over the tokens: partial[c] (E, H) bf16 is the
  * product over tokens [c * ceil(T / chunks), ...) and the caller sums the `chunks` partials.  The reference leaves this

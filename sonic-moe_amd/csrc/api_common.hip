@@ -67,15 +67,18 @@ int device_compute_units(int* out) {
   return SMOE_OK;
 }
 
-__global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __restrict__ off, int E, int BM,
+// order == nullptr: experts are listed 0, 1, ...; otherwise position i of the list holds expert order[i]
+__global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __restrict__ off,
+                                                              const int32_t* __restrict__ order, int E, int BM,
                                                               TileMap tm) {
   __shared__ int32_t wave_tot[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int32_t base = 0;
   for (int e0 = 0; e0 < E; e0 += 1024) {
-    const int e = e0 + tid;
+    int e = e0 + tid;
     int32_t lo = 0, cnt = 0;
     if (e < E) {
+      if (order != nullptr) e = order[e];
       lo = off[e];
       cnt = off[e + 1] - lo;
     }
@@ -103,8 +106,8 @@ __global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __r
   if (tid == 0) tm.header[0] = base;
 }
 
-int launch_build_tile_map(const int32_t* off, int E, int BM, TileMap tm, hipStream_t st) {
-  hipLaunchKernelGGL(build_tile_map_kernel, dim3(1), dim3(1024), 0, st, off, E, BM, tm);
+int launch_build_tile_map(const int32_t* off, const int32_t* order, int E, int BM, TileMap tm, hipStream_t st) {
+  hipLaunchKernelGGL(build_tile_map_kernel, dim3(1), dim3(1024), 0, st, off, order, E, BM, tm);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }

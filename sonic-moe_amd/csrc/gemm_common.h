@@ -783,7 +783,7 @@ static inline TileMap carve_tile_map(void* ws, int64_t TK, int E, int BM) {
 // single workgroup of 1024 threads
 __global__ void build_tile_map_kernel(const int32_t* __restrict__ off, int E, int BM, TileMap tm);
 
-int launch_build_tile_map(const int32_t* off, int E, int BM, TileMap tm, hipStream_t st);
+int launch_build_tile_map(const int32_t* off, const int32_t* order, int E, int BM, TileMap tm, hipStream_t st);
 
 // XCD-aware linear tile id: workgroups are dealt round-robin to the 8 XCDs, so workgroup b runs on XCD b % 8;
 // give every XCD one contiguous range of the tile space so that tiles sharing operands share an L2.

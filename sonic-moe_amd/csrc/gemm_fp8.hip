@@ -380,7 +380,7 @@ static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t
     if (rc_attr) return rc_attr;
   }
   p.tm = carve_tile_map(workspace, TK, E, C::BM);
-  int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
+  int rc = launch_build_tile_map(off, nullptr, E, C::BM, p.tm, st);
   if (rc) return rc;
   p.n_tiles = (int)ceil_div(p.N, C::BN);
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;

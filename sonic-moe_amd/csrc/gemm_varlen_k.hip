@@ -22,6 +22,7 @@ struct VarlenKParams {
   int NA, NB;  // output rows / cols
   int tiles_a, tiles_b;
   int E;
+  const int32_t* order;  // nullable: position i of the tile order works on expert order[i]
   int uniform_rows;  // off == nullptr: group e is rows [e * uniform_rows, min((e + 1) * uniform_rows, total_rows))
   int64_t total_rows;
   int xcd_chunked;  // tile order: 2 blocked, 1 contiguous tile range per XCD (probe: unbalanced on skewed experts), 0 round-robin
@@ -96,6 +97,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 
   int e, ta, tb;
   if (!decode_tile(p, (int64_t)blockIdx.x, e, ta, tb)) return;
+  if (p.order != nullptr) e = p.order[e];
   const int a0 = ta * C::BA, b0 = tb * C::BB;
   int row_begin, row_end;
   if (p.off != nullptr) {
@@ -331,10 +333,12 @@ static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st) {
 }
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
-              void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
-              const int32_t* sidx, int64_t TK, int H, int I, int E, int activation, void* workspace, hipStream_t st);
+              void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* order,
+              const int32_t* gidx, const int32_t* sidx, int64_t TK, int H, int I, int E, int activation,
+              void* workspace, hipStream_t st);
 int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
-              const int32_t* off, int64_t TK, int H, int N1, int E, void* workspace, hipStream_t st);
+              const int32_t* off, const int32_t* order, int64_t TK, int H, int N1, int E, void* workspace,
+              hipStream_t st);
 
 }  // namespace smoe
 
@@ -354,9 +358,9 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
                                              int64_t w2_stride_row, const void* b2, void* dw2, int64_t dw2_stride_e,
                                              int64_t dw2_stride_row, void* db2, void* dz, void* y1s, float* ds,
                                              float* ds_partial, const float* scores, const int32_t* off,
-                                             const int32_t* x_gather_idx, const int32_t* s_scatter_idx, int64_t T,
-                                             int64_t TK, int H, int I, int E, int activation, void* workspace,
-                                             size_t workspace_bytes, void* stream) {
+                                             const int32_t* expert_schedule_order, const int32_t* x_gather_idx,
+                                             const int32_t* s_scatter_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                             int activation, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_bwd(TK, H, I, E, workspace, workspace_bytes, "down_projection_backward");
   if (rc) return rc;
   SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
@@ -376,8 +380,8 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
                SMOE_ERR_UNSUPPORTED, "down_projection_backward: weight strides must be multiples of 8 elements");
   hipStream_t st = (hipStream_t)stream;
   if (TK > 0 && dz) {
-    rc = launch_dz(dout, z, w2, w2_stride_e, w2_stride_row, dz, y1s, ds_partial, scores, off, x_gather_idx,
-                   s_scatter_idx, TK, H, I, E, activation, workspace, st);
+    rc = launch_dz(dout, z, w2, w2_stride_e, w2_stride_row, dz, y1s, ds_partial, scores, off, expert_schedule_order,
+                   x_gather_idx, s_scatter_idx, TK, H, I, E, activation, workspace, st);
     if (rc) return rc;
     rc = launch_ds_finalize(ds_partial, smoe_dz_partial_cols(I), s_scatter_idx, ds, TK, st);
     if (rc) return rc;
@@ -406,6 +410,7 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
   p.NA = H;
   p.NB = I;
   p.E = E;
+  p.order = expert_schedule_order;
   p.total_rows = TK;
   return launch_varlen_k_variant<true, false>(p, st);
 }
@@ -413,8 +418,9 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
 extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
                                            const void* dz, void* dw1, int64_t dw1_stride_e, int64_t dw1_stride_row,
                                            void* db1, void* dx_expanded, const int32_t* off,
-                                           const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
-                                           int activation, void* workspace, size_t workspace_bytes, void* stream) {
+                                           const int32_t* expert_schedule_order, const int32_t* x_gather_idx,
+                                           int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                           size_t workspace_bytes, void* stream) {
   int rc = check_bwd(TK, H, I, E, workspace, workspace_bytes, "up_projection_backward");
   if (rc) return rc;
   SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
@@ -448,12 +454,14 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     p.NA = N1;
     p.NB = H;
     p.E = E;
+    p.order = expert_schedule_order;
     p.total_rows = TK;
     rc = launch_varlen_k_variant<false, true>(p, st);
     if (rc) return rc;
   }
   if (TK > 0 && dx_expanded) {
-    rc = launch_dx(dz, w1, w1_stride_e, w1_stride_row, dx_expanded, off, TK, H, N1, E, workspace, st);
+    rc = launch_dx(dz, w1, w1_stride_e, w1_stride_row, dx_expanded, off, expert_schedule_order, TK, H, N1, E, workspace,
+                   st);
     if (rc) return rc;
   }
   return SMOE_OK;

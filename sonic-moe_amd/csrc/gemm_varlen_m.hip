@@ -19,6 +19,7 @@ struct VarlenMParams {
   const uint16_t* Q;
   int64_t q_stride_e, q_stride_row;
   const int32_t* off;
+  const int32_t* order;  // nullable: the tile map lists the experts in this order (a permutation of 0 .. E-1)
   TileMap tm;
   int N, Kdim, n_tiles;
   uint16_t* out0;
@@ -550,7 +551,7 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
     if (rc_attr) return rc_attr;
   }
   p.tm = carve_tile_map(workspace, TK, E, C::BM);
-  int rc = launch_build_tile_map(off, E, C::BM, p.tm, st);
+  int rc = launch_build_tile_map(off, p.order, E, C::BM, p.tm, st);
   if (rc) return rc;
   p.n_tiles = (int)ceil_div(p.N, C::BN);
   if (ROLE == ROLE_DZ) p.ds_cols = p.n_tiles * C::WN;
@@ -632,8 +633,9 @@ extern "C" int smoe_dz_partial_cols(int I) { return (int)ceil_div(I, dz_tile_col
 
 extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
                                           const void* b1, void* z, void* y1, const int32_t* off,
-                                          const int32_t* x_gather_idx, int64_t T, int64_t TK, int H, int I, int E,
-                                          int activation, void* workspace, size_t workspace_bytes, void* stream) {
+                                          const int32_t* expert_schedule_order, const int32_t* x_gather_idx, int64_t T,
+                                          int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
   int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "up_projection_forward");
   if (rc) return rc;
   SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
@@ -654,6 +656,7 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
   p.off = off;
+  p.order = expert_schedule_order;
   p.N = act_is_glu(activation) ? 2 * I : I;
   p.Kdim = H;
   p.bias = (const uint16_t*)b1;
@@ -665,8 +668,9 @@ extern "C" int smoe_up_projection_forward(const void* x, const void* w1, int64_t
 }
 
 extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
-                                            const void* b2, void* y2, const int32_t* off, int64_t TK, int H, int I,
-                                            int E, void* workspace, size_t workspace_bytes, void* stream) {
+                                            const void* b2, void* y2, const int32_t* off,
+                                            const int32_t* expert_schedule_order, int64_t TK, int H, int I, int E,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "down_projection_forward");
   if (rc) return rc;
   if (TK == 0) return SMOE_OK;
@@ -682,6 +686,7 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
   p.q_stride_e = w2_stride_e;
   p.q_stride_row = w2_stride_row;
   p.off = off;
+  p.order = expert_schedule_order;
   p.N = H;
   p.Kdim = I;
   p.bias = (const uint16_t*)b2;
@@ -694,8 +699,9 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
 namespace smoe {
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
-              void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* gidx,
-              const int32_t* sidx, int64_t TK, int H, int I, int E, int activation, void* workspace, hipStream_t st) {
+              void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* order,
+              const int32_t* gidx, const int32_t* sidx, int64_t TK, int H, int I, int E, int activation,
+              void* workspace, hipStream_t st) {
   const int zw = act_is_glu(activation) ? 2 : 1;
   VarlenMParams p = {};
   p.P = (const uint16_t*)dout;
@@ -706,6 +712,7 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
   p.q_stride_e = w2_stride_e;
   p.q_stride_row = w2_stride_row;
   p.off = off;
+  p.order = order;
   p.N = I;
   p.Kdim = H;
   p.out0 = (uint16_t*)dz;
@@ -721,7 +728,8 @@ int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride
 }
 
 int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
-              const int32_t* off, int64_t TK, int H, int N1, int E, void* workspace, hipStream_t st) {
+              const int32_t* off, const int32_t* order, int64_t TK, int H, int N1, int E, void* workspace,
+              hipStream_t st) {
   VarlenMParams p = {};
   p.P = (const uint16_t*)dz;
   p.p_stride = N1;
@@ -729,6 +737,7 @@ int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_st
   p.q_stride_e = w1_stride_e;
   p.q_stride_row = w1_stride_row;
   p.off = off;
+  p.order = order;
   p.N = H;
   p.Kdim = N1;
   p.out0 = (uint16_t*)dx_expanded;

@@ -31,17 +31,21 @@ _SIGNATURES = {
     "smoe_routing_metadata_static_capacity": (c_size_t, []),
     "smoe_routing_metadata_static": (c_int, [_P, _P, _L, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     "smoe_gemm_workspace_bytes": (c_size_t, [_L, _I]),
-    "smoe_up_projection_forward": (c_int, [_P, _P, _L, _L, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P]),
-    "smoe_down_projection_forward": (c_int, [_P, _P, _L, _L, _P, _P, _P, _L, _I, _I, _I, _P, _Z, _P]),
+    "smoe_up_projection_forward": (
+        c_int,
+        [_P, _P, _L, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
+    ),
+    "smoe_down_projection_forward": (c_int, [_P, _P, _L, _L, _P, _P, _P, _P, _L, _I, _I, _I, _P, _Z, _P]),
     "smoe_gather_sum": (c_int, [_P, _P, _P, _P, _P, _L, _I, _I, _P]),
     "smoe_dz_partial_cols": (c_int, [_I]),
     "smoe_down_projection_backward": (
         c_int,
-        [_P, _P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
+        [_P, _P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z,
+         _P],
     ),
     "smoe_up_projection_backward": (
         c_int,
-        [_P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
+        [_P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
     "smoe_router_weight_grad": (c_int, [_P, _P, _P, _L, _I, _I, _I, _P]),
     "smoe_switch_loss_workspace_bytes": (c_size_t, [_L, _I]),

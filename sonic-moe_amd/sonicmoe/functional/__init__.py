@@ -11,6 +11,7 @@ inside the weight-gradient kernels.
 from __future__ import annotations
 
 import os
+from contextlib import contextmanager
 
 import torch
 import torch.nn.functional as F
@@ -176,8 +177,38 @@ class TC_Softmax_Topk_Router_Function(torch.autograd.Function):
         return dlogits, None, None
 
 
+_SCHEDULE_POLICY = "expert_index"
+
+
+@contextmanager
+def expert_schedule(policy: str = "largest_first"):
+    """Order in which the grouped GEMMs of the layers called inside take up the experts' tiles: "expert_index" (default;
+    what the reference runs, whose layers pass expert_schedule_order=None, sonicmoe/functional/__init__.py:161, :248)
+    or "largest_first" (longest processing time first: the experts sorted by token count, descending).  Results do not
+    depend on it."""
+    global _SCHEDULE_POLICY
+    if policy not in ("expert_index", "largest_first"):
+        raise ValueError(f"unknown expert schedule policy {policy!r}")
+    previous, _SCHEDULE_POLICY = _SCHEDULE_POLICY, policy
+    try:
+        yield
+    finally:
+        _SCHEDULE_POLICY = previous
+
+
+def largest_first_schedule_order(expert_frequency_offset: torch.Tensor) -> torch.Tensor:
+    """An expert_schedule_order for the grouped-GEMM operators: the experts by descending token count (ties by expert
+    index), int32 (E,)."""
+    counts = expert_frequency_offset[1:] - expert_frequency_offset[:-1]
+    return torch.argsort(counts, descending=True, stable=True).to(torch.int32)
+
+
+def _schedule_order(off):
+    return largest_first_schedule_order(off) if _SCHEDULE_POLICY == "largest_first" else None
+
+
 def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
-                     stream_id, inference):
+                     stream_id, inference, order=None):
     """o = combine(down(act(up(gather(x))))); returns (o, z) with z = None in inference mode."""
     T, H = x.shape
     N1, _, E = w1.shape
@@ -202,8 +233,8 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
         _down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, b2, off, E, stream_id)
         del y1q, y1s, w2q, w2s
     else:
-        _up_projection_forward(x, w1, z, y1, b1, off, None, gidx, stream_id, activation_type.value, glu, inference)
-        _down_projection_forward(w2, y1, y2, b2, off, None, gidx, stream_id)
+        _up_projection_forward(x, w1, z, y1, b1, off, order, gidx, stream_id, activation_type.value, glu, inference)
+        _down_projection_forward(w2, y1, y2, b2, off, order, gidx, stream_id)
     del y1
     o = torch.empty(T, H, dtype=x.dtype, device=x.device)
     _router_forward(y2, o, scores_flat, ridx, tok_off, K_or_maxK, H, is_varlen_K)
@@ -211,7 +242,7 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
 
 
 def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
-                      activation_type, stream_id, has_b1):
+                      activation_type, stream_id, has_b1, order=None):
     """Returns (dx, dw1, db1, dw2, db2, ds) of _experts_forward; `has_b1` says whether the forward pass had an
     up-projection bias (b1 itself is not needed for any gradient and is not kept)."""
     T, H = x.shape
@@ -224,12 +255,12 @@ def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx
     dz = torch.empty_like(z)
     ds = torch.empty(TK, dtype=torch.float32, device=x.device)
     _down_projection_backward(
-        dout, z, w2, dw2, dz, ds, b2, db2, scores_flat, off, None, gidx, sidx, stream_id, glu, activation_type.value
+        dout, z, w2, dw2, dz, ds, b2, db2, scores_flat, off, order, gidx, sidx, stream_id, glu, activation_type.value
     )
     dw1 = torch.empty_like(w1)
     db1 = torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device) if has_b1 else None
     dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
-    _up_projection_backward(x, w1, dx_expanded, dw1, dz, db1, off, None, gidx, sidx, glu, stream_id)
+    _up_projection_backward(x, w1, dx_expanded, dw1, dz, db1, off, order, gidx, sidx, glu, stream_id)
     del dz
     dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
     _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
@@ -265,8 +296,10 @@ class _ExpertsFunction(torch.autograd.Function):
     ):
         x = x.contiguous()
         scores_flat = scores_flat.contiguous()
+        order = _schedule_order(off)
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K,
-                                activation_type, stream_id, inference)
+                                activation_type, stream_id, inference, order)
+        ctx.order = order
         if not inference:
             ctx.save_for_backward(x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference, b1 is not None)
@@ -280,7 +313,7 @@ class _ExpertsFunction(torch.autograd.Function):
         x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
         dx, dw1, db1, dw2, db2, ds = _experts_backward(
             dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
-            stream_id, has_b1,
+            stream_id, has_b1, ctx.order,
         )
         return dx, dw1, db1, dw2, db2, ds, None, None, None, None, None, None, None, None, None, None
 
@@ -471,6 +504,8 @@ __all__ = [
     "is_using_quack_gemm",
     "enable_fp8_forward",
     "is_using_fp8_forward",
+    "expert_schedule",
+    "largest_first_schedule_order",
     "moe_TC_softmax_topk_layer",
     "moe_general_routing_inputs",
     "switch_loss",

@@ -9,7 +9,7 @@ import torch
 from .. import _lib
 from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
 from ..utils import expert_major_strides
-from .forward import _check_bf16, _gather_sum, _gemm_workspace
+from .forward import _check_bf16, _check_schedule_order, _gather_sum, _gemm_workspace
 
 
 @torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_backward", mutates_args={"dw1", "dx_expanded", "db1"})
@@ -29,9 +29,8 @@ def _up_projection_backward(
 ) -> None:
     """dw1[e] = sum_m dz[m]^T x[t_m], db1[e] = sum_m dz[m] (zeros for empty experts), dx_expanded = dz W1[e]; any
     output may be None to skip it."""
-    if expert_schedule_order is not None:
-        raise NotImplementedError("_up_projection_backward: expert_schedule_order is not supported")
-    _lib.require_device(x, w1, dx_expanded, dw1, db1, dz, expert_frequency_offset, x_gather_idx)
+    _lib.require_device(x, w1, dx_expanded, dw1, db1, dz, expert_frequency_offset, expert_schedule_order, x_gather_idx)
+    _check_schedule_order(expert_schedule_order, w1.size(2))
     _check_bf16(("x", x), ("w1", w1), ("dx_expanded", dx_expanded), ("dw1", dw1), ("db1", db1), ("dz", dz))
     N1, H, E = w1.shape
     I = N1 // 2 if is_glu_activation else N1
@@ -53,6 +52,7 @@ def _up_projection_backward(
         _lib.ptr(db1),
         _lib.ptr(dx_expanded),
         _lib.ptr(expert_frequency_offset),
+        _lib.ptr(expert_schedule_order),
         _lib.ptr(x_gather_idx),
         T,
         TK,
@@ -89,10 +89,9 @@ def _down_projection_backward(
 ) -> None:
     """dz, ds (flat routing-slot order), dw2 and db2 of the down projection + weighted combine; y1 is recomputed from z
     and the dout rows are re-gathered, nothing of size (TK, H) is kept from the forward."""
-    if expert_schedule_order is not None:
-        raise NotImplementedError("_down_projection_backward: expert_schedule_order is not supported")
-    _lib.require_device(dout, z, w2, dw2, dz, ds, b2, db2, topk_scores, expert_frequency_offset, x_gather_idx,
-                        s_scatter_idx)
+    _lib.require_device(dout, z, w2, dw2, dz, ds, b2, db2, topk_scores, expert_frequency_offset, expert_schedule_order,
+                        x_gather_idx, s_scatter_idx)
+    _check_schedule_order(expert_schedule_order, w2.size(2))
     _check_bf16(("dout", dout), ("z", z), ("w2", w2), ("dw2", dw2), ("dz", dz), ("b2", b2), ("db2", db2))
     H, I, E = w2.shape
     assert (b2 is None) == (db2 is None), "b2 and db2 have to be given together"
@@ -125,6 +124,7 @@ def _down_projection_backward(
         _lib.ptr(ds_partial),
         _lib.ptr(topk_scores),
         _lib.ptr(expert_frequency_offset),
+        _lib.ptr(expert_schedule_order),
         _lib.ptr(x_gather_idx),
         _lib.ptr(s_scatter_idx),
         T,

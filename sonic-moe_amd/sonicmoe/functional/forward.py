@@ -34,6 +34,14 @@ def _check_bf16(*named):
             raise NotImplementedError(f"{name}: the HIP grouped GEMMs take bfloat16 tensors, got {t.dtype}")
 
 
+def _check_schedule_order(order: torch.Tensor | None, E: int) -> None:
+    """expert_schedule_order: None or E int32 holding a permutation of the experts (position i of the tile schedule works
+    on expert order[i]); the values are not inspected -- that would cost a host round trip."""
+    if order is not None and (order.dtype != torch.int32 or order.shape != (E,) or not order.is_contiguous()):
+        raise ValueError(f"expert_schedule_order must be a contiguous int32 tensor of {E} experts, got "
+                         f"{order.dtype} {tuple(order.shape)}")
+
+
 @torch.library.custom_op(f"{LIBRARY_NAME}::_topk_fwd", mutates_args={"values", "indices"})
 def _topk_fwd(
     x: torch.Tensor, k: int, values: torch.Tensor, indices: torch.Tensor, require_softmax_fusion: bool = True
@@ -86,9 +94,8 @@ def _up_projection_forward(
 ) -> None:
     """z = gather(x) W1^T (+ b1), y1 = act(z); w1 is the (N1, H, E) view of the (E, N1, H) parameter, N1 = 2I for the
     gated activations and I otherwise; b1 is (E, N1)."""
-    if expert_schedule_order is not None:
-        raise NotImplementedError("_up_projection_forward: expert_schedule_order is not supported")
-    _lib.require_device(x, w1, y1, b1, expert_frequency_offset, x_gather_idx)
+    _lib.require_device(x, w1, y1, b1, expert_frequency_offset, expert_schedule_order, x_gather_idx)
+    _check_schedule_order(expert_schedule_order, w1.size(2))
     _check_bf16(("x", x), ("w1", w1), ("z", z), ("y1", y1), ("b1", b1))
     N1, H, E = w1.shape
     I = N1 // 2 if is_glu_activation else N1
@@ -106,6 +113,7 @@ def _up_projection_forward(
         None if is_inference_mode_enabled else _lib.ptr(z),
         _lib.ptr(y1),
         _lib.ptr(expert_frequency_offset),
+        _lib.ptr(expert_schedule_order),
         _lib.ptr(x_gather_idx),
         T,
         TK,
@@ -132,9 +140,8 @@ def _down_projection_forward(
     stream_id: int,
 ) -> None:
     """y2 = y1 W2^T (+ b2) per expert; w2 is the (H, I, E) view of the (E, H, I) parameter, b2 is (E, H)."""
-    if expert_schedule_order is not None:
-        raise NotImplementedError("_down_projection_forward: expert_schedule_order is not supported")
-    _lib.require_device(w2, y1, y2, b2, expert_frequency_offset)
+    _lib.require_device(w2, y1, y2, b2, expert_frequency_offset, expert_schedule_order)
+    _check_schedule_order(expert_schedule_order, w2.size(2))
     _check_bf16(("w2", w2), ("y1", y1), ("y2", y2), ("b2", b2))
     H, I, E = w2.shape
     TK = y1.size(0)
@@ -150,6 +157,7 @@ def _down_projection_forward(
         _lib.ptr(b2),
         _lib.ptr(y2),
         _lib.ptr(expert_frequency_offset),
+        _lib.ptr(expert_schedule_order),
         TK,
         H,
         I,

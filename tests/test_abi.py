@@ -53,16 +53,18 @@ def test_argument_checks_return_status_codes(lib):
     # K > E
     assert lib.smoe_topk_softmax_fwd(p, 0, 4, 8, 9, 8, p, p, 1, None) == 2
     # H not a multiple of 64
-    assert lib.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, p, 4, 8, 96, 64, 2, 0, p, 1 << 20, None) == 2
+    assert lib.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, None, p, 4, 8, 96, 64, 2, 0, p, 1 << 20,
+                                          None) == 2
     assert b"multiple of 64" in lib.smoe_last_error()
     # workspace too small
-    assert lib.smoe_down_projection_forward(p, p, 0, 0, None, p, p, 1 << 20, 64, 64, 2, p, 8, None) == 4
+    assert lib.smoe_down_projection_forward(p, p, 0, 0, None, p, p, None, 1 << 20, 64, 64, 2, p, 8, None) == 4
     # activation code outside the enum -> SMOE_ERR_INVALID
-    assert lib.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, p, 4, 8, 64, 64, 2, 7, p, 1 << 20, None) == 1
+    assert lib.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, None, p, 4, 8, 64, 64, 2, 7, p, 1 << 20,
+                                          None) == 1
     assert b"activation" in lib.smoe_last_error()
     # a backward call with every output null has nothing to do
-    assert lib.smoe_up_projection_backward(p, p, 0, 0, p, None, 0, 0, None, None, p, p, 4, 8, 64, 64, 2, 0, p, 1 << 20,
-                                           None) == 1
+    assert lib.smoe_up_projection_backward(p, p, 0, 0, p, None, 0, 0, None, None, p, None, p, 4, 8, 64, 64, 2, 0, p,
+                                           1 << 20, None) == 1
     # switch loss: E outside [1, 4096] -> unsupported; workspace too small -> SMOE_ERR_WORKSPACE
     assert lib.smoe_switch_loss_fwd(p, 0, 8192, 16, 8192, p, p, p, p, 1 << 20, None) == 2
     assert b"E=8192" in lib.smoe_last_error()
@@ -81,9 +83,10 @@ def test_misaligned_operands_are_rejected(lib):
     base += (-base) % 16
     p, q = ctypes.c_void_p(base), ctypes.c_void_p(base + 2)
     # a weight pointer that is not 16-byte aligned, then a row stride that is not a multiple of 8 elements
-    assert lib.smoe_up_projection_forward(p, q, 64, 64, None, p, p, p, p, 4, 8, 64, 64, 2, 0, p, 1 << 20, None) == 2
+    assert lib.smoe_up_projection_forward(p, q, 64, 64, None, p, p, p, None, p, 4, 8, 64, 64, 2, 0, p, 1 << 20,
+                                          None) == 2
     assert b"16-byte aligned" in lib.smoe_last_error()
-    assert lib.smoe_down_projection_forward(p, p, 64 * 64, 68, None, p, p, 8, 64, 64, 2, p, 1 << 20, None) == 2
+    assert lib.smoe_down_projection_forward(p, p, 64 * 64, 68, None, p, p, None, 8, 64, 64, 2, p, 1 << 20, None) == 2
     assert b"multiples of 8" in lib.smoe_last_error()
 
 

@@ -216,6 +216,62 @@ def test_kernel_selection_knobs(dev, tuning, knob, value):
         assert torch.equal(a, b), name
 
 
+@pytest.mark.parametrize("stream_kernels", [1, 0])
+@pytest.mark.parametrize("order_kind", ["reversed", "largest_first", "random"])
+def test_expert_schedule_order(dev, tuning, order_kind, stream_kernels):
+    """The four grouped-GEMM operators with an expert_schedule_order (the reference operators' argument,
+    sonicmoe/functional/forward.py:61, backward.py:204, :298): every permutation of the experts gives the results of
+    the default order bit for bit -- only the order in which the tiles are taken up changes."""
+    fwd, bwd = _ops()
+    tuning("gemm_stream", stream_kernels)
+    tuning("gemm_stream_grid", 16)
+    T, H, I, E, K = 3072, 512, 256, 24, 4
+    _, w1, w2 = make_weights(E, H, I, dev, seed=41)
+    idx, scores, meta, md = make_tc_routing(T, E, K, dev, seed=42, skew=1.0, empty=(5, 23))
+    g = torch.Generator().manual_seed(43)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    dout = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    TK = T * K
+    off, gidx, sidx = (md[k] for k in ("expert_frequency_offset", "x_gather_idx", "s_scatter_idx"))
+    stream = torch.cuda.current_stream().cuda_stream
+    s_flat = torch.from_numpy(scores).to(dev).view(-1)
+    if order_kind == "reversed":
+        order = torch.arange(E - 1, -1, -1, dtype=torch.int32, device=dev)
+    elif order_kind == "largest_first":
+        from sonicmoe.functional import largest_first_schedule_order
+
+        order = largest_first_schedule_order(off)
+        counts = off.diff()
+        assert bool((counts[order.long()].diff() <= 0).all()) and sorted(order.tolist()) == list(range(E))
+    else:
+        order = torch.randperm(E, generator=g).to(torch.int32).to(dev)
+
+    def run(order):
+        z = torch.empty(TK, 2 * I, dtype=torch.bfloat16, device=dev)
+        y1 = torch.empty(TK, I, dtype=torch.bfloat16, device=dev)
+        fwd._up_projection_forward(x, w1.permute(1, 2, 0), z, y1, None, off, order, gidx, stream, "swiglu", True, False)
+        y2 = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
+        fwd._down_projection_forward(w2.permute(1, 2, 0), y1, y2, None, off, order, gidx, stream)
+        dw2 = torch.full((E, H, I), 3.0, dtype=torch.bfloat16, device=dev).permute(1, 2, 0)
+        dz = torch.empty_like(z)
+        ds = torch.empty(TK, dtype=torch.float32, device=dev)
+        bwd._down_projection_backward(dout, z, w2.permute(1, 2, 0), dw2, dz, ds, None, None, s_flat, off, order, gidx,
+                                      sidx, stream, True, "swiglu")
+        dw1 = torch.full((E, 2 * I, H), 3.0, dtype=torch.bfloat16, device=dev).permute(1, 2, 0)
+        dxe = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
+        bwd._up_projection_backward(x, w1.permute(1, 2, 0), dxe, dw1, dz, None, off, order, gidx, sidx, True, stream)
+        return z, y1, y2, dz, ds, dw2, dw1, dxe
+
+    base = run(None)
+    other = run(order)
+    for name, a, b in zip(["z", "y1", "y2", "dz", "ds", "dw2", "dw1", "dx_expanded"], base, other):
+        assert torch.equal(a, b), name
+    with pytest.raises(ValueError, match="expert_schedule_order"):
+        run(order.long())
+    with pytest.raises(ValueError, match="expert_schedule_order"):
+        run(order[:-1])
+
+
 @pytest.mark.parametrize("T,E,H", [(4096, 64, 512), (300, 128, 256), (1000, 8, 64), (8192, 128, 1024), (5000, 264, 320)])
 def test_router_weight_grad(dev, T, E, H):
     """dWr = dlogits^T x as a token-split GEMM (partials summed by the caller) against the fp32 product; ragged last
