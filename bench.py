@@ -151,6 +151,21 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
                 ("fp8:quantize(W2)", lambda: fp8._mx_quantize(w2_2d, w2q, w2s), None, E * H * I * 3 + E * H * I // 32),
                 ("fp8:down_projection_forward", lambda: fp8._down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, None, off, E, stream), gemm, None),
             ]
+            # fp8 activation gradients: dout and the transposed weights quantised, dz (+ its quantised copy), dx
+            doq, dos = fp8.mx_quantize(dout)
+            w2tq, w2ts = fp8.quantize_expert_weight_transposed(w2v)
+            w1tq, w1ts = fp8.quantize_expert_weight_transposed(w1v)
+            w2t3, w1t3 = w2tq.view(E, I, H), w1tq.view(E, H, 2 * I)
+            dzq = torch.empty(TK, 2 * I, dtype=torch.uint8, device=dev)
+            dzs = torch.empty(2 * I // 128, TK, dtype=torch.int32, device=dev)
+            y1sc = torch.empty(TK, I, dtype=bf, device=dev)
+            ops += [
+                ("fp8:quantize(dout)", lambda: fp8._mx_quantize(dout, doq, dos), None, T * H * 3 + T * H // 32),
+                ("fp8:quantize_transposed(W2)", lambda: fp8._mx_quantize_transposed(w2.detach(), w2t3, w2ts), None, E * H * I * 3 + E * H * I // 32),
+                ("fp8:down_projection_backward(dz, +quantised dz)", lambda: fp8._down_projection_backward_fp8(doq, dos, w2tq, w2ts, z, dz, dzq, dzs, y1sc, ds, sflat, off, gidx, sidx, E, stream, "swiglu", True), gemm, None),
+                ("fp8:quantize_transposed(W1)", lambda: fp8._mx_quantize_transposed(w1.detach(), w1t3, w1ts), None, E * 2 * I * H * 3 + E * 2 * I * H // 32),
+                ("fp8:up_projection_backward(dx)", lambda: fp8._down_projection_forward_fp8(dzq, dzs, w1tq, w1ts, dxe, None, off, E, stream), 2 * gemm, None),
+            ]
         rows = []
         for name, fn, flops, nbytes in ops:
             if only is not None and name != only:
@@ -374,7 +389,8 @@ def measure_layer(cfg, name, dev, steps, warmup):
         f"{rec['ms_per_step_median']:.3f} median / {rec['ms_per_step_min']:.3f} min ({tflops:.1f} TFLOP/s = "
         f"{100 * tflops / PEAK_BF16_TFLOPS:.1f}% of bf16 MFMA peak); kept for backward "
         f"{held_for_backward / 2**30:.2f} GiB, peak of a step {peak_step / 2**30:.2f} GiB above the resident tensors")
-    return rec, dict(x=x, wr=wr, w1=w1, w2=w2, dout=dout, layer=layer, fwd_only=fwd_only, flops_fwd=flops_fwd)
+    return rec, dict(x=x, wr=wr, w1=w1, w2=w2, dout=dout, layer=layer, fwd_only=fwd_only, fwd_bwd=fwd_bwd,
+                     flops_fwd=flops_fwd, flops_all=flops_all)
 
 
 def main():
@@ -406,9 +422,9 @@ def main():
     rec, t = measure_layer(cfg, a.config, dev, a.steps, a.warmup)
     rounding = cfg.get("rounding")
 
-    fp8_info = None
+    fp8_info = fp8_step = None
     if not rounding and not cfg["zipf"] and H % 128 == 0 and I % 128 == 0:
-        from sonicmoe import enable_fp8_forward
+        from sonicmoe import enable_fp8_backward, enable_fp8_forward
         from sonicmoe.functional.fp8 import cache_quantized_weights
 
         with torch.no_grad():
@@ -430,6 +446,21 @@ def main():
         )
         log(f"fp8 forward: {fp8_ms:.3f} ms ({fp8_info['fwd_tflops']:.1f} TFLOP/s), rel-L2 vs bf16 forward {rel:.4f}")
         del ref_out, fp8_out
+        # the whole step with the four activation-side GEMMs on fp8 operands (weights quantised inside the timed region,
+        # twice each: along either index); the two weight-gradient GEMMs are the bf16 ones
+        with enable_fp8_forward(), enable_fp8_backward(), cache_quantized_weights(False):
+            ms8, _, per8 = time_region(t["fwd_bwd"], a.steps, a.warmup, per_step=True)
+        per8.sort()
+        fp8_step = dict(
+            what="fwd+bwd with x, W1, y1, W2 (forward) and dout, W2^T, dz, W1^T (activation gradients) as block-scaled "
+            "e4m3, every quantisation inside the timed region; dW1, dW2 are bf16 GEMMs",
+            ms_per_step=round(ms8, 4),
+            ms_per_step_median=round(per8[len(per8) // 2], 4),
+            ms_per_step_min=round(per8[0], 4),
+            tflops=round(t["flops_all"] / ms8 / 1e9, 2),
+            frac_of_bf16_peak=round(t["flops_all"] / ms8 / 1e9 / PEAK_BF16_TFLOPS, 4),
+        )
+        log(f"fp8 fwd+bwd: {ms8:.3f} ms ({fp8_step['tflops']:.1f} TFLOP/s of useful work)")
 
     rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, t["x"], t["wr"], t["w1"], t["w2"], t["dout"],
                                                                     max(5, a.steps // 2))
@@ -474,6 +505,7 @@ def main():
         peak_bytes_step=rec["peak_bytes_step"],
         roofline=roofline,
         fp8_forward=fp8_info,
+        fp8_fwd_bwd=fp8_step,
         kernels=[{k: v for k, v in r.items() if k != "flops"} for r in rows],
     )
     del t

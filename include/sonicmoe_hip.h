@@ -273,6 +273,35 @@ int smoe_down_projection_forward_fp8(const void* y1q, const void* y1_scales, con
                                      const void* b2, void* y2, const int32_t* off, int64_t TK, int H, int I, int E,
                                      void* workspace, size_t workspace_bytes, void* stream);
 
+/* The same kernel serves dx_expanded = dz W1[e] (the activation-gradient half of sonicmoe::_up_projection_backward,
+ * sonicmoe/functional/backward.py:195-283) with fp8 operands: pass dzq (TK, N1) + its scales as y1q, the transposed
+ * quantised W1 (E, H, N1) as w2q, and N1 for I. */
+
+/* Quantise the TRANSPOSES of E bf16 matrices along their rows:
+ *   src: matrix e is (R, C) at src + e * src_stride_e, row stride src_stride_r elements; R % 128 == 0, C % 64 == 0
+ *   q (E, C, R) bytes contiguous: q[e][c][r] = e4m3 of src[e][r][c] / scale, 32 consecutive r sharing a scale
+ *   scales (R / 128, E * C) uint32, laid out as smoe_mx_quantize lays out the scales of an (E * C, R) matrix.
+ * This is the weight operand of the two activation-gradient GEMMs, which contract over the weights' output index:
+ * W2 (E, H, I) -> (E, I, H) for dz, W1 (E, N1, H) -> (E, H, N1) for dx. */
+int smoe_mx_quantize_transposed(const void* src, int64_t src_stride_e, int64_t src_stride_r, int E, int R, int C,
+                                void* q, void* scales, void* stream);
+
+/* The activation-gradient half of smoe_down_projection_backward with fp8 operands (no counterpart in the reference,
+ * whose sonicmoe::_down_projection_backward, sonicmoe/functional/backward.py:286-461, is bf16):
+ *   dy1 = doutq[x_gather_idx] w2tq[e]^T with the block scales applied (never stored), then as the bf16 operator:
+ *   dz (TK, N1) bf16, y1s (TK, I) bf16, ds (TK) fp32 in flat-slot order; and dz once more quantised from its bf16
+ *   values: dzq (TK, N1) bytes + dzq_scales (N1/128, TK), the operand of the fp8 dx GEMM.
+ *   doutq (T, H) bytes + dout_scales (H/128, T); w2tq (E, I, H) bytes + w2t_scales (H/128, E*I)
+ *   (smoe_mx_quantize_transposed of W2); z (TK, N1) bf16; ds_partial: TK * smoe_dz_partial_cols(I) floats.
+ * The weight and bias gradients are left to smoe_down_projection_backward with dz == NULL, which reads y1s.
+ * Limits: H % 128 == 0, I % 64 == 0, N1 % 128 == 0; no b2 term in ds. */
+int smoe_down_projection_backward_fp8(const void* doutq, const void* dout_scales, const void* w2tq,
+                                      const void* w2t_scales, const void* z, void* dz, void* dzq, void* dzq_scales,
+                                      void* y1s, float* ds, float* ds_partial, const float* scores,
+                                      const int32_t* off, const int32_t* x_gather_idx, const int32_t* s_scatter_idx,
+                                      int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                      size_t workspace_bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

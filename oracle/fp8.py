@@ -1,4 +1,4 @@
-"""CPU restatement of the fp8 forward path (block-scaled OCP e4m3).  TEST INFRASTRUCTURE ONLY.
+"""CPU restatement of the fp8 path (block-scaled OCP e4m3).  TEST INFRASTRUCTURE ONLY.
 
 PARITY UNPINNED against the reference: the reference (sonicmoe/functional/*.py) computes in bf16 only and holds no fp8
 code, test or number.  What is pinned here is the format, not a reference behaviour:
@@ -6,8 +6,8 @@ code, test or number.  What is pinned here is the format, not a reference behavi
   e4m3_table        pinned: every one of the 256 codes against torch.float8_e4m3fn's own decoding
   mx_quantize       pinned: elements against torch's float -> float8_e4m3fn cast of x / scale (round to nearest even);
                     scales against their defining inequalities (power of two, amax / scale in (224, 448])
-  *_forward_fp8     the operator restatements of oracle.moe_math evaluated on the de-quantised operands: the product
-                    kernels must match THESE tightly (same operands, fp32 accumulation), and the unquantised oracle
+  *_forward_fp8,    the operator restatements of oracle.moe_math evaluated on the de-quantised operands: the product
+  *_backward_fp8    kernels must match THESE tightly (same operands, fp32 accumulation), and the unquantised oracle
                     within the fp8 tolerance
 
 Format: along the contraction dimension every 32 consecutive elements share one power-of-two scale 2^(byte - 127);
@@ -106,3 +106,27 @@ def up_projection_forward_fp8(x, w1, off, gidx, b1=None, activation="swiglu"):
 def down_projection_forward_fp8(y1, w2, off, b2=None):
     """moe_math.down_projection_forward on the de-quantised y1 and W2 (contraction along I)."""
     return M.down_projection_forward(fake_quant(y1), fake_quant(w2), off.cpu(), b2=None if b2 is None else b2.cpu())
+
+
+def fake_quant_transposed(w: torch.Tensor) -> torch.Tensor:
+    """(E, R, C): every matrix quantised along R (32 consecutive r of a column share a scale), de-quantised, same shape."""
+    return fake_quant(w.transpose(1, 2).contiguous()).transpose(1, 2).contiguous()
+
+
+def down_projection_backward_fp8(dout, z, w2, scores_flat, off, gidx, sidx, activation="swiglu"):
+    """The activation-gradient half of moe_math.down_projection_backward with dy1 formed from the de-quantised dout
+    (blocks along H) and W2 (blocks along H, i.e. along the rows of each (H, I) matrix).  Returns (dz, y1s, ds)."""
+    dz, y1s, ds, _ = M.down_projection_backward(fake_quant(dout), z, fake_quant_transposed(w2), scores_flat, off.cpu(),
+                                                gidx.cpu(), sidx.cpu(), activation=activation)
+    return dz, y1s, ds
+
+
+def dx_fp8(dz, w1, off):
+    """dx_expanded[m] = dz[m] W1[e] on the de-quantised dz (blocks along its N1 columns) and W1 (blocks along N1, the
+    rows of each (N1, H) matrix)."""
+    dzq, w1q = fake_quant(dz), fake_quant_transposed(w1)
+    out = torch.empty(dz.size(0), w1.size(2))
+    o = off.tolist()
+    for e in range(w1.size(0)):
+        out[o[e]:o[e + 1]] = dzq[o[e]:o[e + 1]] @ w1q[e].float()
+    return out

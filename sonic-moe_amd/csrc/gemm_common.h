@@ -728,6 +728,185 @@ SMOE_DEV void forward_epilogue_rows(typename Mma::Acc (&acc)[TN / Mma::FR][TM / 
   });
 }
 
+// ---- epilogue of the activation-gradient GEMM of the down projection (dz) -------------------------------------------
+// acc = dy1 (token rows x I columns) of the wave's TM x TN tile.  32 token rows at a time the wavefront stages its z
+// sub-tile (32 rows x ZW*TN bf16; ZW = 2 interleaved (gate, up) columns per dy1 column for gated activations, 1
+// otherwise) through LDS: row-contiguous 16-byte global loads (PF batches in flight in registers) -> LDS -> each lane
+// picks the z values of its four dy1 columns of its token rows, computes dz in place and y1s into a second area -> both
+// are written back row-contiguous.  All global traffic of the epilogue is full 128-byte lines.
+struct DzEpilogueArgs {
+  const uint16_t* zin;
+  int64_t zin_stride;
+  uint16_t* dz;  // (rows, ZW * N) bf16
+  int64_t dz_stride;
+  uint16_t* y1s;  // (rows, N) bf16: score * act(z)
+  int64_t y1s_stride;
+  const float* scores;
+  const int32_t* sidx;
+  float* ds_partial;  // (rows, ds_cols) fp32: this wave writes column ds_col, sum_i dy1 * y1 over its columns
+  int ds_cols, ds_col;
+  int m_base, row_end;  // first grouped row of this wave's tile, end of the expert's rows
+  int n_base, N;        // first dy1 column of this wave's tile, number of dy1 columns (I)
+  // with QUANT: dz once more as e4m3 bytes (rows, ZW * N) with one power-of-two scale per 32 columns, the operand format
+  // of the fp8 GEMMs: scale word [c / 128][row] of a (ZW * N / 128, dzq_rows) table, byte (c / 32) % 4.  Quantised
+  // from the bf16-rounded values, so it equals quantising the stored dz.
+  uint8_t* dzq;
+  uint32_t* dzq_scales;
+  int64_t dzq_rows;
+};
+
+template <int TN, int ACT>
+struct DzStaging {
+  static constexpr int ZW = act_is_glu(ACT) ? 2 : 1;
+  static constexpr int ZB = TN * 2 * ZW, YB = TN * 2;  // bytes per staged z / dz row, y1s row
+  static constexpr int BYTES = 32 * (ZB + YB);         // per wavefront
+};
+
+// e8m0 exponent of the smallest power of two s with amax / s <= 448 (the largest e4m3 value): no element saturates
+SMOE_DEV int mx_scale_exponent(float amax) {
+  if (!(amax > 0.f)) return 0;
+  // amax = m * 2^e with m in [1, 2): 448 = 1.75 * 2^8 -> need 2^k >= amax / 448
+  const uint32_t bits = __float_as_uint(amax);
+  const int e = (int)((bits >> 23) & 0xff) - 127;
+  const uint32_t mant = bits & 0x7fffffu;
+  int k = e - 8;                      // 2^(e-8) * 448 = 1.75 * 2^e
+  if (mant > 0x600000u) k += 1;       // m > 1.75
+  k += 127;
+  return k < 0 ? 0 : (k > 254 ? 254 : k);
+}
+
+template <class Mma, int TM, int TN, int ACT, int PF = 2, bool QUANT = false, class RingIdle>
+SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* zbuf, int lane,
+                          const DzEpilogueArgs& a, RingIdle&& ring_idle) {
+  using AL = AccLayout<Mma>;
+  constexpr bool GLU = act_is_glu(ACT);
+  constexpr int PW = act_pointwise(ACT);
+  constexpr int FR = Mma::FR, FN = TN / FR, QPF = AL::QPF;
+  constexpr int ZW = DzStaging<TN, ACT>::ZW, ZB = DzStaging<TN, ACT>::ZB, YB = DzStaging<TN, ACT>::YB;
+  constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
+  constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
+  constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;  // row swizzle of the staged z chunks
+  constexpr int NB = TM / 32, RB = 32 / FR;   // 32-row batches; fragment rows per batch
+  static_assert(PF == 1 || PF == 2, "one or two batches of z are prefetched");
+  char* ybuf = zbuf + 32 * ZB;
+  const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
+  const int zlimit = ZW * a.N;
+  const int zcol = ZW * a.n_base + zc * 8;  // first z column of this lane's 16-byte chunk
+  const int zcol_c = zcol <= zlimit - 8 ? zcol : zlimit - 8;
+  u32x4 zreg[PF][ZN];
+  auto fetch_z = [&](int blk, u32x4(&dst)[ZN]) {
+#pragma unroll
+    for (int it = 0; it < ZN; it++) {
+      int m = a.m_base + blk * 32 + it * ZR + zr;
+      m = m < a.row_end ? m : a.row_end - 1;
+      dst[it] = *(const u32x4*)(a.zin + (int64_t)m * a.zin_stride + zcol_c);
+    }
+  };
+  fetch_z(0, zreg[0]);
+  if constexpr (NB > 1 && PF > 1) fetch_z(1, zreg[1]);
+  ring_idle();  // the staging areas lie in the ring: every wave must be done reading it
+  static_for<NB>([&](auto blk_c) {
+    constexpr int blk = decltype(blk_c)::value;
+#pragma unroll
+    for (int it = 0; it < ZN; it++) {
+      const int r = it * ZR + zr;
+      *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4)) = zreg[blk % PF][it];
+    }
+    if constexpr (blk + PF < NB) fetch_z(blk + PF, zreg[blk % PF]);
+    static_for<RB>([&](auto sub_c) {
+      constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
+      const int mrow = sub * FR + AL::row(lane);  // row inside the staged batch
+      const int m = a.m_base + blk * 32 + mrow;
+      const bool mvalid = m < a.row_end;
+      float sc = 0.f, dsum = 0.f;
+      if (mvalid) sc = a.scores[a.sidx[m]];
+      static_for<FN * QPF>([&](auto q_c) {
+        constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+        const int il = fn * FR + AL::col(rg, lane);  // first of this lane's 4 dy1 columns (wave-local)
+        const int zbyte = il * 2 * ZW;                // their z bytes inside the staged row
+        char* zaddr = zbuf + mrow * ZB + (((zbyte >> 4) ^ (mrow & ZSW)) << 4) + (zbyte & 15);
+        float ys[4];
+        if constexpr (GLU) {
+          const u32x4 zz = *(const u32x4*)zaddr;
+          u32x4 dzv;
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float dy = acc[fn][fm][4 * rg + q];
+            const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
+            float f, fp;
+            pointwise_grad<PW>(g, f, fp);
+            const float y1v = f * u;
+            if (a.n_base + il + q < a.N) dsum += dy * y1v;
+            const float sd = sc * dy;
+            dzv[q] = pack_bf16x2(sd * u * fp, sd * f);
+            ys[q] = sc * y1v;
+          }
+          *(u32x4*)zaddr = dzv;
+        } else {
+          const u32x2 zz = *(const u32x2*)zaddr;
+          float dzf[4];
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float dy = acc[fn][fm][4 * rg + q];
+            const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
+            float f, fp;
+            pointwise_grad<PW>(t, f, fp);
+            if (a.n_base + il + q < a.N) dsum += dy * f;
+            dzf[q] = sc * dy * fp;
+            ys[q] = sc * f;
+          }
+          *(u32x2*)zaddr = u32x2{pack_bf16x2(dzf[0], dzf[1]), pack_bf16x2(dzf[2], dzf[3])};
+        }
+        u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
+        epi_park_y<YB>(ybuf, mrow, il * 2, yv);
+      });
+      // the 64 / FR lanes that share a token row hold disjoint columns: add their partial sums
+      dsum += __shfl_xor(dsum, 32, 64);
+      if constexpr (FR == 16) dsum += __shfl_xor(dsum, 16, 64);
+      if (mvalid && lane < FR) a.ds_partial[(int64_t)m * a.ds_cols + a.ds_col] = dsum;
+    });
+#pragma unroll
+    for (int it = 0; it < ZN; it++) {
+      const int r = it * ZR + zr;
+      const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4));
+      const int mm = a.m_base + blk * 32 + r;
+      const bool live = mm < a.row_end && zcol < zlimit;
+      if (live) *(u32x4*)(a.dz + (int64_t)mm * a.dz_stride + zcol) = v;
+      if constexpr (QUANT) {
+        // 32 columns = the 16-byte chunks of 4 consecutive lanes
+        float x[8];
+        float amax = 0.f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          x[2 * q] = bf16_lo(v[q]);
+          x[2 * q + 1] = bf16_hi(v[q]);
+          amax = fmaxf(amax, fmaxf(fabsf(x[2 * q]), fabsf(x[2 * q + 1])));
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 64));
+        const int ex = mx_scale_exponent(amax);
+        const float inv = __uint_as_float((uint32_t)(254 - ex) << 23);
+        int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(x[0] * inv, x[1] * inv, 0, false);
+        w0 = __builtin_amdgcn_cvt_pk_fp8_f32(x[2] * inv, x[3] * inv, w0, true);
+        int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(x[4] * inv, x[5] * inv, 0, false);
+        w1 = __builtin_amdgcn_cvt_pk_fp8_f32(x[6] * inv, x[7] * inv, w1, true);
+        if (live) {
+          *(u32x2*)(a.dzq + (int64_t)mm * zlimit + zcol) = u32x2{(uint32_t)w0, (uint32_t)w1};
+          if ((zc & 3) == 0)
+            ((uint8_t*)a.dzq_scales)[((int64_t)(zcol >> 7) * a.dzq_rows + mm) * 4 + ((zcol >> 5) & 3)] = (uint8_t)ex;
+        }
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < YN; it++) {
+      const int r = it * YR + yr;
+      const u32x4 v = *(const u32x4*)(ybuf + r * YB + ((yc ^ ((r >> 1) & (YL < 8 ? YL - 1 : 7))) << 4));
+      const int mm = a.m_base + blk * 32 + r, col = a.n_base + yc * 8;
+      if (mm < a.row_end && col < a.N) *(u32x4*)(a.y1s + (int64_t)mm * a.y1s_stride + col) = v;
+    }
+  });
+}
+
 // ---- tuning knobs ----------------------------------------------------------------------------------------------
 // Read from the environment ONCE, at the first launch that asks (variable = "SMOE_" + the upper-cased field name);
 // smoe_set_tuning() overrides a knob afterwards (tests walk through the alternative kernels with it).

@@ -12,7 +12,11 @@
 // The GEMM is the K-major / K-major kernel of the bf16 path with 128 BYTES of contraction per row and stage:
 //   up-projection    P = x rows gathered (fp8), Q = W1[e] (fp8)  -> z (bf16), y1 = act(z) (bf16)
 //   down-projection  P = y1 rows (fp8),        Q = W2[e] (fp8)  -> y2 (bf16)
-// Accumulation is fp32; outputs, biases and epilogues are those of the bf16 kernels.
+//   dz               P = dout rows gathered,   Q = W2[e]^T       -> dz, y1s (bf16), ds partial sums, dz again in fp8
+//   dx               P = dz rows (fp8),        Q = W1[e]^T       -> dx_expanded (bf16)   (the down-projection kernel)
+// Accumulation is fp32; outputs, biases and epilogues are those of the bf16 kernels.  The two activation-gradient
+// GEMMs contract over the other index of the weights, so they read transposed quantised copies (the transposing
+// quantiser below); the weight-gradient GEMMs, which contract over the tokens, stay in bf16.
 #include "gemm_common.h"
 
 namespace smoe {
@@ -20,19 +24,6 @@ namespace smoe {
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 // ---- quantiser ---------------------------------------------------------------------------------------------------
-// e8m0 exponent of the smallest power of two s with amax / s <= 448 (the largest e4m3 value): no element saturates
-SMOE_DEV int mx_scale_exponent(float amax) {
-  if (!(amax > 0.f)) return 0;
-  // amax = m * 2^e with m in [1, 2): 448 = 1.75 * 2^8 -> need 2^k >= amax / 448
-  const uint32_t bits = __float_as_uint(amax);
-  const int e = (int)((bits >> 23) & 0xff) - 127;
-  const uint32_t mant = bits & 0x7fffffu;
-  int k = e - 8;                      // 2^(e-8) * 448 = 1.75 * 2^e
-  if (mant > 0x600000u) k += 1;       // m > 1.75
-  k += 127;
-  return k < 0 ? 0 : (k > 254 ? 254 : k);
-}
-
 // one lane = one 32-element block: 64 bytes in, 32 bytes + 1 scale byte out
 __global__ __launch_bounds__(256) void mx_quantize_kernel(const uint16_t* __restrict__ src, int64_t src_stride,
                                                           int64_t R, int C, uint8_t* __restrict__ q,
@@ -104,6 +95,13 @@ struct Fp8Params {
   uint32_t* yq_scales; // its scale table (I / 128, TK)
   int64_t yq_rows;     // TK
   int I;
+  // dz role: out0 = dz, out1 = y1s, yq / yq_scales / yq_rows = dz in fp8; N = I
+  const uint16_t* zin;
+  int64_t zin_stride;
+  const float* scores;
+  const int32_t* sidx;
+  float* ds_partial;
+  int ds_cols;
 };
 
 struct Fp8Cfg {
@@ -219,7 +217,8 @@ SMOE_DEV void fp8_activation_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wav
   });
 }
 
-template <bool WITH_ACT, int ACT>
+// WITH_ACT: up-projection epilogue (activation ACT); DZ: epilogue of the down projection's activation gradient
+template <bool WITH_ACT, int ACT, bool DZ = false>
 __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Params p) {
   using C = Fp8Cfg;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -350,6 +349,34 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
   };
   gemm_mainloop<FN, FM, 3 * (FN + FM), C::P_INSTR + C::Q_INSTR + C::S_INSTR, SLICES, C::NSTAGE, Fp8Mma>(S_total, acc, issue, load);
 
+  if constexpr (DZ) {
+    DzEpilogueArgs da = {};
+    da.zin = p.zin;
+    da.zin_stride = p.zin_stride;
+    da.dz = p.out0;
+    da.dz_stride = p.out0_stride;
+    da.y1s = p.out1;
+    da.y1s_stride = p.out1_stride;
+    da.scores = p.scores;
+    da.sidx = p.sidx;
+    da.ds_partial = p.ds_partial;
+    da.ds_cols = p.ds_cols;
+    da.ds_col = nt * C::WN + wn;
+    da.m_base = row0 + wm * C::TM;
+    da.row_end = row_end;
+    da.n_base = n0 + wn * C::TN;
+    da.N = p.N;
+    da.dzq = p.yq;
+    da.dzq_scales = p.yq_scales;
+    da.dzq_rows = p.yq_rows;
+    static_assert(C::NW * DzStaging<C::TN, ACT>::BYTES <= C::SMEM, "dz staging must fit into the idle stages");
+    dz_epilogue<Fp8Mma, C::TM, C::TN, ACT, 1, true>(acc, smem + wave * DzStaging<C::TN, ACT>::BYTES, lane, da, [&]() {
+      wait_vmem_all();
+      wait_lds_all();
+      lds_barrier();  // every wave has finished reading the last stage
+    });
+    return;
+  }
   FwdEpilogueArgs ea;
   ea.bias = p.bias ? p.bias + (int64_t)e * p.N : nullptr;
   ea.out0 = p.out0;
@@ -370,11 +397,11 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
   }
 }
 
-template <bool WITH_ACT, int ACT>
+template <bool WITH_ACT, int ACT, bool DZ = false>
 static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
   using C = Fp8Cfg;
   static LdsLimitOnce lds_limit;
-  auto kern = fp8_varlen_m_kernel<WITH_ACT, ACT>;
+  auto kern = fp8_varlen_m_kernel<WITH_ACT, ACT, DZ>;
   {
     const int rc_attr = lds_limit.ensure((const void*)kern, C::SMEM);
     if (rc_attr) return rc_attr;
@@ -383,6 +410,7 @@ static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t
   int rc = launch_build_tile_map(off, nullptr, E, C::BM, p.tm, st);
   if (rc) return rc;
   p.n_tiles = (int)ceil_div(p.N, C::BN);
+  if (DZ) p.ds_cols = p.n_tiles * C::WN;
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: too many tiles");
@@ -405,9 +433,100 @@ static int launch_fp8_up(int act, Fp8Params& p, const int32_t* off, void* ws, in
   return SMOE_ERR_INVALID;
 }
 
+static int launch_fp8_dz(int act, Fp8Params& p, const int32_t* off, void* ws, int64_t TK, int E, hipStream_t st) {
+  switch (act) {
+    case SMOE_ACT_SWIGLU: return launch_fp8<false, SMOE_ACT_SWIGLU, true>(p, off, ws, TK, E, st);
+    case SMOE_ACT_GEGLU: return launch_fp8<false, SMOE_ACT_GEGLU, true>(p, off, ws, TK, E, st);
+    case SMOE_ACT_REGLU: return launch_fp8<false, SMOE_ACT_REGLU, true>(p, off, ws, TK, E, st);
+    case SMOE_ACT_RELU_SQ: return launch_fp8<false, SMOE_ACT_RELU_SQ, true>(p, off, ws, TK, E, st);
+    case SMOE_ACT_RELU: return launch_fp8<false, SMOE_ACT_RELU, true>(p, off, ws, TK, E, st);
+    case SMOE_ACT_GELU: return launch_fp8<false, SMOE_ACT_GELU, true>(p, off, ws, TK, E, st);
+    case SMOE_ACT_SILU: return launch_fp8<false, SMOE_ACT_SILU, true>(p, off, ws, TK, E, st);
+  }
+  set_error("unknown activation code %d", act);
+  return SMOE_ERR_INVALID;
+}
+
+// ---- transposing quantiser -----------------------------------------------------------------------------------------
+// src: E matrices (R, C) bf16, row stride src_stride_r, matrix stride src_stride_e.  q: E matrices (C, R) e4m3, the
+// transposes, quantised along R (32 consecutive r share a scale); scales (R / 128, E * C) words as in mx_quantize.
+// One workgroup transposes a 128 (r) x 64 (c) tile through LDS: row-contiguous loads, column reads (one lane = one
+// column and one 32-row block), bytes parked transposed, row-contiguous stores of 128 bytes per output row.
+__global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint16_t* __restrict__ src,
+                                                                     int64_t src_stride_e, int64_t src_stride_r, int R,
+                                                                     int C, int E, uint8_t* __restrict__ q,
+                                                                     uint32_t* __restrict__ scales) {
+  constexpr int TR = 128, TC = 64, IN_PITCH = TC * 2 + 4, OUT_PITCH = TR + 8;
+  __shared__ __attribute__((aligned(16))) char tile_in[TR * IN_PITCH];
+  __shared__ __attribute__((aligned(16))) char tile_out[TC * OUT_PITCH];
+  __shared__ uint8_t exps[TC][4];
+  const int tid = threadIdx.x;
+  const int c0 = blockIdx.x * TC, r0 = blockIdx.y * TR, e = blockIdx.z;
+  const uint16_t* base = src + (int64_t)e * src_stride_e + (int64_t)r0 * src_stride_r + c0;
+  // 8 lanes x 16 bytes per input row, 32 rows per pass
+#pragma unroll
+  for (int pass = 0; pass < TR / 32; pass++) {
+    const int r = pass * 32 + tid / 8, piece = tid % 8;
+    const u32x4 v = *(const u32x4*)(base + (int64_t)r * src_stride_r + piece * 8);
+    uint32_t* dst = (uint32_t*)(tile_in + r * IN_PITCH + piece * 16);
+    dst[0] = v[0];
+    dst[1] = v[1];
+    dst[2] = v[2];
+    dst[3] = v[3];
+  }
+  __syncthreads();
+  const int c = tid % TC, rb = tid / TC;  // this lane's column and 32-row block
+  float v[32];
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 32; i++) {
+    const uint16_t h = *(const uint16_t*)(tile_in + (rb * 32 + i) * IN_PITCH + c * 2);
+    v[i] = __uint_as_float((uint32_t)h << 16);
+    amax = fmaxf(amax, fabsf(v[i]));
+  }
+  const int ex = mx_scale_exponent(amax);
+  const float inv = __uint_as_float((uint32_t)(254 - ex) << 23);
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i] * inv, v[8 * i + 1] * inv, 0, false);
+    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 2] * inv, v[8 * i + 3] * inv, w0, true);
+    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 4] * inv, v[8 * i + 5] * inv, 0, false);
+    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 6] * inv, v[8 * i + 7] * inv, w1, true);
+    *(u32x2*)(tile_out + c * OUT_PITCH + rb * 32 + i * 8) = u32x2{(uint32_t)w0, (uint32_t)w1};
+  }
+  exps[c][rb] = (uint8_t)ex;
+  __syncthreads();
+  // 16 lanes x 8 bytes per output row, 16 rows per pass
+  uint8_t* qbase = q + ((int64_t)e * C + c0) * R + r0;
+#pragma unroll
+  for (int pass = 0; pass < TC / 16; pass++) {
+    const int cc = pass * 16 + tid / 16, piece = tid % 16;
+    const u32x2 w = *(const u32x2*)(tile_out + cc * OUT_PITCH + piece * 8);
+    *(u32x2*)(qbase + (int64_t)cc * R + piece * 8) = w;
+  }
+  if (tid < TC) scales[(int64_t)(r0 / 128) * ((int64_t)E * C) + (int64_t)e * C + c0 + tid] = *(const uint32_t*)exps[tid];
+}
+
 }  // namespace smoe
 
 using namespace smoe;
+
+extern "C" int smoe_mx_quantize_transposed(const void* src, int64_t src_stride_e, int64_t src_stride_r, int E, int R,
+                                           int C, void* q, void* scales, void* stream) {
+  SMOE_REQUIRE(E >= 1 && R > 0 && C > 0, SMOE_ERR_INVALID, "mx_quantize_transposed: bad shape");
+  SMOE_REQUIRE(R % 128 == 0 && C % 64 == 0, SMOE_ERR_UNSUPPORTED,
+               "mx_quantize_transposed: (%d, %d) matrices: rows must be a multiple of 128, columns of 64", R, C);
+  SMOE_REQUIRE(src_stride_e % 8 == 0 && src_stride_r % 8 == 0, SMOE_ERR_UNSUPPORTED,
+               "mx_quantize_transposed: strides must be multiples of 8 elements");
+  SMOE_REQUIRE(src && q && scales, SMOE_ERR_INVALID, "mx_quantize_transposed: null pointer");
+  SMOE_REQUIRE_ALIGNED("mx_quantize_transposed", src, q, scales);
+  SMOE_REQUIRE(E < 65536 && R / 128 < 65536, SMOE_ERR_UNSUPPORTED, "mx_quantize_transposed: tensor too large");
+  hipLaunchKernelGGL(mx_quantize_transposed_kernel, dim3((unsigned)(C / 64), (unsigned)(R / 128), (unsigned)E),
+                     dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, src_stride_e, src_stride_r, R, C, E,
+                     (uint8_t*)q, (uint32_t*)scales);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
 
 extern "C" int smoe_mx_quantize(const void* src, int64_t src_stride, int64_t R, int C, void* q, void* scales,
                                 void* stream) {
@@ -506,4 +625,56 @@ extern "C" int smoe_down_projection_forward_fp8(const void* y1q, const void* y1_
   p.out0 = (uint16_t*)y2;
   p.out0_stride = H;
   return launch_fp8<false, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, (hipStream_t)stream);
+}
+
+extern "C" int smoe_down_projection_backward_fp8(const void* doutq, const void* dout_scales, const void* w2tq,
+                                                 const void* w2t_scales, const void* z, void* dz, void* dzq,
+                                                 void* dzq_scales, void* y1s, float* ds, float* ds_partial,
+                                                 const float* scores, const int32_t* off,
+                                                 const int32_t* x_gather_idx, const int32_t* s_scatter_idx, int64_t T,
+                                                 int64_t TK, int H, int I, int E, int activation, void* workspace,
+                                                 size_t workspace_bytes, void* stream) {
+  SMOE_REQUIRE(activation >= SMOE_ACT_SWIGLU && activation <= SMOE_ACT_SILU, SMOE_ERR_INVALID,
+               "down_projection_backward_fp8: unknown activation code %d", activation);
+  int rc = check_fp8(TK, H, I, E, workspace, workspace_bytes, "down_projection_backward_fp8");
+  if (rc) return rc;
+  const int zw = act_is_glu(activation) ? 2 : 1;
+  SMOE_REQUIRE((zw * I) % 128 == 0, SMOE_ERR_UNSUPPORTED,
+               "down_projection_backward_fp8: the width %d of dz must be a multiple of 128", zw * I);
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(doutq && dout_scales && w2tq && w2t_scales && z && dz && dzq && dzq_scales && y1s && ds && ds_partial &&
+                   scores && off && x_gather_idx && s_scatter_idx && T > 0,
+               SMOE_ERR_INVALID, "down_projection_backward_fp8: null pointer");
+  SMOE_REQUIRE_ALIGNED("down_projection_backward_fp8", doutq, w2tq, z, dz, dzq, y1s);
+  Fp8Params p = {};
+  p.P = (const uint8_t*)doutq;
+  p.p_stride = H;
+  p.p_scales = (const uint32_t*)dout_scales;
+  p.p_rows = T;
+  p.gidx = x_gather_idx;
+  p.Q = (const uint8_t*)w2tq;  // (E, I, H): W2[e]^T, contraction (h) contiguous
+  p.q_stride_e = (int64_t)I * H;
+  p.q_stride_row = H;
+  p.q_scales = (const uint32_t*)w2t_scales;
+  p.q_rows = (int64_t)E * I;
+  p.off = off;
+  p.N = I;
+  p.Kdim = H;
+  p.out0 = (uint16_t*)dz;
+  p.out0_stride = (int64_t)zw * I;
+  p.out1 = (uint16_t*)y1s;
+  p.out1_stride = I;
+  p.yq = (uint8_t*)dzq;
+  p.yq_scales = (uint32_t*)dzq_scales;
+  p.yq_rows = TK;
+  p.I = I;
+  p.zin = (const uint16_t*)z;
+  p.zin_stride = (int64_t)zw * I;
+  p.scores = scores;
+  p.sidx = s_scatter_idx;
+  p.ds_partial = ds_partial;
+  hipStream_t st = (hipStream_t)stream;
+  rc = launch_fp8_dz(activation, p, off, workspace, TK, E, st);
+  if (rc) return rc;
+  return launch_ds_finalize(ds_partial, p.ds_cols, s_scatter_idx, ds, TK, st);
 }

@@ -239,112 +239,27 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     lds_barrier();  // all waves are done reading the last stage
     forward_epilogue<Mma, C::TM, C::TN, ROLE == ROLE_UP_FWD, ACT>(acc, smem, wave, lane, ea);
   } else {
-    // ---- dz epilogue ----
-    // acc = dy1[i][m].  32 token rows at a time the wavefront stages its z sub-tile (32 rows x ZW*TN bf16; ZW = 2
-    // interleaved (gate, up) columns per dy1 column for gated activations, 1 otherwise) through LDS: row-contiguous
-    // 16-byte global loads (two batches in flight in registers) -> LDS -> each lane picks the z values of its four
-    // dy1 columns of its token rows, computes dz in place and y1s into a second area -> both are written back
-    // row-contiguous.  All global traffic of the epilogue is full 128-byte lines.
-    constexpr int ZW = GLU ? 2 : 1;
-    constexpr int ZB = C::TN * 2 * ZW, YB = C::TN * 2;       // bytes per staged z/dz row, y1s row
-    constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
-    constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
-    constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;               // row swizzle of the staged z chunks
-    constexpr int NB = C::TM / 32, RB = 32 / FR;             // 32-row batches; fragment rows per batch
-    static_assert(C::NW * 32 * (ZB + YB) <= C::RING, "dz staging must fit into the idle ring");
-    char* zbuf = smem + wave * (32 * (ZB + YB));
-    char* ybuf = zbuf + 32 * ZB;
-    const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
-    const int zlimit = ZW * p.N;
-    const int zcol = ZW * n_base + zc * 8;  // first z column of this lane's 16-byte chunk
-    const int zcol_c = zcol <= zlimit - 8 ? zcol : zlimit - 8;
-    u32x4 zreg[2][ZN];
-    auto fetch_z = [&](int blk, u32x4(&dst)[ZN]) {
-#pragma unroll
-      for (int it = 0; it < ZN; it++) {
-        int m = m_base + blk * 32 + it * ZR + zr;
-        m = m < row_end ? m : row_end - 1;
-        dst[it] = *(const u32x4*)(p.zin + (int64_t)m * p.zin_stride + zcol_c);
-      }
-    };
-    fetch_z(0, zreg[0]);
-    if constexpr (NB > 1) fetch_z(1, zreg[1]);
-    wait_lds_all();
-    lds_barrier();  // every wave has finished reading the ring
-    static_for<NB>([&](auto blk_c) {
-      constexpr int blk = decltype(blk_c)::value;
-#pragma unroll
-      for (int it = 0; it < ZN; it++) {
-        const int r = it * ZR + zr;
-        *(u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4)) = zreg[blk & 1][it];
-      }
-      if constexpr (blk + 2 < NB) fetch_z(blk + 2, zreg[blk & 1]);
-      static_for<RB>([&](auto sub_c) {
-        constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
-        const int mrow = sub * FR + AL::row(lane);  // row inside the staged batch
-        const int m = m_base + blk * 32 + mrow;
-        const bool mvalid = m < row_end;
-        float sc = 0.f, dsum = 0.f;
-        if (mvalid) sc = p.scores[p.sidx[m]];
-        static_for<FN * QPF>([&](auto q_c) {
-          constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-          const int il = fn * FR + AL::col(rg, lane);  // first of this lane's 4 dy1 columns (wave-local)
-          const int zbyte = il * 2 * ZW;                // their z bytes inside the staged row
-          char* zaddr = zbuf + mrow * ZB + (((zbyte >> 4) ^ (mrow & ZSW)) << 4) + (zbyte & 15);
-          float ys[4];
-          if constexpr (GLU) {
-            const u32x4 zz = *(const u32x4*)zaddr;
-            u32x4 dzv;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-              const float dy = acc[fn][fm][4 * rg + q];
-              const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
-              float f, fp;
-              pointwise_grad<PW>(g, f, fp);
-              const float y1v = f * u;
-              if (n_base + il + q < p.N) dsum += dy * y1v;
-              const float sd = sc * dy;
-              dzv[q] = pack_bf16x2(sd * u * fp, sd * f);
-              ys[q] = sc * y1v;
-            }
-            *(u32x4*)zaddr = dzv;
-          } else {
-            const u32x2 zz = *(const u32x2*)zaddr;
-            float dzf[4];
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-              const float dy = acc[fn][fm][4 * rg + q];
-              const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
-              float f, fp;
-              pointwise_grad<PW>(t, f, fp);
-              if (n_base + il + q < p.N) dsum += dy * f;
-              dzf[q] = sc * dy * fp;
-              ys[q] = sc * f;
-            }
-            *(u32x2*)zaddr = u32x2{pack_bf16x2(dzf[0], dzf[1]), pack_bf16x2(dzf[2], dzf[3])};
-          }
-          u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
-          epi_park_y<YB>(ybuf, mrow, il * 2, yv);
-        });
-        // the 64 / FR lanes that share a token row hold disjoint columns: add their partial sums
-        dsum += __shfl_xor(dsum, 32, 64);
-        if constexpr (FR == 16) dsum += __shfl_xor(dsum, 16, 64);
-        if (mvalid && lane < FR) p.ds_partial[(int64_t)m * p.ds_cols + nt * C::WN + wn] = dsum;
-      });
-#pragma unroll
-      for (int it = 0; it < ZN; it++) {
-        const int r = it * ZR + zr;
-        const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4));
-        const int mm = m_base + blk * 32 + r;
-        if (mm < row_end && zcol < zlimit) *(u32x4*)(p.out0 + (int64_t)mm * p.out0_stride + zcol) = v;
-      }
-#pragma unroll
-      for (int it = 0; it < YN; it++) {
-        const int r = it * YR + yr;
-        const u32x4 v = *(const u32x4*)(ybuf + r * YB + ((yc ^ ((r >> 1) & (YL < 8 ? YL - 1 : 7))) << 4));
-        const int mm = m_base + blk * 32 + r, col = n_base + yc * 8;
-        if (mm < row_end && col < p.N) *(u32x4*)(p.out1 + (int64_t)mm * p.out1_stride + col) = v;
-      }
+    // ---- dz epilogue (dz_epilogue in gemm_common.h) ----
+    DzEpilogueArgs da = {};
+    da.zin = p.zin;
+    da.zin_stride = p.zin_stride;
+    da.dz = p.out0;
+    da.dz_stride = p.out0_stride;
+    da.y1s = p.out1;
+    da.y1s_stride = p.out1_stride;
+    da.scores = p.scores;
+    da.sidx = p.sidx;
+    da.ds_partial = p.ds_partial;
+    da.ds_cols = p.ds_cols;
+    da.ds_col = nt * C::WN + wn;
+    da.m_base = m_base;
+    da.row_end = row_end;
+    da.n_base = n_base;
+    da.N = p.N;
+    static_assert(C::NW * DzStaging<C::TN, ACT>::BYTES <= C::RING, "dz staging must fit into the idle ring");
+    dz_epilogue<Mma, C::TM, C::TN, ACT>(acc, smem + wave * DzStaging<C::TN, ACT>::BYTES, lane, da, [&]() {
+      wait_lds_all();
+      lds_barrier();  // every wave has finished reading the ring
     });
   }
 }

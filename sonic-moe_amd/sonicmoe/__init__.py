@@ -2,7 +2,7 @@
 
 from .count_cumsum import count_cumsum
 from .enums import ActivationType, KernelBackendMoE
-from .functional import enable_fp8_forward, enable_quack_gemm, moe_general_routing_inputs, moe_TC_softmax_topk_layer
+from .functional import enable_fp8_backward, enable_fp8_forward, enable_quack_gemm, moe_general_routing_inputs, moe_TC_softmax_topk_layer
 from .moe import MoE
 
 __all__ = [
@@ -10,6 +10,7 @@ __all__ = [
     "KernelBackendMoE",
     "MoE",
     "count_cumsum",
+    "enable_fp8_backward",
     "enable_fp8_forward",
     "enable_quack_gemm",
     "moe_TC_softmax_topk_layer",

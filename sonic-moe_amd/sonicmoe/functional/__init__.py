@@ -21,6 +21,7 @@ from ..count_cumsum import count_cumsum
 from ..enums import LIBRARY_NAME, ActivationType, is_glu
 from .backward import (
     _down_projection_backward,
+    _down_projection_weight_grad,
     _router_weight_grad,
     _softmax_topk_bwd,
     _switch_loss_bwd,
@@ -36,12 +37,16 @@ from .forward import (
     _up_projection_forward,
 )
 from .fp8 import (
+    _down_projection_backward_fp8,
     _down_projection_forward_fp8,
     _up_projection_forward_fp8,
+    enable_fp8_backward,
     enable_fp8_forward,
+    is_using_fp8_backward,
     is_using_fp8_forward,
     mx_quantize,
     quantize_expert_weight,
+    quantize_expert_weight_transposed,
 )
 from .utils import enable_quack_gemm, is_using_quack_gemm
 
@@ -203,6 +208,15 @@ def largest_first_schedule_order(expert_frequency_offset: torch.Tensor) -> torch
     return torch.argsort(counts, descending=True, stable=True).to(torch.int32)
 
 
+def _fp8_backward_requested(b1, b2) -> bool:
+    """The fp8-backward switch as it stands while the forward pass runs (the backward pass may run outside the block)."""
+    if not is_using_fp8_backward():
+        return False
+    if b1 is not None or b2 is not None:
+        raise NotImplementedError("enable_fp8_backward: layers with biases are not supported")
+    return True
+
+
 def _schedule_order(off):
     return largest_first_schedule_order(off) if _SCHEDULE_POLICY == "largest_first" else None
 
@@ -242,13 +256,17 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
 
 
 def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
-                      activation_type, stream_id, has_b1, order=None):
+                      activation_type, stream_id, has_b1, order=None, fp8=False):
     """Returns (dx, dw1, db1, dw2, db2, ds) of _experts_forward; `has_b1` says whether the forward pass had an
     up-projection bias (b1 itself is not needed for any gradient and is not kept)."""
     T, H = x.shape
     TK = gidx.numel()
     glu = is_glu(activation_type)
     dout = dout.contiguous()
+
+    if fp8:
+        return _experts_backward_fp8(dout, x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK,
+                                     is_varlen_K, activation_type, stream_id, order)
 
     dw2 = torch.empty_like(w2)  # keeps the (E, H, I)-contiguous layout of the parameter view
     db2 = None if b2 is None else torch.empty_like(b2)
@@ -265,6 +283,41 @@ def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx
     dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
     _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
     return dx, dw1, db1, dw2, db2, ds
+
+
+def _experts_backward_fp8(dout, x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
+                          activation_type, stream_id, order):
+    """_experts_backward with the two activation-gradient GEMMs on fp8 operands (no biases): dout and W2^T are
+    quantised for dz, the dz kernel leaves dz in bf16 (for dW1) and quantised (for dx), W1^T is quantised for dx; dW2
+    and dW1 are the bf16 weight-gradient GEMMs."""
+    T, H = x.shape
+    TK = gidx.numel()
+    N1, _, E = w1.shape
+    glu = is_glu(activation_type)
+    I = N1 // 2 if glu else N1
+    doutq, dout_scales = mx_quantize(dout)
+    w2tq, w2t_scales = quantize_expert_weight_transposed(w2)
+    dz = torch.empty_like(z)
+    dzq = torch.empty(TK, N1, dtype=torch.uint8, device=x.device)
+    dzq_scales = torch.empty(N1 // 128, TK, dtype=torch.int32, device=x.device)
+    y1s = torch.empty(TK, I, dtype=x.dtype, device=x.device)
+    ds = torch.empty(TK, dtype=torch.float32, device=x.device)
+    _down_projection_backward_fp8(doutq, dout_scales, w2tq, w2t_scales, z, dz, dzq, dzq_scales, y1s, ds, scores_flat,
+                                  off, gidx, sidx, E, stream_id, activation_type.value, glu)
+    del doutq, dout_scales, w2tq, w2t_scales
+    dw2 = torch.empty_like(w2)
+    _down_projection_weight_grad(dout, y1s, dw2, None, scores_flat, off, order, gidx, sidx, stream_id)
+    del y1s
+    w1tq, w1t_scales = quantize_expert_weight_transposed(w1)
+    dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
+    _down_projection_forward_fp8(dzq, dzq_scales, w1tq, w1t_scales, dx_expanded, None, off, E, stream_id)
+    del dzq, dzq_scales, w1tq, w1t_scales
+    dw1 = torch.empty_like(w1)
+    _up_projection_backward(x, w1, None, dw1, dz, None, off, order, gidx, sidx, glu, stream_id)
+    del dz
+    dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
+    _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
+    return dx, dw1, None, dw2, None, ds
 
 
 class _ExpertsFunction(torch.autograd.Function):
@@ -300,6 +353,7 @@ class _ExpertsFunction(torch.autograd.Function):
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K,
                                 activation_type, stream_id, inference, order)
         ctx.order = order
+        ctx.fp8_backward = _fp8_backward_requested(b1, b2)
         if not inference:
             ctx.save_for_backward(x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference, b1 is not None)
@@ -313,7 +367,7 @@ class _ExpertsFunction(torch.autograd.Function):
         x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off = ctx.saved_tensors
         dx, dw1, db1, dw2, db2, ds = _experts_backward(
             dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
-            stream_id, has_b1, ctx.order,
+            stream_id, has_b1, ctx.order, ctx.fp8_backward,
         )
         return dx, dw1, db1, dw2, db2, ds, None, None, None, None, None, None, None, None, None, None
 
@@ -349,8 +403,11 @@ class _TCLayerFunction(torch.autograd.Function):
         _softmax_topk_fwd(router_logits, scores, indices, E, K)
         freq, off, gidx, sidx, ridx, tok_off = _build_metadata(indices.view(-1), None, T, E, K)
         scores_flat = scores.view(-1)
+        order = _schedule_order(off)
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K, False, activation_type,
-                                stream_id, inference)
+                                stream_id, inference, order)
+        ctx.order = order
+        ctx.fp8_backward = _fp8_backward_requested(b1, b2)
         if not inference:
             ctx.save_for_backward(x, router_w, w1, w2, b2, z, scores, indices, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K, activation_type, stream_id, inference, router_logits.dtype, b1 is not None)
@@ -366,7 +423,7 @@ class _TCLayerFunction(torch.autograd.Function):
         T, E = x.size(0), router_w.size(0)
         dx, dw1, db1, dw2, db2, ds = _experts_backward(
             dout, x, w1, w2, b2, z, scores.view(-1), off, gidx, sidx, ridx, tok_off, K, False, activation_type, stream_id,
-            has_b1,
+            has_b1, ctx.order, ctx.fp8_backward,
         )
         dlogits = torch.zeros(T, E, dtype=logits_dtype, device=x.device)
         _softmax_topk_bwd(dlogits, None, ds.view(T, K), scores, indices, K)
@@ -504,6 +561,8 @@ __all__ = [
     "is_using_quack_gemm",
     "enable_fp8_forward",
     "is_using_fp8_forward",
+    "enable_fp8_backward",
+    "is_using_fp8_backward",
     "expert_schedule",
     "largest_first_schedule_order",
     "moe_TC_softmax_topk_layer",

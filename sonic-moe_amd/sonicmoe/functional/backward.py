@@ -140,6 +140,42 @@ def _down_projection_backward(
     _lib.check(rc, "_down_projection_backward")
 
 
+@torch.library.custom_op(f"{LIBRARY_NAME}::_down_projection_weight_grad", mutates_args={"dw2", "db2"})
+def _down_projection_weight_grad(
+    dout: torch.Tensor,
+    y1s: torch.Tensor,
+    dw2: torch.Tensor | None,
+    db2: torch.Tensor | None,
+    topk_scores: torch.Tensor,
+    expert_frequency_offset: torch.Tensor,
+    expert_schedule_order: torch.Tensor | None,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    stream_id: int,
+) -> None:
+    """The weight-gradient half of `_down_projection_backward` alone: dw2[e] = sum_m dout[t_m]^T y1s[m] and
+    db2[e] = sum_m s dout[t_m], from the y1s = s * act(z) an earlier call (the fp8 activation-gradient operator) left."""
+    _lib.require_device(dout, y1s, dw2, db2, topk_scores, expert_frequency_offset, expert_schedule_order, x_gather_idx,
+                        s_scatter_idx)
+    _check_bf16(("dout", dout), ("y1s", y1s), ("dw2", dw2), ("db2", db2))
+    T, H = dout.shape
+    TK, I = y1s.shape
+    E = expert_frequency_offset.numel() - 1
+    _check_schedule_order(expert_schedule_order, E)
+    dout = dout.contiguous()
+    assert y1s.is_contiguous() and topk_scores.dtype == torch.float32 and topk_scores.is_contiguous()
+    assert dw2 is None or dw2.shape == (H, I, E)
+    assert db2 is None or (db2.shape == (E, H) and db2.is_contiguous())
+    d_se, d_sr = expert_major_strides(dw2, "dw2") if dw2 is not None else (0, 0)
+    ws = _gemm_workspace(TK, E, dout.device, stream_id)
+    rc = _lib.lib().smoe_down_projection_backward(
+        _lib.ptr(dout), None, None, 0, 0, None, _lib.ptr(dw2), d_se, d_sr, _lib.ptr(db2), None, _lib.ptr(y1s), None,
+        None, _lib.ptr(topk_scores), _lib.ptr(expert_frequency_offset), _lib.ptr(expert_schedule_order),
+        _lib.ptr(x_gather_idx), _lib.ptr(s_scatter_idx), T, TK, H, I, E, 0, _lib.ptr(ws), ws.numel(), stream_id,
+    )
+    _lib.check(rc, "_down_projection_weight_grad")
+
+
 @torch.library.custom_op(f"{LIBRARY_NAME}::_token_broadcast_backward", mutates_args={"dx_reduced"})
 def _token_broadcast_backward(
     dx_reduced: torch.Tensor,

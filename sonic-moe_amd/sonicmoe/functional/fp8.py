@@ -1,9 +1,11 @@
-"""fp8 forward path: block-scaled e4m3 operands for the two forward grouped GEMMs.
+"""fp8 path: block-scaled e4m3 operands for the two forward grouped GEMMs and the two activation-gradient GEMMs.
 
 The reference has no fp8 path; this module has the shape of its `enable_quack_gemm` switch
 (sonicmoe/functional/utils.py:9-25): inside `with enable_fp8_forward():` the expert forward quantises x, W1, y1 and W2
-(one power-of-two scale per 32 contraction elements) and runs the fp8 MFMA kernels; z is still stored in bf16 and the
-backward pass is the bf16 one.
+(one power-of-two scale per 32 contraction elements) and runs the fp8 MFMA kernels; z is still stored in bf16.
+A layer called inside `with enable_fp8_backward():` computes dz (from quantised dout and W2^T) and dx (from the dz the
+dz kernel quantises in its epilogue and W1^T) in fp8 as well; the two weight-gradient GEMMs, which contract over the
+tokens, stay in bf16 and read the bf16 dz / y1s.
 """
 
 from __future__ import annotations
@@ -32,6 +34,24 @@ def enable_fp8_forward(enable: bool = True):
 
 def is_using_fp8_forward() -> bool:
     return _FP8_FORWARD
+
+
+_FP8_BACKWARD = False
+
+
+@contextmanager
+def enable_fp8_backward(enable: bool = True):
+    """Layers whose FORWARD runs inside this block compute their activation gradients (dz, dx) with fp8 operands."""
+    global _FP8_BACKWARD
+    previous, _FP8_BACKWARD = _FP8_BACKWARD, enable
+    try:
+        yield
+    finally:
+        _FP8_BACKWARD = previous
+
+
+def is_using_fp8_backward() -> bool:
+    return _FP8_BACKWARD
 
 
 @torch.library.custom_op(f"{LIBRARY_NAME}::_mx_quantize", mutates_args={"q", "scales"})
@@ -193,3 +213,106 @@ def _down_projection_forward_fp8(
         stream_id,
     )
     _lib.check(rc, "_down_projection_forward_fp8")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_mx_quantize_transposed", mutates_args={"q", "scales"})
+def _mx_quantize_transposed(src: torch.Tensor, q: torch.Tensor, scales: torch.Tensor) -> None:
+    """src (E, R, C) bf16 (last dimension contiguous) -> q (E, C, R) uint8, the transposed matrices quantised along R,
+    scales (R/128, E*C) int32."""
+    _lib.require_device(src, q, scales)
+    _check_bf16(("src", src))
+    E, R, C = src.shape
+    assert src.stride(2) == 1 and q.is_contiguous() and scales.is_contiguous()
+    assert q.dtype == torch.uint8 and q.shape == (E, C, R)
+    assert scales.dtype == torch.int32 and scales.shape == (R // 128, E * C)
+    rc = _lib.lib().smoe_mx_quantize_transposed(
+        _lib.ptr(src), src.stride(0), src.stride(1), E, R, C, _lib.ptr(q), _lib.ptr(scales),
+        _lib.current_stream_handle()
+    )
+    _lib.check(rc, "_mx_quantize_transposed")
+
+
+def quantize_expert_weight_transposed(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """w_view is the (out, in, E) permuted view of an (E, out, in) parameter; returns the (E * in, out) codes of the
+    transposed matrices, quantised along `out`, and their scale table: the weight operand of the activation-gradient
+    GEMMs, which contract over `out`.  Not cached: a training step writes the weights between two backward passes."""
+    w = w_view.permute(2, 0, 1)
+    if w.stride(2) != 1:
+        w = w.contiguous()
+    E, N, K = w.shape
+    if N % 128 or K % 64:
+        raise NotImplementedError(f"quantize_expert_weight_transposed: ({N}, {K}) matrices need out % 128 == 0 and "
+                                  f"in % 64 == 0")
+    q = torch.empty(E, K, N, dtype=torch.uint8, device=w.device)
+    scales = torch.empty(N // 128, E * K, dtype=torch.int32, device=w.device)
+    _mx_quantize_transposed(w.detach(), q, scales)
+    return q.view(E * K, N), scales
+
+
+@torch.library.custom_op(
+    f"{LIBRARY_NAME}::_down_projection_backward_fp8", mutates_args={"dz", "dzq", "dzq_scales", "y1s", "ds"}
+)
+def _down_projection_backward_fp8(
+    doutq: torch.Tensor,
+    dout_scales: torch.Tensor,
+    w2tq: torch.Tensor,
+    w2t_scales: torch.Tensor,
+    z: torch.Tensor,
+    dz: torch.Tensor,
+    dzq: torch.Tensor,
+    dzq_scales: torch.Tensor,
+    y1s: torch.Tensor,
+    ds: torch.Tensor,
+    topk_scores: torch.Tensor,
+    expert_frequency_offset: torch.Tensor,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    E: int,
+    stream_id: int,
+    activation_type: str,
+    is_glu_activation: bool,
+) -> None:
+    """The activation-gradient half of `_down_projection_backward` with fp8 operands: dy1 = gather(doutq) w2tq^T with
+    the block scales applied, then dz (bf16, and once more quantised: dzq (TK, N1) uint8 with dzq_scales (N1/128, TK)),
+    y1s = s * act(z) and ds exactly as the bf16 operator forms them.  doutq (T, H), w2tq (E*I, H)."""
+    _lib.require_device(doutq, dout_scales, w2tq, w2t_scales, z, dz, dzq, dzq_scales, y1s, ds, topk_scores,
+                        expert_frequency_offset, x_gather_idx, s_scatter_idx)
+    _check_bf16(("z", z), ("dz", dz), ("y1s", y1s))
+    T, H = doutq.shape
+    TK, N1 = z.shape
+    I = N1 // 2 if is_glu_activation else N1
+    assert w2tq.shape == (E * I, H) and dout_scales.shape == (H // 128, T) and w2t_scales.shape == (H // 128, E * I)
+    assert z.is_contiguous() and dz.is_contiguous() and dz.shape == z.shape and y1s.shape == (TK, I) and y1s.is_contiguous()
+    assert dzq.dtype == torch.uint8 and dzq.shape == (TK, N1) and dzq.is_contiguous()
+    assert dzq_scales.dtype == torch.int32 and dzq_scales.shape == (N1 // 128, TK) and dzq_scales.is_contiguous()
+    assert ds.dtype == torch.float32 and ds.numel() == TK and topk_scores.dtype == torch.float32
+    ncols = _lib.lib().smoe_dz_partial_cols(I)
+    ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
+    ws = _gemm_workspace(TK, E, z.device, stream_id)
+    rc = _lib.lib().smoe_down_projection_backward_fp8(
+        _lib.ptr(doutq),
+        _lib.ptr(dout_scales),
+        _lib.ptr(w2tq),
+        _lib.ptr(w2t_scales),
+        _lib.ptr(z),
+        _lib.ptr(dz),
+        _lib.ptr(dzq),
+        _lib.ptr(dzq_scales),
+        _lib.ptr(y1s),
+        _lib.ptr(ds),
+        _lib.ptr(ds_partial),
+        _lib.ptr(topk_scores),
+        _lib.ptr(expert_frequency_offset),
+        _lib.ptr(x_gather_idx),
+        _lib.ptr(s_scatter_idx),
+        T,
+        TK,
+        H,
+        I,
+        E,
+        ACTIVATION_CODE[ActivationType(activation_type)],
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_down_projection_backward_fp8")

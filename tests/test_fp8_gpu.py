@@ -1,6 +1,7 @@
-"""GPU tests of the fp8 forward path (block-scaled e4m3): quantiser bit-exact against the oracle, the two fp8 grouped
-GEMMs against the oracle evaluated on the same de-quantised operands (tight) and against the unquantised fp32 oracle
-within the fp8 tolerance 5e-2, and the layer with `enable_fp8_forward()`.
+"""GPU tests of the fp8 path (block-scaled e4m3): quantisers bit-exact against the oracle, the fp8 grouped GEMMs
+(up and down projection forward, dz and dx backward) against the oracle evaluated on the same de-quantised operands
+(tight) and against the unquantised fp32 oracle within the fp8 tolerance 5e-2, and the layer with
+`enable_fp8_forward()` / `enable_fp8_backward()`.
 
 Parity against the reference is unpinned for this path (the reference has no fp8 code).  Per operator the format stays
 inside 5e-2; through the whole layer (two quantised GEMMs and a gated activation in series) the relative L2 against
@@ -106,6 +107,125 @@ def test_fp8_forward_operators(dev, T, H, I, E, K, activation, with_bias, skew, 
     assert rel_l2(y2, y2_fq) < 5e-3
     y2_ref = M.down_projection_forward(y1.float().cpu(), w2, off.cpu(), b2=b2)
     assert rel_l2(y2, y2_ref) < 5e-2
+
+
+@pytest.mark.parametrize("E,R,C", [(1, 128, 64), (3, 256, 192), (8, 1024, 512), (2, 384, 4096)])
+def test_transposing_quantiser_bit_exact(dev, E, R, C):
+    """Quantising the transposes of E (R, C) matrices = the row quantiser applied to the transposed copies."""
+    from sonicmoe.functional import fp8
+
+    g = torch.Generator().manual_seed(E + R + C)
+    w = (torch.randn(E, R, C, generator=g) * torch.logspace(-3, 2, C)[None, None, :]).to(torch.bfloat16)
+    w[0, :32, 0] = 0.0
+    q, s = fp8.quantize_expert_weight_transposed(w.to(dev).permute(1, 2, 0))
+    q_ref, ex_ref = Q.mx_quantize(w.transpose(1, 2).reshape(E * C, R))
+    assert q.shape == (E * C, R) and torch.equal(s.cpu(), Q.pack_scales(ex_ref))
+    got, ref = q.cpu(), q_ref
+    zero = ((got & 0x7F) == 0) & ((ref & 0x7F) == 0)
+    assert bool(((got == ref) | zero).all())
+    # a view whose matrices are not densely packed (row stride > C)
+    wide = torch.zeros(E, R, C + 64, dtype=torch.bfloat16, device=dev)
+    wide[:, :, :C] = w.to(dev)
+    q2, s2 = fp8.quantize_expert_weight_transposed(wide[:, :, :C].permute(1, 2, 0))
+    assert torch.equal(q2, q) and torch.equal(s2, s)
+
+
+@pytest.mark.parametrize("T,H,I,E,K,activation,skew,empty", [
+    (512, 256, 128, 8, 2, "swiglu", 0.0, ()),
+    (1500, 384, 256, 8, 2, "swiglu", 0.8, (5,)),     # ragged tiles, an empty expert
+    (2048, 1024, 512, 16, 4, "geglu", 0.5, ()),
+    (1024, 512, 384, 4, 2, "gelu", 0.0, ()),         # not gated: z and dz have I columns
+    (1024, 512, 192, 4, 2, "reglu", 0.0, ()),        # I is not a multiple of 128 (N1 is)
+])
+def test_fp8_backward_operators(dev, T, H, I, E, K, activation, skew, empty):
+    """dz / y1s / ds from quantised dout and W2^T, dz quantised in the epilogue, dx from that and W1^T."""
+    from sonicmoe.functional import backward, fp8
+
+    glu, N1, w1, w2, _, _, x, md, meta = _problem(dev, T, H, I, E, K, 3 * T + H, activation, skew, empty)
+    TK = T * K
+    off, gidx, sidx = md["expert_frequency_offset"], md["x_gather_idx"], md["s_scatter_idx"]
+    stream = torch.cuda.current_stream().cuda_stream
+    bf = dict(dtype=torch.bfloat16, device=dev)
+    g = torch.Generator().manual_seed(T)
+    dout = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    scores = torch.rand(TK, generator=g) + 0.05
+    z, _ = M.up_projection_forward(x, w1, off.cpu(), gidx.cpu(), activation=activation)
+    z = z.to(torch.bfloat16)
+
+    doutq, douts = fp8.mx_quantize(dout.to(dev))
+    w2tq, w2ts = fp8.quantize_expert_weight_transposed(w2.to(dev).permute(1, 2, 0))
+    dz = torch.full((TK, N1), 7.0, **bf)
+    dzq = torch.zeros(TK, N1, dtype=torch.uint8, device=dev)
+    dzs = torch.zeros(N1 // 128, TK, dtype=torch.int32, device=dev)
+    y1s = torch.full((TK, I), 7.0, **bf)
+    ds = torch.full((TK,), 7.0, dtype=torch.float32, device=dev)
+    fp8._down_projection_backward_fp8(doutq, douts, w2tq, w2ts, z.to(dev), dz, dzq, dzs, y1s, ds, scores.to(dev), off,
+                                      gidx, sidx, E, stream, activation, glu)
+    dz_fq, y1s_fq, ds_fq = Q.down_projection_backward_fp8(dout, z, w2, scores, off, gidx, sidx, activation)
+    assert rel_l2(dz, dz_fq) < 5e-3      # same operands, fp32 accumulation: what is left is the bf16 rounding
+    assert rel_l2(y1s, y1s_fq) < 5e-3
+    assert rel_l2(ds, ds_fq) < 2e-3
+    dz_ref, y1s_ref, ds_ref, dw2_ref = M.down_projection_backward(dout, z, w2, scores, off.cpu(), gidx.cpu(), sidx.cpu(),
+                                                                  activation=activation)
+    assert rel_l2(dz, dz_ref) < 5e-2     # one quantised GEMM against the unquantised one: the fp8 tolerance
+    assert rel_l2(ds, ds_ref) < 5e-2
+    assert rel_l2(y1s, y1s_ref) < 5e-3   # y1s does not depend on the quantised GEMM
+
+    # dz quantised in the epilogue == the row quantiser applied to the stored bf16 dz, bit for bit
+    q_ref, s_ref = fp8.mx_quantize(dz)
+    zero = ((dzq & 0x7F) == 0) & ((q_ref & 0x7F) == 0)
+    assert bool(((dzq == q_ref) | zero).all()) and torch.equal(dzs, s_ref)
+
+    # the weight-gradient half from the stored y1s (bf16 GEMM)
+    dw2 = torch.full((E, H, I), 3.0, **bf).permute(1, 2, 0)
+    backward._down_projection_weight_grad(dout.to(dev), y1s, dw2, None, scores.to(dev), off, None, gidx, sidx, stream)
+    assert rel_l2(dw2.permute(2, 0, 1), dw2_ref) < 1e-2
+
+    # dx from the quantised dz and the transposed quantised W1: the down-projection forward kernel
+    w1tq, w1ts = fp8.quantize_expert_weight_transposed(w1.to(dev).permute(1, 2, 0))
+    dxe = torch.full((TK, H), 7.0, **bf)
+    fp8._down_projection_forward_fp8(dzq, dzs, w1tq, w1ts, dxe, None, off, E, stream)
+    dxe_fq = Q.dx_fp8(dz.float().cpu(), w1, off.cpu())
+    assert rel_l2(dxe, dxe_fq) < 5e-3
+    _, dxe_ref = M.up_projection_backward(x, w1, dz.float().cpu(), off.cpu(), gidx.cpu())
+    assert rel_l2(dxe, dxe_ref) < 5e-2
+
+
+def test_layer_with_fp8_forward_and_backward(dev):
+    """fp8 forward and fp8 activation gradients against the bf16 path of the same module; the weight gradients are
+    bf16 GEMMs on operands that went through fp8 GEMMs."""
+    from sonicmoe import MoE, enable_fp8_backward, enable_fp8_forward
+    from sonicmoe.enums import ActivationType
+
+    T, H, I, E, K = 2048, 1024, 512, 16, 4
+    torch.manual_seed(3)
+    moe = MoE(E, K, H, I, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+    x = torch.randn(T, H, device=dev).to(torch.bfloat16).requires_grad_()
+    dy = torch.randn(T, H, device=dev).to(torch.bfloat16)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_proj.weight]
+    out, _ = moe(x)
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+    with enable_fp8_backward():
+        out_b, _ = moe(x)                      # bf16 forward, fp8 activation gradients
+    grads_b = torch.autograd.grad(out_b, [x] + params, grad_outputs=dy)   # the switch is read when the forward runs
+    assert torch.equal(out_b, out)
+    errs_b = [rel_l2(a, b) for a, b in zip(grads_b, grads)]
+    with enable_fp8_forward(), enable_fp8_backward():
+        out8, _ = moe(x)
+        grads8 = torch.autograd.grad(out8, [x] + params, grad_outputs=dy)
+    errs8 = [rel_l2(a, b) for a, b in zip(grads8, grads)]
+    print("fp8 backward only: dx, dWr, dW1, dW2 rel-L2 vs bf16:", errs_b, "fp8 forward+backward:", errs8)
+    assert errs_b[3] < 1e-2          # dW2 = dout^T y1s: no quantised GEMM in its path
+    # dWr (through ds) and dW1 (through dz) have ONE quantised GEMM on their way: inside the fp8 tolerance 5e-2
+    assert errs_b[1] < 5e-2 and errs_b[2] < 5e-2, errs_b
+    # dx has two in series (dz, then dx from the quantised dz): measured 5.2e-2, just outside 5e-2 -- recorded bound
+    assert 1e-2 < errs_b[0] < 7e-2, errs_b
+    # fp8 forward and backward in series (three quantised GEMMs on the way to dx): measured 5.4e-2 .. 6.7e-2, outside
+    # the 5e-2 stated for fp8 -- recorded bound, like the forward-only layer test below
+    assert all(e < 9e-2 for e in errs8), errs8
+    moe_b = MoE(E, K, H, I, ActivationType.SWIGLU, True, 0.02).to(device=dev, dtype=torch.bfloat16)
+    with enable_fp8_backward(), pytest.raises(NotImplementedError, match="biases"):
+        moe_b(x)
 
 
 def test_layer_with_fp8_forward(dev):
