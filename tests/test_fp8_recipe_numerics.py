@@ -44,3 +44,38 @@ def test_e4m3_block_scaled_recipe_error_levels():
     d0 = dout @ w2
     d1 = _qdq(dout) @ _qdq(w2, dim=0)
     assert 0.02 < _rel(d1, d0) < 0.05
+
+
+def test_power_of_two_scales_per_32_against_fp32_scales_per_128():
+    """Config 5 of the benchmark list words its recipe as "per-128-element block scales (amax/448)"; the kernels use the
+    format the fp8 matrix instruction multiplies natively instead: one power-of-two scale per 32 elements.  Same
+    problem, both recipes, against the fp32 evaluation.  An fp32 scale amax/448 puts each block's largest element
+    exactly on the top code, so the elements that carry most of the norm round a little better than under a
+    power-of-two scale, which leaves the data's own mantissas in place; the smaller block does not make up for that.
+    Measured: the built format is 3 .. 10 % less accurate in relative L2 at every stage, in the same regime (one
+    quantised GEMM ~3.5e-2).  The bounds below pin that difference."""
+    from oracle import fp8 as Q
+
+    torch.manual_seed(1)
+    T, H, I = 512, 1024, 256
+    x, dout = torch.randn(T, H), torch.randn(T, H)
+    x[:, ::7] *= 30.0  # outlier channels
+    w1, w2 = torch.randn(2 * I, H) * 0.02, torch.randn(H, I) * 0.02
+
+    def mx(t, dim=-1):
+        t2 = t.transpose(dim, -1).contiguous()
+        return Q.fake_quant(t2).transpose(dim, -1)
+
+    def run(Qf):
+        z = Qf(x) @ Qf(w1).t()
+        y1 = torch.nn.functional.silu(z[:, 0::2]) * z[:, 1::2]
+        out = Qf(y1) @ Qf(w2).t()
+        dy1 = Qf(dout) @ Qf(w2, dim=0)
+        return z, y1, out, dy1
+
+    ref = run(lambda t, dim=-1: t)
+    per128 = [_rel(a, b) for a, b in zip(run(_qdq), ref)]
+    per32 = [_rel(a, b) for a, b in zip(run(mx), ref)]
+    for name, e32, e128 in zip(("z", "y1", "out", "dy1"), per32, per128):
+        assert 0.95 * e128 < e32 < 1.15 * e128, (name, e32, e128)
+    assert per32[0] < 5e-2 and per128[0] < 5e-2 and per32[3] < 5e-2 and per128[3] < 5e-2  # one quantised GEMM
