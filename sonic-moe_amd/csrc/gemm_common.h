@@ -57,11 +57,17 @@ SMOE_DEV void buffer_load16_to_lds(i32x4 rsrc, uint32_t voff, uint32_t soff, uin
                : "memory");
 }
 
-// piece swizzle of a K-major stage with BK_ of the contraction per row (BK_*2/16 pieces): chosen so that the 16 lanes
-// of a ds_read_b128 quarter-wave (16 consecutive rows, same piece) hit 16 different 16-byte bank groups
-template <int BK_>
+// Piece swizzle of a K-major stage with BK_ of the contraction per row (BK_*2/16 pieces).  The LDS has 64 banks and
+// serves a ds_read_b128 16 lanes at a time, in the groups {0-3, 12-15, 20-23, 24-27}, {4-7, 8-11, 16-19, 28-31} and the
+// same of the upper half-wave: the 16 pieces of a group have to fall into the 16 different 16-byte bank groups (row
+// parity, piece).  With 32-row fragments (FR_ = 32: lane l reads row l % 32) a group holds 16 rows of one piece; with
+// 16-row fragments (FR_ = 16: row l % 16, piece c + l / 16) it holds rows 0-3 and 12-15 of piece c and rows 4-11 of
+// piece c ^ 1, which the first swizzle sends to the same banks twice (SQ_LDS_BANK_CONFLICT equal to half of
+// SQ_LDS_IDX_ACTIVE); the second one is row / 2 with the low bit flipped for the rows 4-11.
+template <int BK_, int FR_ = 32>
 SMOE_DEV int kswz(int row) {
   if constexpr (BK_ == 32) return (row >> 2) & 3;
+  else if constexpr (FR_ == 16) return ((row >> 1) & 7) ^ (((row >> 2) ^ (row >> 3)) & 1);
   else return (row & 7) ^ ((row >> 3) & 1);
 }
 

@@ -79,13 +79,13 @@ SMOE_DEV void fragment_offsets(int wm, int wn, int lane, int (&p_off)[C::KSL], i
   constexpr int FR = C::FR, PPS = C::Mma::KSTEP / 8;  // 16-byte pieces per row and k-slice
   {
     const int row = wm * C::TM + (lane & (FR - 1));
-    const int sw = kswz<C::BK>(row);
+    const int sw = kswz<C::BK, C::FR>(row);
 #pragma unroll
     for (int ks = 0; ks < C::KSL; ks++) p_off[ks] = row * C::KROW + (((PPS * ks + lane / FR) ^ sw) << 4);
   }
   if constexpr (!C::QMN) {
     const int row = wn * C::TN + (lane & (FR - 1));
-    const int sw = kswz<C::BK>(row);
+    const int sw = kswz<C::BK, C::FR>(row);
 #pragma unroll
     for (int ks = 0; ks < C::KSL; ks++) q_off[ks] = row * C::KROW + (((PPS * ks + lane / FR) ^ sw) << 4);
   } else {
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     int m = row0 + r;
     m = m < row_end ? m : row_end - 1;
     const int64_t src_row = p.gidx ? (int64_t)p.gidx[m] : (int64_t)m;
-    p_src[i] = p.P + src_row * p.p_stride + (((lane % C::KPR) ^ kswz<BK>(r)) << 3);
+    p_src[i] = p.P + src_row * p.p_stride + (((lane % C::KPR) ^ kswz<BK, C::FR>(r)) << 3);
   }
   const uint16_t* q_src[C::Q_INSTR];
   const uint16_t* qe = p.Q + (int64_t)e * p.q_stride_e;
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
       const int r = (wave * C::Q_INSTR + i) * C::KRPI + lane / C::KPR;
       int n = n0 + r;
       n = n < p.N ? n : p.N - 1;
-      q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane % C::KPR) ^ kswz<BK>(r)) << 3);
+      q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane % C::KPR) ^ kswz<BK, C::FR>(r)) << 3);
     }
     q_step = BK;
   } else {
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
 #pragma unroll
     for (int i = 0; i < C::P_INSTR; i++) {
       const int r = (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
-      p_voff[i] = (uint32_t)rows[i] * p_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK>(r)) << 4);
+      p_voff[i] = (uint32_t)rows[i] * p_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK, C::FR>(r)) << 4);
     }
   };
   auto point_q = [&](const Tile& t) {
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
         const int r = (wave * C::Q_INSTR + i) * C::KRPI + ln / C::KPR;
         int n = t.n0 + r;
         n = n < p.N ? n : p.N - 1;
-        q_voff[i] = (uint32_t)n * q_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK>(r)) << 4);
+        q_voff[i] = (uint32_t)n * q_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK, C::FR>(r)) << 4);
       } else {
         const int kl = (wave * C::Q_INSTR + i) * C::RPI + ln / C::LPR;
         const int phys16 = ln % C::LPR;
