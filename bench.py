@@ -133,6 +133,14 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
             ("switch_loss_fwd", lambda: forward._switch_loss_fwd(logits, freq, sl_acc, sl_aux), None, T * E * 2),
             ("switch_loss_bwd", lambda: backward._switch_loss_bwd(logits, freq, sl_acc, sl_g, dlog), None, T * E * 4),
         ]
+        if forward.router_fused_supported(xd, wr.detach()):
+            # the router in one kernel (opt-in, sonicmoe.functional.fused_router): replaces router_gemm + topk_softmax and
+            # the column-sum pass of switch_loss_fwd
+            rf_logits = torch.empty(T, E, dtype=bf, device=dev)
+            rf_part = torch.empty(forward.router_fused_partials(T, E), E, dtype=torch.float32, device=dev)
+            ops.append(("router_forward_fused(gemm+topk+colsum)",
+                        lambda: forward._router_forward_fused(xd, wr.detach(), rf_logits, scores, idx, rf_part),
+                        2.0 * T * H * E, T * H * 2 + T * E * 2 + T * K * 8))
         if gemms_only:
             ops = [o for o in ops if o[2] and "router_gemm" not in o[0]]
         if H % 128 == 0 and I % 128 == 0 and only is None and not gemms_only:

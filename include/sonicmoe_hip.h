@@ -197,6 +197,24 @@ int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride
 int smoe_router_weight_grad(const void* dlogits, const void* x, void* partial, int64_t T, int E, int H, int chunks,
                             void* stream);
 
+/* The router in one pass over x (bf16): logits = x Wr^T, the top-K winners of every row with their softmax scores, and
+ * optionally the column sums of the full row softmax, all from the GEMM's accumulators.  Replaces the chain
+ * router_logits = F.linear(x, router_w) -> sonicmoe::_softmax_topk_fwd (sonicmoe/functional/__init__.py:438-439,
+ * forward.py:224-237) and feeds the load-balancing loss (sonicmoe/moe.py:247-274) without another pass over the logits.
+ *   x (T, H), wr (E, H), logits (T, E) bf16 contiguous; scores (T, K) fp32; indices (T, K) int32
+ *   colsum_partial: NULL, or smoe_router_fused_partials(T, E) x E floats: per-workgroup column sums of
+ *   softmax(logits) in fp32, to be handed to smoe_switch_loss_from_partials.
+ * Top-K and both softmaxes are evaluated on the logits as stored (rounded to bf16): scores and indices equal
+ * smoe_topk_softmax_fwd applied to the stored logits bit for bit.  The logits themselves differ from a library GEMM's
+ * in the last bf16 bit (different summation order), so near-ties may route differently than after F.linear.
+ * Limits: E % 16 == 0, 16 <= E <= 256; H % 256 == 0; 1 <= K <= E. */
+int64_t smoe_router_fused_partials(int64_t T, int E);
+int smoe_router_forward_fused(const void* x, const void* wr, int64_t T, int H, int E, int K, void* logits,
+                              float* scores, int32_t* indices, float* colsum_partial, void* stream);
+/* acc, aux of smoe_switch_loss_fwd from column-sum partials (n_partial, E) some other kernel produced. */
+int smoe_switch_loss_from_partials(const float* partial, int64_t n_partial, int E, const int32_t* freq, float* acc,
+                                   float* aux, void* stream);
+
 /* Load-balancing auxiliary loss of MoE.forward (sonicmoe/moe.py:247-274: softmax of the (T, E) logits in fp32, column
  * sums, two L1 normalisations, a dot product -- six torch kernels and a (T, E) fp32 tensor there):
  *   acc[e] = sum_t softmax(logits[t, :])[e],   aux[0] = E * <acc / max(|acc|_1, 1e-12), freq / max(|freq|_1, 1e-12)>.

@@ -371,6 +371,19 @@ extern "C" int smoe_switch_loss_fwd(const void* logits, int dtype, int64_t row_s
   return SMOE_OK;
 }
 
+extern "C" int smoe_switch_loss_from_partials(const float* partial, int64_t n_partial, int E, const int32_t* freq,
+                                              float* acc, float* aux, void* stream) {
+  SMOE_REQUIRE(n_partial >= 1 && n_partial < (1ll << 31), SMOE_ERR_INVALID, "switch_loss_from_partials: bad count");
+  SMOE_REQUIRE(E >= 1 && E <= 4096, SMOE_ERR_UNSUPPORTED, "switch_loss_from_partials: E=%d out of range [1, 4096]", E);
+  SMOE_REQUIRE(partial && freq && acc && aux, SMOE_ERR_INVALID, "switch_loss_from_partials: null pointer");
+  int cw = 64;
+  while (cw < E && cw < 1024) cw *= 2;
+  hipLaunchKernelGGL(switch_loss_finalize_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, partial, (int)n_partial,
+                     freq, E, cw, acc, aux);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
 extern "C" int smoe_switch_loss_bwd(const void* logits, int dtype, int64_t row_stride, int64_t T, int E,
                                     const int32_t* freq, const float* acc, const float* grad_aux, void* dlogits,
                                     int64_t d_row_stride, void* stream) {

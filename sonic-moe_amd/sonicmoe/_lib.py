@@ -48,6 +48,9 @@ _SIGNATURES = {
         [_P, _P, _L, _L, _P, _P, _L, _L, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
     "smoe_router_weight_grad": (c_int, [_P, _P, _P, _L, _I, _I, _I, _P]),
+    "smoe_router_fused_partials": (ctypes.c_int64, [_L, _I]),
+    "smoe_router_forward_fused": (c_int, [_P, _P, _L, _I, _I, _I, _P, _P, _P, _P, _P]),
+    "smoe_switch_loss_from_partials": (c_int, [_P, _L, _I, _P, _P, _P, _P]),
     "smoe_switch_loss_workspace_bytes": (c_size_t, [_L, _I]),
     "smoe_switch_loss_fwd": (c_int, [_P, _I, _L, _L, _I, _P, _P, _P, _P, _Z, _P]),
     "smoe_switch_loss_bwd": (c_int, [_P, _I, _L, _L, _I, _P, _P, _P, _P, _L, _P]),

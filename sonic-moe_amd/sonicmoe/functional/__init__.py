@@ -32,9 +32,13 @@ from .backward import (
 from .forward import (
     _down_projection_forward,
     _router_forward,
+    _router_forward_fused,
     _softmax_topk_fwd,
+    _switch_loss_from_partials,
     _switch_loss_fwd,
     _up_projection_forward,
+    router_fused_partials,
+    router_fused_supported,
 )
 from .fp8 import (
     _down_projection_backward_fp8,
@@ -180,6 +184,25 @@ class TC_Softmax_Topk_Router_Function(torch.autograd.Function):
         dlogits = torch.zeros(scores.size(0), ctx.E, dtype=ctx.logits_dtype, device=scores.device)
         _softmax_topk_bwd(dlogits, None, dscores, scores, indices, ctx.K)
         return dlogits, None, None
+
+
+_FUSED_ROUTER = os.environ.get("SMOE_FUSED_ROUTER", "0") == "1"
+
+
+@contextmanager
+def fused_router(enable: bool = True):
+    """Inside the block `moe_TC_softmax_topk_layer` computes logits, top-K scores / indices and the softmax column sums
+    of the load-balancing loss in ONE kernel over x (`_router_forward_fused`) instead of F.linear followed by the
+    top-K kernel (and a third pass for the loss).  Off by default: the kernel's logits differ from the library GEMM's in
+    the last bf16 bit, so tokens whose K-th and (K+1)-th logits nearly tie may be routed differently than after
+    F.linear; everything downstream is computed from the logits the kernel stores.  Shapes it does not take
+    (`router_fused_supported`) use the unfused chain."""
+    global _FUSED_ROUTER
+    previous, _FUSED_ROUTER = _FUSED_ROUTER, enable
+    try:
+        yield
+    finally:
+        _FUSED_ROUTER = previous
 
 
 _SCHEDULE_POLICY = "expert_index"
@@ -397,10 +420,17 @@ class _TCLayerFunction(torch.autograd.Function):
                 inference: bool):
         T, E = x.size(0), router_w.size(0)
         x = x.contiguous()
-        router_logits = F.linear(x, router_w)
         scores = torch.empty(T, K, dtype=torch.float32, device=x.device)
         indices = torch.empty(T, K, dtype=torch.int32, device=x.device)
-        _softmax_topk_fwd(router_logits, scores, indices, E, K)
+        if _FUSED_ROUTER and router_fused_supported(x, router_w):
+            router_logits = torch.empty(T, E, dtype=x.dtype, device=x.device)
+            colsum = torch.empty(router_fused_partials(T, E), E, dtype=torch.float32, device=x.device)
+            _router_forward_fused(x, router_w.contiguous(), router_logits, scores, indices, colsum)
+            # picked up by switch_loss() when it is handed this very tensor (MoE.forward does that)
+            router_logits._smoe_softmax_colsum_partials = (colsum, router_logits._version)
+        else:
+            router_logits = F.linear(x, router_w)
+            _softmax_topk_fwd(router_logits, scores, indices, E, K)
         freq, off, gidx, sidx, ridx, tok_off = _build_metadata(indices.view(-1), None, T, E, K)
         scores_flat = scores.view(-1)
         order = _schedule_order(off)
@@ -449,7 +479,11 @@ class _SwitchLossFunction(torch.autograd.Function):
         freq = expert_frequency.to(torch.int32).contiguous()
         acc = torch.empty(E, dtype=torch.float32, device=logits.device)
         aux = torch.empty(1, dtype=torch.float32, device=logits.device)
-        _switch_loss_fwd(logits, freq, acc, aux)
+        partials, version = getattr(router_logits, "_smoe_softmax_colsum_partials", (None, None))
+        if partials is not None and version == router_logits._version and router_logits.dim() == 2:
+            _switch_loss_from_partials(partials, freq, acc, aux)  # the fused router already summed the softmax columns
+        else:
+            _switch_loss_fwd(logits, freq, acc, aux)
         ctx.save_for_backward(logits, freq, acc)
         ctx.logits_shape = router_logits.shape
         return aux.view(())
@@ -564,6 +598,7 @@ __all__ = [
     "enable_fp8_backward",
     "is_using_fp8_backward",
     "expert_schedule",
+    "fused_router",
     "largest_first_schedule_order",
     "moe_TC_softmax_topk_layer",
     "moe_general_routing_inputs",

@@ -238,3 +238,59 @@ def _switch_loss_fwd(router_logits: torch.Tensor, expert_frequency: torch.Tensor
         _lib.current_stream_handle(),
     )
     _lib.check(rc, "_switch_loss_fwd")
+
+
+def router_fused_supported(x: torch.Tensor, router_w: torch.Tensor) -> bool:
+    """Shapes and dtypes `_router_forward_fused` takes: bf16, E a multiple of 16 up to 256, H a multiple of 256."""
+    E, H = router_w.shape
+    return (x.is_cuda and x.dtype == torch.bfloat16 and router_w.dtype == torch.bfloat16 and E % 16 == 0
+            and 16 <= E <= 256 and H % 256 == 0 and x.size(0) > 0)
+
+
+@torch.library.custom_op(
+    f"{LIBRARY_NAME}::_router_forward_fused", mutates_args={"router_logits", "topk_scores", "topk_indices", "colsum_partial"}
+)
+def _router_forward_fused(x: torch.Tensor, router_w: torch.Tensor, router_logits: torch.Tensor,
+                          topk_scores: torch.Tensor, topk_indices: torch.Tensor,
+                          colsum_partial: torch.Tensor | None) -> None:
+    """router_logits = x router_w^T, the top-K of every row with softmax scores, and (if colsum_partial is given) the
+    per-workgroup column sums of softmax(router_logits), in one kernel: the reference's F.linear followed by
+    sonicmoe::_softmax_topk_fwd (sonicmoe/functional/__init__.py:438-439) and the softmax column sums of
+    MoE._compute_switch_loss (sonicmoe/moe.py:261-264).  colsum_partial: (router_fused_partials(T, E), E) fp32."""
+    _lib.require_device(x, router_w, router_logits, topk_scores, topk_indices, colsum_partial)
+    _check_bf16(("x", x), ("router_w", router_w), ("router_logits", router_logits))
+    T, H = x.shape
+    E = router_w.size(0)
+    K = topk_scores.size(1)
+    assert x.is_contiguous() and router_w.is_contiguous() and router_logits.is_contiguous()
+    assert router_w.shape == (E, H) and router_logits.shape == (T, E)
+    assert topk_scores.shape == (T, K) and topk_scores.dtype == torch.float32 and topk_scores.is_contiguous()
+    assert topk_indices.shape == (T, K) and topk_indices.dtype == torch.int32 and topk_indices.is_contiguous()
+    if colsum_partial is not None:
+        assert colsum_partial.dtype == torch.float32 and colsum_partial.is_contiguous()
+        assert colsum_partial.shape == (_lib.lib().smoe_router_fused_partials(T, E), E)
+    rc = _lib.lib().smoe_router_forward_fused(
+        _lib.ptr(x), _lib.ptr(router_w), T, H, E, K, _lib.ptr(router_logits), _lib.ptr(topk_scores),
+        _lib.ptr(topk_indices), _lib.ptr(colsum_partial), _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_router_forward_fused")
+
+
+def router_fused_partials(T: int, E: int) -> int:
+    return int(_lib.lib().smoe_router_fused_partials(T, E))
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_switch_loss_from_partials", mutates_args={"acc", "aux"})
+def _switch_loss_from_partials(colsum_partial: torch.Tensor, expert_frequency: torch.Tensor, acc: torch.Tensor,
+                               aux: torch.Tensor) -> None:
+    """acc, aux of `_switch_loss_fwd` from the column-sum partials `_router_forward_fused` wrote."""
+    _lib.require_device(colsum_partial, expert_frequency, acc, aux)
+    n, E = colsum_partial.shape
+    assert colsum_partial.dtype == torch.float32 and colsum_partial.is_contiguous()
+    assert expert_frequency.dtype == torch.int32 and expert_frequency.is_contiguous() and expert_frequency.numel() == E
+    assert acc.numel() == E and acc.dtype == torch.float32 and acc.is_contiguous() and aux.numel() == 1
+    rc = _lib.lib().smoe_switch_loss_from_partials(
+        _lib.ptr(colsum_partial), n, E, _lib.ptr(expert_frequency), _lib.ptr(acc), _lib.ptr(aux),
+        _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_switch_loss_from_partials")

@@ -253,6 +253,31 @@ def test_layer_with_fp8_forward(dev):
         assert rel_l2(a, b) < 8e-2  # bf16 backward from the fp8-forward z
 
 
+@pytest.mark.xfail(strict=False, reason="chains of two or three e4m3 GEMMs exceed the 5e-2 stated for fp8 (measured: forward output "
+                   "6.6e-2, dx 6.7e-2, dWr 6.6e-2, dW1 5.5e-2, dW2 5.4e-2); the format's rounding, not the kernels: a CPU "
+                   "simulation of the recipe lands there too (tests/test_fp8_recipe_numerics.py)")
+def test_fp8_layer_within_the_stated_tolerance(dev):
+    """The bound the fp8 variant is asked to meet, end to end through the layer: 5e-2 against the bf16 path.  Met per
+    quantised GEMM (the operator tests above), not through the chain; kept here as an expected failure so that the
+    bound stays visible instead of being widened."""
+    from sonicmoe import MoE, enable_fp8_backward, enable_fp8_forward
+    from sonicmoe.enums import ActivationType
+
+    T, H, I, E, K = 2048, 1024, 512, 16, 4
+    torch.manual_seed(3)
+    moe = MoE(E, K, H, I, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+    x = torch.randn(T, H, device=dev).to(torch.bfloat16).requires_grad_()
+    dy = torch.randn(T, H, device=dev).to(torch.bfloat16)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_proj.weight]
+    out, _ = moe(x)
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+    with enable_fp8_forward(), enable_fp8_backward():
+        out8, _ = moe(x)
+        grads8 = torch.autograd.grad(out8, [x] + params, grad_outputs=dy)
+    errs = [rel_l2(out8, out)] + [rel_l2(a, b) for a, b in zip(grads8, grads)]
+    assert all(e < 5e-2 for e in errs), errs
+
+
 def test_quantised_weight_cache_follows_parameter_updates(dev):
     """The cached quantised weights are dropped when the parameter is written to (optimizer step)."""
     from sonicmoe import MoE, enable_fp8_forward
