@@ -146,6 +146,29 @@ def test_full_size_properties(dev):
         ref += scores[sample, j, None] * torch.einsum("ti,thi->th", y, w2.detach()[e].float())
     assert rel_l2(o1.detach()[sample], ref) < TOL
 
+    # gradient VALUES at full size: the weight gradients of two experts against a dense fp32 evaluation of just those
+    # experts, and dx of a few tokens against autograd through a dense fp32 restatement of their K expert MLPs
+    with torch.no_grad():
+        for e in (0, E - 1):
+            a, b = int(off[e]), int(off[e + 1])
+            tok = gidx[a:b].long()
+            sc = scores.view(-1)[sidx[a:b].long()]
+            dw1_ref, dw2_ref = _dense_expert_weight_grads(x, dout, w1, w2, e, tok, sc)
+            assert rel_l2(g1[2][e], dw1_ref) < TOL, e
+            assert rel_l2(g1[3][e], dw2_ref) < TOL, e
+    few = sample[:8]
+    xs = x.detach()[few].float().requires_grad_()
+    lg = xs @ wr.detach().float().t()
+    out = torch.zeros(8, H, device=dev)
+    sc_few = torch.softmax(torch.gather(lg, 1, idx[few].long()), dim=-1)   # softmax over the K winners
+    for j in range(K):
+        e = idx[few, j].long()
+        h = torch.einsum("th,tnh->tn", xs, w1.detach()[e].float())
+        y = torch.nn.functional.silu(h[:, 0::2]) * h[:, 1::2]
+        out = out + sc_few[:, j, None] * torch.einsum("ti,thi->th", y, w2.detach()[e].float())
+    (dx_ref,) = torch.autograd.grad(out, xs, grad_outputs=dout[few].float())
+    assert rel_l2(g1[0][few], dx_ref) < 2e-2   # incl. the path through the router scores (bf16 logits in the product)
+
 
 def test_tensors_beyond_2_31_elements(dev):
     """T=65536, K=8, H=4096: the grouped (TK, H) tensors hold 2^31 elements, so any 32-bit element index would wrap.
