@@ -761,11 +761,11 @@ struct DzEpilogueArgs {
   int64_t dzq_rows;
 };
 
-template <int TN, int ACT>
+template <int TN, int ACT, int BR = 32>
 struct DzStaging {
   static constexpr int ZW = act_is_glu(ACT) ? 2 : 1;
   static constexpr int ZB = TN * 2 * ZW, YB = TN * 2;  // bytes per staged z / dz row, y1s row
-  static constexpr int BYTES = 32 * (ZB + YB);         // per wavefront
+  static constexpr int BYTES = BR * (ZB + YB);         // per wavefront: BR token rows are staged at a time
 };
 
 // e8m0 exponent of the smallest power of two s with amax / s <= 448 (the largest e4m3 value): no element saturates
@@ -781,7 +781,7 @@ SMOE_DEV int mx_scale_exponent(float amax) {
   return k < 0 ? 0 : (k > 254 ? 254 : k);
 }
 
-template <class Mma, int TM, int TN, int ACT, int PF = 2, bool QUANT = false, class RingIdle>
+template <class Mma, int TM, int TN, int ACT, int PF = 2, bool QUANT = false, int BR = 32, class RingIdle>
 SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* zbuf, int lane,
                           const DzEpilogueArgs& a, RingIdle&& ring_idle) {
   using AL = AccLayout<Mma>;
@@ -789,12 +789,13 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
   constexpr int PW = act_pointwise(ACT);
   constexpr int FR = Mma::FR, FN = TN / FR, QPF = AL::QPF;
   constexpr int ZW = DzStaging<TN, ACT>::ZW, ZB = DzStaging<TN, ACT>::ZB, YB = DzStaging<TN, ACT>::YB;
-  constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = 32 / ZR;  // lanes per row, rows per instruction, instructions
-  constexpr int YL = YB / 16, YR = 64 / YL, YN = 32 / YR;
+  constexpr int ZL = ZB / 16, ZR = 64 / ZL, ZN = BR / ZR;  // lanes per row, rows per instruction, instructions
+  constexpr int YL = YB / 16, YR = 64 / YL, YN = BR / YR;
   constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;  // row swizzle of the staged z chunks
-  constexpr int NB = TM / 32, RB = 32 / FR;   // 32-row batches; fragment rows per batch
+  constexpr int NB = TM / BR, RB = BR / FR;   // batches of BR rows; fragment rows per batch
+  static_assert(BR % FR == 0 && ZN >= 1 && YN >= 1, "a batch is whole fragment rows and whole load instructions");
   static_assert(PF == 1 || PF == 2, "one or two batches of z are prefetched");
-  char* ybuf = zbuf + 32 * ZB;
+  char* ybuf = zbuf + BR * ZB;
   const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
   const int zlimit = ZW * a.N;
   const int zcol = ZW * a.n_base + zc * 8;  // first z column of this lane's 16-byte chunk
@@ -803,7 +804,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
   auto fetch_z = [&](int blk, u32x4(&dst)[ZN]) {
 #pragma unroll
     for (int it = 0; it < ZN; it++) {
-      int m = a.m_base + blk * 32 + it * ZR + zr;
+      int m = a.m_base + blk * BR + it * ZR + zr;
       m = m < a.row_end ? m : a.row_end - 1;
       dst[it] = *(const u32x4*)(a.zin + (int64_t)m * a.zin_stride + zcol_c);
     }
@@ -822,7 +823,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
     static_for<RB>([&](auto sub_c) {
       constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
       const int mrow = sub * FR + AL::row(lane);  // row inside the staged batch
-      const int m = a.m_base + blk * 32 + mrow;
+      const int m = a.m_base + blk * BR + mrow;
       const bool mvalid = m < a.row_end;
       float sc = 0.f, dsum = 0.f;
       if (mvalid) sc = a.scores[a.sidx[m]];
@@ -875,7 +876,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
     for (int it = 0; it < ZN; it++) {
       const int r = it * ZR + zr;
       const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4));
-      const int mm = a.m_base + blk * 32 + r;
+      const int mm = a.m_base + blk * BR + r;
       const bool live = mm < a.row_end && zcol < zlimit;
       if (live) *(u32x4*)(a.dz + (int64_t)mm * a.dz_stride + zcol) = v;
       if constexpr (QUANT) {
@@ -907,7 +908,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
     for (int it = 0; it < YN; it++) {
       const int r = it * YR + yr;
       const u32x4 v = *(const u32x4*)(ybuf + r * YB + ((yc ^ ((r >> 1) & (YL < 8 ? YL - 1 : 7))) << 4));
-      const int mm = a.m_base + blk * 32 + r, col = a.n_base + yc * 8;
+      const int mm = a.m_base + blk * BR + r, col = a.n_base + yc * 8;
       if (mm < a.row_end && col < a.N) *(u32x4*)(a.y1s + (int64_t)mm * a.y1s_stride + col) = v;
     }
   });
@@ -920,6 +921,7 @@ struct Tuning {
   int gemm_stream;          // 1 (default): up-projection forward, down-projection forward and dx run as tile streams
   int gemm_stream_grid;     // workgroups of the tile-stream kernels; 0 (default) = one per compute unit
   int varlen_k_tile_order;  // 2 blocked (default), 0 single tiles round-robin over the XCDs, 1 whole experts per XCD
+  int dz_stream;            // 1: dz runs as a tile stream too (with gemm_stream); 0: one tile per workgroup
 };
 const Tuning& tuning();
 

@@ -269,7 +269,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
 // the ring running across tile boundaries (gemm_stream_loop).  ROLE_UP_FWD and ROLE_PLAIN only; needs Kdim >= 3 * BK.
 template <class C, int ROLE, int ACT>
 __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMParams p) {
-  static_assert(ROLE == ROLE_UP_FWD || ROLE == ROLE_PLAIN, "the dz epilogue is not built as a stream");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   using Mma = typename C::Mma;
   constexpr int BN = C::BN, FM = C::FM, FN = C::FN, BK = C::BK;
@@ -427,9 +426,45 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
 #pragma unroll
     for (int i = 0; i < C::P_INSTR; i++) asm volatile("" : "+v"(rows_next[i]));
   };
-  constexpr int PARK = 32 * EpiLayout<C::TN>::ROW_BYTES;  // one wave's parked fragment row
+  // what a wave parks in the two ring slots the tile's last stage vacates: a 32-row fragment row of its output, or (dz)
+  // 16 staged rows of z / dz and of y1s
+  constexpr int PARK = ROLE == ROLE_DZ ? DzStaging<C::TN, ACT, 16>::BYTES : 32 * EpiLayout<C::TN>::ROW_BYTES;
   static_assert((C::NW / 2) * PARK <= C::P_STAGE && (C::NW / 2) * PARK <= C::Q_STAGE, "parking must fit into a ring slot");
+  auto advance_tile = [&]() {
+    if (!more) return false;
+    cur = nxt;
+    nxt = nn;
+    more = nxt.valid;
+    if (!more) nxt = cur;
+    nn = tile_at(vb += gridDim.x);
+    token_rows(nxt, rows_next);
+    return true;
+  };
   auto tile_end = [&](int p_slot, int q_slot) {
+    // waves 0..NW/2-1 park in the vacated P slot, the others in the vacated Q slot
+    char* region = wave < C::NW / 2 ? smem + p_slot * C::P_STAGE + wave * PARK
+                                    : smem + Q_RING + q_slot * C::Q_STAGE + (wave - C::NW / 2) * PARK;
+    if constexpr (ROLE == ROLE_DZ) {
+      DzEpilogueArgs da = {};
+      da.zin = p.zin;
+      da.zin_stride = p.zin_stride;
+      da.dz = p.out0;
+      da.dz_stride = p.out0_stride;
+      da.y1s = p.out1;
+      da.y1s_stride = p.out1_stride;
+      da.scores = p.scores;
+      da.sidx = p.sidx;
+      da.ds_partial = p.ds_partial;
+      da.ds_cols = p.ds_cols;
+      da.ds_col = (cur.n0 / BN) * C::WN + wn;
+      da.m_base = cur.row0 + wm * C::TM;
+      da.row_end = cur.row_end;
+      da.n_base = cur.n0 + wn * C::TN;
+      da.N = p.N;
+      // every wave has issued its reads of the last stage ahead of the barrier in front of the last step
+      dz_epilogue<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) ? 2 : 1, false, 16>(acc, region, opaque_lane(), da, [] {});
+      return advance_tile();
+    }
     FwdEpilogueArgs ea;
     ea.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
     ea.out0 = p.out0;
@@ -440,18 +475,8 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
     ea.row_end = cur.row_end;
     ea.n_base = cur.n0 + wn * C::TN;
     ea.N = p.N;
-    // waves 0..NW/2-1 park in the vacated P slot, the others in the vacated Q slot
-    char* region = wave < C::NW / 2 ? smem + p_slot * C::P_STAGE + wave * PARK
-                                    : smem + Q_RING + q_slot * C::Q_STAGE + (wave - C::NW / 2) * PARK;
     forward_epilogue_rows<Mma, C::TM, C::TN, ROLE == ROLE_UP_FWD, ACT>(acc, region, opaque_lane(), ea);
-    if (!more) return false;
-    cur = nxt;
-    nxt = nn;
-    more = nxt.valid;
-    if (!more) nxt = cur;
-    nn = tile_at(vb += gridDim.x);
-    token_rows(nxt, rows_next);
-    return true;
+    return advance_tile();
   };
   gemm_stream_loop<FN, C::NP, (C::QMN ? 2 * FN : FN) + C::NP, C::P_INSTR, C::Q_INSTR, C::STEPS, Mma>(
       S_total, acc, issue_p, issue_q, load, issued_p, issued_q, first_boundary, tile_end);
@@ -473,11 +498,11 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
-  if constexpr (ROLE != ROLE_DZ) {
+  {
     const Tuning& tune = tuning();
     // the tile-stream kernel addresses a gathered token operand with 32-bit byte offsets from the tensor's start
     const bool offsets_fit = p.gidx == nullptr || p.p_rows * p.p_stride * 2 <= 0xffffffffll;
-    if (tune.gemm_stream && p.Kdim >= 3 * C::BK && offsets_fit) {
+    if (tune.gemm_stream && (ROLE != ROLE_DZ || tune.dz_stream) && p.Kdim >= 3 * C::BK && offsets_fit) {
       static LdsLimitOnce lds_limit_stream;
       auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
       const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
