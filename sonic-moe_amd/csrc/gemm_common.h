@@ -136,7 +136,7 @@ SMOE_DEV void lds_barrier() {
 struct Bf16Mma32 {
   typedef bf16x8 Frag;
   typedef f32x16 Acc;
-  static constexpr int FR = 32, KSTEP = 16, PH = 1, ACC_REGS = 16;
+  static constexpr int FR = 32, KSTEP = 16, PH = 1, ACC_REGS = 16, FRAG_REGS = 4;
   static constexpr int qset(int step) { return step & 1; }
   static constexpr int phalf(int) { return 0; }
   static constexpr bool reads_q(int) { return true; }
@@ -148,7 +148,7 @@ struct Bf16Mma32 {
 struct Bf16Mma16 {
   typedef bf16x8 Frag;
   typedef f32x4 Acc;
-  static constexpr int FR = 16, KSTEP = 32, PH = 2, ACC_REGS = 4;
+  static constexpr int FR = 16, KSTEP = 32, PH = 2, ACC_REGS = 4, FRAG_REGS = 4;
   static constexpr int qset(int step) { return (step >> 1) & 1; }
   static constexpr int phalf(int step) { return step & 1; }
   static constexpr bool reads_q(int step) { return (step & 1) == 0; }
@@ -191,6 +191,9 @@ SMOE_DEV void mma_step(typename Mma::Acc (&acc)[NQ][NP * Mma::PH], typename Mma:
     __builtin_amdgcn_sched_group_barrier(0x100, RPM, 0);
   }
   __builtin_amdgcn_sched_group_barrier(0x008, NM - NR, 0);
+  // large fragments: keep the scheduler from pulling the reads of later steps up in front of this one (more than two
+  // fragment sets do not fit beside the accumulators)
+  if constexpr (Mma::FRAG_REGS > 4) __builtin_amdgcn_sched_barrier(0);
 }
 
 // The last step of a stage whose ring slots are refilled: `deal(i)` is called behind the i-th matrix instruction and
@@ -383,16 +386,20 @@ SMOE_DEV void gemm_mainloop_asym(const int S, typename Mma::Acc (&acc)[NQ][NP * 
 //                              barrier behind the last stage); advances the caller's tile state and returns false if
 //                              the tile was the workgroup's last.  The accumulators need no clearing: the first
 //                              k-slice of every tile starts them from zero
-// Needs S >= 3 (stage 0 of the next tile is requested at the latest behind stage S-3 of the current one).  Stores and
-// loads share one counter and may retire out of order with respect to each other, so the first wait of a tile is for
-// everything; from then on only loads are outstanding and the counted waits are exact again.
-template <int NQ, int NP, int NREADS, int PI, int QI, int STEPS, class Mma = Bf16Mma, int RPM = 1, class IssueP,
-          class IssueQ, class Load, class IssuedP, class IssuedQ, class First, class TileEnd>
+// QS = 3 is that asymmetric ring and needs S >= 3 (stage 0 of the next tile is requested at the latest behind stage S-3
+// of the current one); QS = 2 is a plain double buffer (both operands two slots, one stage in flight, every wait is
+// for everything) and needs S >= 2.  Stores and loads share one counter and may retire out of order with respect to
+// each other, so the first wait of a tile is for everything; from then on only loads are outstanding and the counted
+// waits are exact again.
+template <int NQ, int NP, int NREADS, int PI, int QI, int STEPS, class Mma = Bf16Mma, int RPM = 1, int QS = 3,
+          class IssueP, class IssueQ, class Load, class IssuedP, class IssuedQ, class First, class TileEnd>
 SMOE_DEV void gemm_stream_loop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mma::PH], IssueP&& issue_p,
                                IssueQ&& issue_q, Load&& load, IssuedP&& issued_p, IssuedQ&& issued_q,
                                First&& first_boundary, TileEnd&& tile_end) {
   static_assert(STEPS % 2 == 0 && PI + 2 * QI < 64, "unsupported pipeline shape");
   static_assert(STEPS > Mma::PH, "a stage holds more than one k-slice");
+  static_assert(QS == 2 || QS == 3, "the weight operand's ring has two or three slots");
+  constexpr int AHEAD = (QS - 2) * QI;  // loads of the stage after next that may be outstanding behind a stage
   typename Mma::Frag qf[2][NQ], pf[2][NP];
   constexpr int NM = NQ * NP, LPS = PI + QI, LAST = STEPS - 1;
   auto all_p = [&](int slot) {
@@ -417,25 +424,36 @@ SMOE_DEV void gemm_stream_loop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mm
     });
   };
   constexpr std::false_type later{};
-  constexpr std::true_type first{};
   constexpr std::integral_constant<int, 0> step0{};
 
   all_p(0);
   all_q(0);
   all_p(1);
   all_q(1);
-  all_q(2);
-  wait_vmem_upto<PI + 2 * QI>();
+  if constexpr (QS == 3) all_q(2);
+  wait_vmem_upto<PI + QI + AHEAD>();
   lds_barrier();
   read_step(0, 0, step0);
   int bp = 0, bq = 0;
+  // Branching code follows the last step of every stage (stream bookkeeping, the epilogue).  Without a use of the
+  // accumulators in front of it the compiler sinks that step's matrix instructions past the branches to where their
+  // results are first read (seen with the 16-register fragments): the matrix pipe idles and the step's operand
+  // fragments stay alive into the epilogue.
+  auto pin_accumulators = [&]() {
+    if constexpr (Mma::FRAG_REGS > 4) {
+#pragma unroll
+      for (int q = 0; q < NQ; q++)
+#pragma unroll
+        for (int pp = 0; pp < NP * Mma::PH; pp++) asm volatile("" : "+v"(acc[q][pp]));
+    }
+  };
   // boundary behind a stage that is not the tile's last: read step 0 of the next stage, refill the vacated slots
   auto boundary = [&]() {
     lds_barrier();
-    const int np = bp ^ 1, nq = bq == 2 ? 0 : bq + 1;
+    const int np = bp ^ 1, nq = bq == QS - 1 ? 0 : bq + 1;
     read_step(np, nq, step0);
     __builtin_amdgcn_sched_barrier(0);
-    // P(s+2), Q(s+3) into the slots stage s leaves behind
+    // P(s+2), Q(s+QS) into the slots stage s leaves behind
     mma_step_refill<Mma, NQ, NP, LAST>(acc, qf, pf, [&](auto i_c) {
       constexpr int i = decltype(i_c)::value;
       static_for<LPS>([&](auto j_c) {
@@ -446,34 +464,41 @@ SMOE_DEV void gemm_stream_loop(const int S, typename Mma::Acc (&acc)[NQ][NP * Mm
         }
       });
     });
+    pin_accumulators();
     issued_p();
     issued_q();
     bp = np;
     bq = nq;
   };
+  // 16-register accumulator fragments: a zero operand would occupy 16 registers through the whole loop, so the tile
+  // is started by clearing the accumulators instead
+  constexpr bool CLEAR = Mma::ACC_REGS > 4;
+  constexpr std::integral_constant<bool, !CLEAR> first{};
   for (;;) {
     // stage 0: stores of the previous epilogue may still be outstanding, wait for everything
+    if constexpr (CLEAR) clear_accumulators<Mma>(acc);
     inner_steps(bp, bq, first);
     wait_vmem_all();
     first_boundary();
     boundary();
     for (int s = 1; s + 1 < S; s++) {
       inner_steps(bp, bq, later);
-      wait_vmem_upto<QI>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
+      wait_vmem_upto<AHEAD>();  // P(s+1) and Q(s+1) have landed; only Q(s+2) may still be on its way
       boundary();
     }
     // last stage: the stages of the next tile that are due are already requested; its own slots become scratch
     inner_steps(bp, bq, later);
-    wait_vmem_upto<QI>();
+    wait_vmem_upto<AHEAD>();
     lds_barrier();
     mma_step<Mma, NQ, NP, NREADS, RPM, LAST, false>(acc, qf, pf);
+    pin_accumulators();
     if (!tile_end(bp, bq)) break;
     wait_lds_all();
     lds_barrier();  // every wave has read its parked rows back: the two slots may be refilled
     all_p(bp);
     all_q(bq);
     bp ^= 1;
-    bq = bq == 2 ? 0 : bq + 1;
+    bq = bq == QS - 1 ? 0 : bq + 1;
     read_step(bp, bq, step0);
   }
   wait_vmem_all();  // the streams ran ahead into ring slots nobody reads any more: let those loads land before the end
@@ -982,6 +1007,48 @@ SMOE_DEV int64_t xcd_linear_tile_of(int64_t b, int64_t total) {
   return lin < total ? lin : -1;
 }
 SMOE_DEV int64_t xcd_linear_tile(int64_t total) { return xcd_linear_tile_of(blockIdx.x, total); }
+
+// The tiles a persistent workgroup of a tile-stream kernel walks through: virtual workgroup vb = b, b + gridDim.x, ...
+// of the XCD-aware order of the one-tile-per-workgroup kernels (groups of GM token tiles share a feature panel).  The
+// bookkeeping is read through the constant address space: uniform addresses then become scalar loads, which do not
+// touch the vector-memory counter the ring is timed with.
+struct StreamTile {
+  int e, row0, row_end, n0;
+  bool valid;
+};
+struct StreamTiles {
+  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+  const_i32_ptr expert, row0, off;
+  int num_m_tiles, n_tiles, bn;
+  int64_t total, per_xcd;
+  __device__ __forceinline__ StreamTiles(const TileMap& tm, const int32_t* off_, int n_tiles_, int bn_)
+      : expert((const_i32_ptr)tm.expert), row0((const_i32_ptr)tm.row0), off((const_i32_ptr)off_), n_tiles(n_tiles_),
+        bn(bn_) {
+    num_m_tiles = ((const_i32_ptr)tm.header)[0];
+    total = (int64_t)num_m_tiles * n_tiles;
+    per_xcd = (total + 7) >> 3;
+  }
+  __device__ __forceinline__ StreamTile at(int64_t vb) const {
+    StreamTile t = {0, 0, 1, 0, false};
+    const int64_t slot = vb >> 3;
+    const int64_t lin = (vb & 7) * per_xcd + slot;
+    if (slot < per_xcd && lin < total) {
+      constexpr int GM = 8;
+      const int64_t per_group = (int64_t)GM * n_tiles;
+      const int group = (int)(lin / per_group);
+      const int first_m = group * GM;
+      const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
+      const int within = (int)(lin - (int64_t)group * per_group);
+      const int mt = first_m + within % gm;
+      t.e = expert[mt];
+      t.row0 = row0[mt];
+      t.row_end = off[t.e + 1];
+      t.n0 = (within / gm) * bn;
+      t.valid = true;
+    }
+    return t;
+  }
+};
 
 int launch_ds_finalize(const float* ds_partial, int ncols, const int32_t* sidx, float* ds, int64_t TK, hipStream_t st);
 

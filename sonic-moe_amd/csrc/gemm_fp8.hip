@@ -105,11 +105,12 @@ struct Fp8Params {
 };
 
 struct Fp8Cfg {
-  // 4 wavefronts, 128 x 128 each: the fragments of an fp8 slice are twice as large as bf16 ones, and two register sets
-  // of them beside a 128 x 64 accumulator tile do not fit the 256 registers of an 8-wavefront workgroup
-  static constexpr int BM = 256, BN = 256, WM = 2, WN = 2, BKB = 128, NSTAGE = 2;  // BKB: contraction bytes per stage
+  // 8 wavefronts (two per SIMD), 128 x 64 each.  The fragments of an fp8 slice are twice as large as bf16 ones: a step
+  // works on half of the wave's token rows, so two register sets of 2 + 2 fragments are all that is live beside the
+  // 128 accumulator registers
+  static constexpr int BM = 256, BN = 256, WM = 2, WN = 4, BKB = 128, NSTAGE = 2;  // BKB: contraction bytes per stage
   static constexpr int NW = WM * WN, NT = NW * 64;
-  static constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32;
+  static constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32, NP = 1;
   static constexpr int P_STAGE = BM * BKB, Q_STAGE = BN * BKB, S_STAGE = (BM + BN) * 4;
   static constexpr int STAGE = P_STAGE + Q_STAGE + S_STAGE;
   static constexpr int P_INSTR = P_STAGE / 1024 / NW, Q_INSTR = Q_STAGE / 1024 / NW;
@@ -117,13 +118,24 @@ struct Fp8Cfg {
   static constexpr int EPI = NW * TM * (TN * 2 + 16);
   static constexpr int SMEM = NSTAGE * STAGE > EPI ? NSTAGE * STAGE : EPI;
   static constexpr int S_INSTR = (BM + BN) / 64 / NW;  // scale loads (64 rows each) per wave and stage
+  // tile-stream kernel: two slots per operand, a slot = the operand's stage + its scale words.  Every wave fetches the
+  // scale words of 32 rows of each operand (its upper 32 lanes repeat the lower ones), 256 bytes per wave and slot
+  static constexpr int SC_BYTES = NW * 256, P_SLOT = P_STAGE + SC_BYTES, Q_SLOT = Q_STAGE + SC_BYTES;
+  static constexpr int STREAM_SMEM = 2 * (P_SLOT + Q_SLOT);
+  static constexpr int PS_INSTR = P_STAGE / 1024 / NW, QS_INSTR = Q_STAGE / 1024 / NW;  // data loads per wave and stage
+  static_assert(BM == NW * 32 && BN == NW * 32, "32 scale rows of each operand per wave");
+  static_assert(STREAM_SMEM <= 160 * 1024, "LDS budget of a CU");
   static_assert(S_INSTR * NW * 64 == BM + BN, "the scale rows must split evenly over the wavefronts");
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
 };
 
-// direct-to-LDS load of one 32-bit word per lane: the wavefront's 64 words land at lds_wave_base + 4 * lane
-SMOE_DEV void load4_to_lds(const void* g, uint32_t lds_wave_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(g), "s"(lds_wave_base) : "memory");
+// direct-to-LDS load of one 32-bit word per lane through a buffer resource: the wavefront's 64 words land at
+// lds_wave_base + 4 * lane
+SMOE_DEV void buffer_load4_to_lds(i32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_wave_base) {
+  asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dword %0, %1, %2 offen lds"
+               :
+               : "v"(voff), "s"(rsrc), "s"(soff), "s"(lds_wave_base)
+               : "memory");
 }
 
 // Operand fragment of v_mfma_scale_f32_32x32x64_f8f6f4: lane l holds row l%32 and, of the 64 contraction bytes of the
@@ -136,12 +148,13 @@ struct Fp8Frag {
 struct Fp8Mma {
   typedef Fp8Frag Frag;
   typedef f32x16 Acc;
-  // a step is one k-slice of 64 contraction bytes and reads all of the wave's fragments (see Bf16Mma32)
-  static constexpr int FR = 32, KSTEP = 64, PH = 1, ACC_REGS = 16;
-  static constexpr int qset(int step) { return step & 1; }
-  static constexpr int phalf(int) { return 0; }
-  static constexpr bool reads_q(int) { return true; }
-  static constexpr int kslice(int step) { return step; }
+  // a step is ONE of the wave's four token fragments on one k-slice of 64 contraction bytes; the feature fragments
+  // are read on the first of a slice's four steps (see Bf16Mma16).  Two sets of 1 + 2 fragments are live.
+  static constexpr int FR = 32, KSTEP = 64, PH = 4, ACC_REGS = 16, FRAG_REGS = 9;
+  static constexpr int qset(int step) { return (step >> 2) & 1; }
+  static constexpr int phalf(int step) { return step & 3; }
+  static constexpr bool reads_q(int step) { return (step & 3) == 0; }
+  static constexpr int kslice(int step) { return step >> 2; }
   static __device__ __forceinline__ f32x16 run(const Frag& q, const Frag& p, f32x16 c) {
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(q.data, p.data, c, 0, 0, 0, q.scale, 0, p.scale);
   }
@@ -152,7 +165,7 @@ struct Fp8Mma {
 // lane's columns of the block, one shuffle for the other half-wave), the e4m3 bytes are parked in LDS and written back
 // 16 bytes per lane; the scale bytes go to the (I / 128, rows) table the down-projection reads.
 template <int TM, int TN, int FM, int FN, int ACT>
-SMOE_DEV void fp8_activation_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wave, int lane, uint8_t* yq, int I,
+SMOE_DEV void fp8_activation_epilogue(f32x16 (&acc)[FN][FM], char* region, int lane, uint8_t* yq, int I,
                                       uint32_t* yq_scales, int64_t yq_rows, int m_base, int row_end, int n_base) {
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
@@ -160,8 +173,7 @@ SMOE_DEV void fp8_activation_epilogue(f32x16 (&acc)[FN][FM], char* smem, int wav
   constexpr int NB = YC / 32, FPB = FN / NB;  // 32-column blocks, accumulator fragments per block
   constexpr int ROWB = YC + 16;               // parked row, padded against bank conflicts
   constexpr int LPR = YC / 16, RPP = 64 / LPR;
-  // the wave's own parking region of forward_epilogue (other waves may still be flushing theirs)
-  char* region = smem + wave * (TM * (TN * 2 + 16));
+  // region: the wave's own parking region of the forward epilogue (32 padded rows are used)
   const int half = lane >> 5, mrow = lane & 31;
   const int y_base = GLU ? n_base / 2 : n_base;
   static_for<FM>([&](auto fm_c) {
@@ -245,42 +257,49 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
   const int row_end = p.off[e + 1];
   const int n0 = nt * C::BN;
 
-  // per-lane global source pointers of the data pieces (advance by one stage per k-step)
-  const uint8_t* p_src[C::P_INSTR];
+  // Operands are fetched through buffer resources: a lane keeps one 32-bit byte offset per load, the position along
+  // the contraction is a wave-uniform offset.  The token operand's resource starts at the tensor (gathered rows: row *
+  // stride fits 32 bits, checked on the host) or at the tile's first row; the weight operand's at the tile's expert.
+  const i32x4 p_rsrc = make_buffer_resource(p.gidx ? p.P : p.P + (int64_t)row0 * p.p_stride);
+  const i32x4 q_rsrc = make_buffer_resource(p.Q + (int64_t)e * p.q_stride_e);
+  uint32_t p_voff[C::P_INSTR], q_voff[C::Q_INSTR];
 #pragma unroll
   for (int i = 0; i < C::P_INSTR; i++) {
     const int r = (wave * C::P_INSTR + i) * C::KRPI + lane / C::KPR;
     int m = row0 + r;
     m = m < row_end ? m : row_end - 1;
-    const int64_t src_row = p.gidx ? (int64_t)p.gidx[m] : (int64_t)m;
-    p_src[i] = p.P + src_row * p.p_stride + (((lane % C::KPR) ^ kswz<64>(r)) << 4);
+    const uint32_t src_row = p.gidx ? (uint32_t)p.gidx[m] : (uint32_t)(m - row0);
+    p_voff[i] = src_row * (uint32_t)p.p_stride + (((lane % C::KPR) ^ kswz<64>(r)) << 4);
   }
-  const uint8_t* q_src[C::Q_INSTR];
-  const uint8_t* qe = p.Q + (int64_t)e * p.q_stride_e;
 #pragma unroll
   for (int i = 0; i < C::Q_INSTR; i++) {
     const int r = (wave * C::Q_INSTR + i) * C::KRPI + lane / C::KPR;
     int n = n0 + r;
     n = n < p.N ? n : p.N - 1;
-    q_src[i] = qe + (int64_t)n * p.q_stride_row + (((lane % C::KPR) ^ kswz<64>(r)) << 4);
+    q_voff[i] = (uint32_t)n * (uint32_t)p.q_stride_row + (((lane % C::KPR) ^ kswz<64>(r)) << 4);
   }
   // this lane's scale words: load j of wave w covers rows (w * S_INSTR + j) * 64 .. + 63 of the tile's 256 token rows
-  // followed by its 256 feature rows
-  const uint32_t* s_src[C::S_INSTR];
-  int64_t s_step[C::S_INSTR];
+  // followed by its 256 feature rows; a table row holds one 128-element block of the contraction for all rows
+  i32x4 s_rsrc[C::S_INSTR];
+  uint32_t s_voff[C::S_INSTR], s_step[C::S_INSTR];
 #pragma unroll
   for (int j = 0; j < C::S_INSTR; j++) {
-    const int r = (wave * C::S_INSTR + j) * 64 + lane;
-    if (r < C::BM) {
-      int m = row0 + r;
+    const int r0 = (wave * C::S_INSTR + j) * 64;  // wave-uniform
+    if (r0 < C::BM) {
+      int m = row0 + r0 + lane;
       m = m < row_end ? m : row_end - 1;
-      s_src[j] = p.p_scales + (p.gidx ? (int64_t)p.gidx[m] : (int64_t)m);
-      s_step[j] = p.p_rows;
+      s_rsrc[j] = make_buffer_resource(p.gidx ? p.p_scales : p.p_scales + row0);
+      s_voff[j] = (p.gidx ? (uint32_t)p.gidx[m] : (uint32_t)(m - row0)) * 4u;
+#ifdef SMOE_PROBE_SCALES_CONTIG
+      s_voff[j] = (uint32_t)lane * 4u;
+#endif
+      s_step[j] = (uint32_t)p.p_rows * 4u;
     } else {
-      int n = n0 + r - C::BM;
+      int n = n0 + r0 - C::BM + lane;
       n = n < p.N ? n : p.N - 1;
-      s_src[j] = p.q_scales + (int64_t)e * p.N + n;
-      s_step[j] = p.q_rows;
+      s_rsrc[j] = make_buffer_resource(p.q_scales + (int64_t)e * p.N);
+      s_voff[j] = (uint32_t)n * 4u;
+      s_step[j] = (uint32_t)p.q_rows * 4u;
     }
   }
 
@@ -312,42 +331,55 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[fn][fm][r] = 0.f;
 
-  auto issue = [&](int buf, int /*s*/, auto i_c) {
+  auto issue = [&](int buf, int s, auto i_c) {
     constexpr int i = decltype(i_c)::value;
     const uint32_t base = smem_base + buf * C::STAGE;
     if constexpr (i < C::P_INSTR) {
-      load16_to_lds(p_src[i], base + (wave * C::P_INSTR + i) * 1024);
-      p_src[i] += C::BKB;
+      buffer_load16_to_lds(p_rsrc, p_voff[i], (uint32_t)s * C::BKB, base + (wave * C::P_INSTR + i) * 1024);
     } else if constexpr (i < C::P_INSTR + C::Q_INSTR) {
       constexpr int j = i - C::P_INSTR;
-      load16_to_lds(q_src[j], base + C::P_STAGE + (wave * C::Q_INSTR + j) * 1024);
-      q_src[j] += C::BKB;
+      buffer_load16_to_lds(q_rsrc, q_voff[j], (uint32_t)s * C::BKB, base + C::P_STAGE + (wave * C::Q_INSTR + j) * 1024);
     } else {
       constexpr int j = i - C::P_INSTR - C::Q_INSTR;
-      load4_to_lds(s_src[j], base + C::P_STAGE + C::Q_STAGE + (wave * C::S_INSTR + j) * 256);
-      s_src[j] += s_step[j];
+#ifndef SMOE_PROBE_NO_SCALE_LOADS
+      buffer_load4_to_lds(s_rsrc[j], s_voff[j], (uint32_t)s * s_step[j],
+                          base + C::P_STAGE + C::Q_STAGE + (wave * C::S_INSTR + j) * 256);
+#endif
     }
   };
-  auto load = [&](int buf, int /*s*/, auto step_c, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[FM]) {
-    constexpr int ks = decltype(step_c)::value;
+  auto load = [&](int buf, int /*s*/, auto step_c, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[C::NP]) {
+    constexpr int step = decltype(step_c)::value, ks = Fp8Mma::kslice(step), ph = Fp8Mma::phalf(step);
     const char* st = smem + buf * C::STAGE;
     const int shift = 8 * (2 * ks + half);
 #pragma unroll
-    for (int fm = 0; fm < FM; fm++) {
+    for (int pp = 0; pp < C::NP; pp++) {
+      const int fm = ph * C::NP + pp;
       const i32x4 lo = *(const i32x4*)(st + p_off[ks][0] + fm * 32 * C::BKB);
       const i32x4 hi = *(const i32x4*)(st + p_off[ks][1] + fm * 32 * C::BKB);
-      pf[fm].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      pf[fm].scale = (int)(*(const uint32_t*)(st + ps_off + fm * 32 * 4) >> shift);
+      pf[pp].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#ifdef SMOE_PROBE_NO_SCALE_READS
+      pf[pp].scale = 127;
+#else
+      pf[pp].scale = (int)(*(const uint32_t*)(st + ps_off + fm * 32 * 4) >> shift);
+#endif
     }
+    if constexpr (Fp8Mma::reads_q(step)) {
 #pragma unroll
-    for (int fn = 0; fn < FN; fn++) {
-      const i32x4 lo = *(const i32x4*)(st + q_off[ks][0] + fn * 32 * C::BKB);
-      const i32x4 hi = *(const i32x4*)(st + q_off[ks][1] + fn * 32 * C::BKB);
-      qf[fn].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-      qf[fn].scale = (int)(*(const uint32_t*)(st + qs_off + fn * 32 * 4) >> shift);
+      for (int fn = 0; fn < FN; fn++) {
+        const i32x4 lo = *(const i32x4*)(st + q_off[ks][0] + fn * 32 * C::BKB);
+        const i32x4 hi = *(const i32x4*)(st + q_off[ks][1] + fn * 32 * C::BKB);
+        qf[fn].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+#ifdef SMOE_PROBE_NO_SCALE_READS
+        qf[fn].scale = 127;
+#else
+        qf[fn].scale = (int)(*(const uint32_t*)(st + qs_off + fn * 32 * 4) >> shift);
+#endif
+      }
     }
   };
-  gemm_mainloop<FN, FM, 3 * (FN + FM), C::P_INSTR + C::Q_INSTR + C::S_INSTR, SLICES, C::NSTAGE, Fp8Mma>(S_total, acc, issue, load);
+  // 3 LDS reads per fragment (two 16-byte pieces and the scale word), dealt out three per matrix instruction
+  gemm_mainloop<FN, C::NP, 3 * (FN + C::NP), C::P_INSTR + C::Q_INSTR + C::S_INSTR, Fp8Mma::PH * SLICES, C::NSTAGE, Fp8Mma, 4>(
+      S_total, acc, issue, load);
 
   if constexpr (DZ) {
     DzEpilogueArgs da = {};
@@ -392,9 +424,213 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
   forward_epilogue<Fp8Mma, C::TM, C::TN, WITH_ACT, ACT>(acc, smem, wave, lane, ea);
   if constexpr (WITH_ACT) {
     if (p.yq != nullptr)  // the parking area of forward_epilogue is read back by the same wave that wrote it: no barrier
-      fp8_activation_epilogue<C::TM, C::TN, FM, FN, ACT>(acc, smem, wave, lane, p.yq, p.I, p.yq_scales, p.yq_rows,
-                                                          ea.m_base, row_end, ea.n_base);
+      fp8_activation_epilogue<C::TM, C::TN, FM, FN, ACT>(acc, smem + wave * (C::TM * (C::TN * 2 + 16)), lane, p.yq, p.I,
+                                                          p.yq_scales, p.yq_rows, ea.m_base, row_end, ea.n_base);
   }
+}
+
+// The same GEMM as a tile stream: one workgroup per compute unit walks through the tiles b, b + gridDim.x, ... and keeps
+// its double buffer running across tile boundaries (gemm_stream_loop with two slots per operand): the first stage of
+// the next tile is on its way while the finished tile's epilogue runs, and the epilogue's stores drain under the next
+// tile's first stages.  Needs Kdim >= 2 stages.  The forward roles only: the dz epilogue stages 32 rows of z and y1s
+// per wave (32-row fragments), which the two vacated slots cannot hold for eight waves.
+template <bool WITH_ACT, int ACT>
+__global__ __launch_bounds__(Fp8Cfg::NT) void fp8_stream_kernel(const Fp8Params p) {
+  using C = Fp8Cfg;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  constexpr int FM = C::FM, FN = C::FN, SLICES = C::BKB / 64, PI = C::PS_INSTR, QI = C::QS_INSTR;
+  const uint32_t smem_base = lds_address(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % C::WM, wn = wave / C::WM;
+
+  const StreamTiles tiles(p.tm, p.off, p.n_tiles, C::BN);
+  int64_t vb = blockIdx.x;
+  StreamTile cur = tiles.at(vb);
+  if (!cur.valid) return;
+  StreamTile nxt = tiles.at(vb += gridDim.x);
+  bool more = nxt.valid;  // a tile follows the current one
+  if (!more) nxt = cur;   // the streams always run on: past the last tile they re-read it into slots nobody reads
+  StreamTile nn = tiles.at(vb += gridDim.x);
+
+  // Everything a tile switch computes from the lane number starts from a copy of it the compiler cannot see through:
+  // otherwise the per-lane parts are hoisted out of the tile loop and occupy registers the main loop needs.
+  auto opaque_lane = [&]() {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
+  // source rows of a tile's token operand: one per data load and the row whose scale word the lane fetches
+  auto token_rows = [&](const StreamTile& t, int(&rows)[PI + 1]) {
+    const int ln = opaque_lane();
+#pragma unroll
+    for (int i = 0; i <= PI; i++) {
+      int m = t.row0 + (i < PI ? (wave * PI + i) * C::KRPI + ln / C::KPR : wave * 32 + (ln & 31));
+      m = m < t.row_end ? m : t.row_end - 1;
+      rows[i] = p.gidx ? p.gidx[m] : m - t.row0;
+    }
+  };
+  // Operands and scale tables are fetched through buffer resources: a lane keeps one 32-bit byte offset per load
+  // (fixed for a tile), the position along the contraction is a wave-uniform offset.  The token operand's resources
+  // start at the tensors (gathered rows) or at the tile's first row; the weight operand's at the tile's expert.
+  uint32_t p_voff[PI + 1], q_voff[QI + 1];
+  i32x4 p_rsrc = make_buffer_resource(p.P), ps_rsrc = make_buffer_resource(p.p_scales);
+  i32x4 q_rsrc = make_buffer_resource(p.Q), qs_rsrc = make_buffer_resource(p.q_scales);
+  const uint32_t p_row_bytes = (uint32_t)p.p_stride, q_row_bytes = (uint32_t)p.q_stride_row;
+  const uint32_t ps_step = (uint32_t)p.p_rows * 4u, qs_step = (uint32_t)p.q_rows * 4u;
+  auto point_p = [&](const int(&rows)[PI + 1], const StreamTile& t) {
+    const int ln = opaque_lane();
+    if (!p.gidx) {
+      p_rsrc = make_buffer_resource(p.P + (int64_t)t.row0 * p.p_stride);
+      ps_rsrc = make_buffer_resource(p.p_scales + t.row0);
+    }
+#pragma unroll
+    for (int i = 0; i < PI; i++) {
+      const int r = (wave * PI + i) * C::KRPI + ln / C::KPR;
+      // rows and row sizes are below 2^24 (checked on the host): one 32-bit multiply-add per offset
+      p_voff[i] = __umul24((uint32_t)rows[i], p_row_bytes) + ((((uint32_t)ln % C::KPR) ^ kswz<64>(r)) << 4);
+    }
+    p_voff[PI] = (uint32_t)rows[PI] * 4u;
+  };
+  auto point_q = [&](const StreamTile& t) {
+    const int ln = opaque_lane();
+    q_rsrc = make_buffer_resource(p.Q + (int64_t)t.e * p.q_stride_e);
+    qs_rsrc = make_buffer_resource(p.q_scales + (int64_t)t.e * p.N);
+#pragma unroll
+    for (int i = 0; i <= QI; i++) {
+      const int r = i < QI ? (wave * QI + i) * C::KRPI + ln / C::KPR : wave * 32 + (ln & 31);
+      int n = t.n0 + r;
+      n = n < p.N ? n : p.N - 1;
+      q_voff[i] = i < QI ? __umul24((uint32_t)n, q_row_bytes) + ((((uint32_t)ln % C::KPR) ^ kswz<64>(r)) << 4) : (uint32_t)n * 4u;
+    }
+  };
+  int rows_next[PI + 1];  // token rows of nxt: loaded at the start of a tile, picked up behind its first stage
+  {
+    int rows_cur[PI + 1];
+    token_rows(cur, rows_cur);
+    point_p(rows_cur, cur);
+    point_q(cur);
+    token_rows(nxt, rows_next);
+  }
+
+  const int S_total = p.Kdim / C::BKB;
+
+  // per-lane LDS fragment offsets (bytes inside a slot): two 16-byte pieces per slice, one scale word per stage
+  const int half = lane >> 5;
+  int p_off[SLICES][2], q_off[SLICES][2];
+  {
+    const int prow = wm * C::TM + (lane & 31), qrow = wn * C::TN + (lane & 31);
+    const int psw = kswz<64>(prow), qsw = kswz<64>(qrow);
+#pragma unroll
+    for (int ks = 0; ks < SLICES; ks++)
+#pragma unroll
+      for (int j = 0; j < 2; j++) {
+        const int piece = 4 * ks + 2 * j + half;
+        p_off[ks][j] = prow * C::BKB + ((piece ^ psw) << 4);
+        q_off[ks][j] = qrow * C::BKB + ((piece ^ qsw) << 4);
+      }
+  }
+  // the scale word of tile row r lies at (r / 32) * 256 + (r % 32) * 4 of the slot's scale area
+  const int ps_off = C::P_STAGE + wm * (C::TM / 32) * 256 + (lane & 31) * 4;
+  const int qs_off = C::Q_STAGE + wn * (C::TN / 32) * 256 + (lane & 31) * 4;
+
+  f32x16 acc[FN][FM];  // started from zero by the first k-slice of every tile
+
+  constexpr int Q_RING = 2 * C::P_SLOT;
+  int p_stage = 0, q_stage = 0;  // stages issued to each stream for the tile it is on
+  auto issue_p = [&](int slot, auto i_c) {
+    constexpr int i = decltype(i_c)::value;
+    const uint32_t base = smem_base + slot * C::P_SLOT;
+    if constexpr (i < PI)
+      buffer_load16_to_lds(p_rsrc, p_voff[i], (uint32_t)p_stage * C::BKB, base + (wave * PI + i) * 1024);
+    else
+      buffer_load4_to_lds(ps_rsrc, p_voff[PI], (uint32_t)p_stage * ps_step, base + C::P_STAGE + wave * 256);
+  };
+  auto issue_q = [&](int slot, auto j_c) {
+    constexpr int j = decltype(j_c)::value;
+    const uint32_t base = smem_base + Q_RING + slot * C::Q_SLOT;
+    if constexpr (j < QI)
+      buffer_load16_to_lds(q_rsrc, q_voff[j], (uint32_t)q_stage * C::BKB, base + (wave * QI + j) * 1024);
+    else
+      buffer_load4_to_lds(qs_rsrc, q_voff[QI], (uint32_t)q_stage * qs_step, base + C::Q_STAGE + wave * 256);
+  };
+  auto issued_p = [&]() {
+    if (++p_stage == S_total) {
+      p_stage = 0;
+      point_p(rows_next, nxt);
+    }
+  };
+  auto issued_q = [&]() {
+    if (++q_stage == S_total) {
+      q_stage = 0;
+      point_q(nxt);
+    }
+  };
+  auto load = [&](int p_slot, int q_slot, auto step_c, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[C::NP]) {
+    constexpr int step = decltype(step_c)::value, ks = Fp8Mma::kslice(step), ph = Fp8Mma::phalf(step);
+    const char* ps = smem + p_slot * C::P_SLOT;
+    const char* qs = smem + Q_RING + q_slot * C::Q_SLOT;
+    const int shift = 8 * (2 * ks + half);
+#pragma unroll
+    for (int pp = 0; pp < C::NP; pp++) {
+      const int fm = ph * C::NP + pp;
+      const i32x4 lo = *(const i32x4*)(ps + p_off[ks][0] + fm * 32 * C::BKB);
+      const i32x4 hi = *(const i32x4*)(ps + p_off[ks][1] + fm * 32 * C::BKB);
+      pf[pp].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      pf[pp].scale = (int)(*(const uint32_t*)(ps + ps_off + fm * 256) >> shift);
+    }
+    if constexpr (Fp8Mma::reads_q(step)) {
+#pragma unroll
+      for (int fn = 0; fn < FN; fn++) {
+        const i32x4 lo = *(const i32x4*)(qs + q_off[ks][0] + fn * 32 * C::BKB);
+        const i32x4 hi = *(const i32x4*)(qs + q_off[ks][1] + fn * 32 * C::BKB);
+        qf[fn].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        qf[fn].scale = (int)(*(const uint32_t*)(qs + qs_off + fn * 256) >> shift);
+      }
+    }
+  };
+  // the rows loaded in tile_end are complete here; naming them in an asm statement makes this the place where the
+  // compiler waits for them
+  auto first_boundary = [&]() {
+#pragma unroll
+    for (int i = 0; i <= PI; i++) asm volatile("" : "+v"(rows_next[i]));
+  };
+  // what a wave parks in the two slots the tile's last stage vacates: 32 rows of its output
+  constexpr int PARK = 32 * EpiLayout<C::TN>::ROW_BYTES;
+  static_assert((C::NW / 2) * PARK <= C::P_STAGE && (C::NW / 2) * PARK <= C::Q_STAGE, "parking must fit into a slot");
+  auto tile_end = [&](int p_slot, int q_slot) {
+    // waves 0..NW/2-1 park in the vacated token slot, the others in the vacated weight slot
+    char* region = wave < C::NW / 2 ? smem + p_slot * C::P_SLOT + wave * PARK
+                                    : smem + Q_RING + q_slot * C::Q_SLOT + (wave - C::NW / 2) * PARK;
+    const int m_base = cur.row0 + wm * C::TM, n_base = cur.n0 + wn * C::TN;
+    FwdEpilogueArgs ea;
+    ea.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
+    ea.out0 = p.out0;
+    ea.out0_stride = p.out0_stride;
+    ea.out1 = p.out1;
+    ea.out1_stride = p.out1_stride;
+    ea.m_base = m_base;
+    ea.row_end = cur.row_end;
+    ea.n_base = n_base;
+    ea.N = p.N;
+    forward_epilogue_rows<Fp8Mma, C::TM, C::TN, WITH_ACT, ACT>(acc, region, opaque_lane(), ea);
+    if constexpr (WITH_ACT) {
+      if (p.yq != nullptr)  // the region is read back by the same wave that wrote it: no barrier
+        fp8_activation_epilogue<C::TM, C::TN, FM, FN, ACT>(acc, region, opaque_lane(), p.yq, p.I, p.yq_scales,
+                                                            p.yq_rows, m_base, cur.row_end, n_base);
+    }
+    if (!more) return false;
+    cur = nxt;
+    nxt = nn;
+    more = nxt.valid;
+    if (!more) nxt = cur;
+    nn = tiles.at(vb += gridDim.x);
+    token_rows(nxt, rows_next);
+    return true;
+  };
+  // 3 LDS reads per fragment (two 16-byte pieces and the scale word), dealt out three per matrix instruction
+  gemm_stream_loop<FN, C::NP, 3 * (FN + C::NP), PI + 1, QI + 1, Fp8Mma::PH * SLICES, Fp8Mma, 4, 2>(
+      S_total, acc, issue_p, issue_q, load, issued_p, issued_q, first_boundary, tile_end);
 }
 
 template <bool WITH_ACT, int ACT, bool DZ = false>
@@ -411,9 +647,34 @@ static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t
   if (rc) return rc;
   p.n_tiles = (int)ceil_div(p.N, C::BN);
   if (DZ) p.ds_cols = p.n_tiles * C::WN;
+  // the kernel addresses its operands with 32-bit byte offsets from a buffer base
+  const int64_t lim = 1ll << 32;
+  SMOE_REQUIRE((p.gidx ? p.p_rows : (int64_t)C::BM) * p.p_stride < lim && (int64_t)p.N * p.q_stride_row < lim &&
+                   (int64_t)(p.Kdim / C::BKB) * (p.p_rows > p.q_rows ? p.p_rows : p.q_rows) * 4 < lim,
+               SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: operand too large for 32-bit offsets");
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: too many tiles");
+  const Tuning& tune = tuning();
+  const int64_t lim24 = 1ll << 24;  // the tile-stream kernel forms its offsets with 24-bit multiplies
+  const bool fits24 = p.p_rows < lim24 && p.p_stride < lim24 && p.N < lim24 && p.q_stride_row < lim24;
+  if constexpr (!DZ) if (tune.gemm_stream && p.Kdim >= 2 * C::BKB && fits24) {
+    static LdsLimitOnce lds_limit_stream;
+    auto skern = fp8_stream_kernel<WITH_ACT, ACT>;
+    const int rc_s = lds_limit_stream.ensure((const void*)skern, C::STREAM_SMEM);
+    if (rc_s) return rc_s;
+    int cus = 0;
+    const int rc_cu = device_compute_units(&cus);
+    if (rc_cu) return rc_cu;
+    int64_t sgrid = ((int64_t)cus / 8) * 8;  // one resident workgroup per compute unit, the same number on every XCD
+    // a smaller grid makes small problems run several tiles per workgroup (used by the tests)
+    if (tune.gemm_stream_grid > 0) sgrid = ((int64_t)tune.gemm_stream_grid + 7) / 8 * 8;
+    if (sgrid < 8) sgrid = 8;
+    if (sgrid > grid) sgrid = grid;
+    hipLaunchKernelGGL(skern, dim3((unsigned)sgrid), dim3(C::NT), C::STREAM_SMEM, st, p);
+    SMOE_LAUNCH_CHECK();
+    return SMOE_OK;
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;

@@ -1,4 +1,5 @@
-// Sustained MFMA rate under the power limit with random operand data: 32x32x16 against 16x16x32 (bf16), same wave tile
+// Sustained MFMA rate under the power limit with random operand data: 32x32x16 against 16x16x32 (bf16) and the scaled
+// fp8 32x32x64 form, same wave tile
 // (128 x 64 outputs per wave, 8 waves per CU), operands rotating through several random fragment sets in registers.
 #include <hip/hip_runtime.h>
 #include <cstdio>
@@ -56,6 +57,32 @@ __global__ __launch_bounds__(512) void k16(float* out, int iters, int zero) {
   float sum = 0; for (int a = 0; a < 4; a++) for (int b = 0; b < 8; b++) for (int i = 0; i < 4; i++) sum += acc[a][b][i];
   out[blockIdx.x * 512 + threadIdx.x] = sum;
 }
+// e4m3 operands of v_mfma_scale_f32_32x32x64_f8f6f4 (unit scales): random bytes with the top exponent bit cleared (no NaN)
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+__device__ inline i32x8 rnd_frag8(uint32_t seed, int zero) {
+  i32x8 v;
+  for (int i = 0; i < 8; i++) v[i] = zero ? 0 : (int)(hash(seed + i) & 0xbfbfbfbfu);
+  return v;
+}
+template <int SETS>
+__global__ __launch_bounds__(512) void kf8(float* out, int iters, int zero) {
+  i32x8 p[SETS][4], q[SETS][2];  // one set covers k = 64: 4 token fragments of 32 rows, 2 feature fragments
+  const uint32_t s0 = (blockIdx.x * 512 + threadIdx.x) * 128;
+  for (int s = 0; s < SETS; s++) { for (int i = 0; i < 4; i++) p[s][i] = rnd_frag8(s0 + s * 48 + i * 8, zero); for (int i = 0; i < 2; i++) q[s][i] = rnd_frag8(s0 + s * 48 + 32 + i * 8, zero); }
+  f32x16 acc[2][4];
+  for (int a = 0; a < 2; a++) for (int b = 0; b < 4; b++) for (int i = 0; i < 16; i++) acc[a][b][i] = 0;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int s = 0; s < SETS; s++)
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++)
+          acc[a][b] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(q[s][a], p[s][b], acc[a][b], 0, 0, 0, 127, 0, 127);
+  }
+  float sum = 0; for (int a = 0; a < 2; a++) for (int b = 0; b < 4; b++) for (int i = 0; i < 16; i++) sum += acc[a][b][i];
+  out[blockIdx.x * 512 + threadIdx.x] = sum;
+}
 int main() {
   float* out; hipMalloc(&out, 1024 * 512 * 4);
   hipEvent_t e0, e1; hipEventCreate(&e0); hipEventCreate(&e1);
@@ -70,6 +97,9 @@ int main() {
       hipEventRecord(e0); k16<2><<<256, 512>>>(out, iters, zero); hipEventRecord(e1); hipEventSynchronize(e1); hipEventElapsedTime(&ms, e0, e1);
       fl = 256.0 * 8 * iters * 2 * 32 * 16384.0;
       printf("mfma 16x16x32 %s: %8.2f ms %7.1f TFLOP/s\n", zero ? "zeros " : "random", ms, fl / ms / 1e9);
+      hipEventRecord(e0); kf8<2><<<256, 512>>>(out, iters, zero); hipEventRecord(e1); hipEventSynchronize(e1); hipEventElapsedTime(&ms, e0, e1);
+      fl = 256.0 * 8 * iters * 2 * 8 * 131072.0;
+      printf("mfma fp8 32x32x64 (scaled) %s: %8.2f ms %7.1f TFLOP/s\n", zero ? "zeros " : "random", ms, fl / ms / 1e9);
     }
   }
   return 0;
