@@ -272,6 +272,14 @@ int smoe_tr_compact(const uint8_t* keep, const void* probs, int dtype, const int
  *          [128 g + 32 b, 128 g + 32 b + 32) of row r: the smallest power of two with amax / scale <= 448 */
 int smoe_mx_quantize(const void* src, int64_t src_stride, int64_t R, int C, void* q, void* scales, void* stream);
 
+/* Workspace of the two fp8 operators whose token operand is gathered (smoe_up_projection_forward_fp8 and
+ * smoe_down_projection_backward_fp8, contraction size K = H): the tile map of smoe_gemm_workspace_bytes followed by
+ * room for the gathered rows' scale words in grouped order, (K / 128) * TK words, which the operator fills with a
+ * small kernel of its own so that the GEMM reads two cache lines of scales per 64 rows instead of 64.  Both operators
+ * also accept the smaller smoe_gemm_workspace_bytes(TK, E): the GEMM then fetches every row's scale word through the
+ * gather index (same results, a few per cent slower).  No counterpart in the reference. */
+size_t smoe_fp8_gemm_workspace_bytes(int64_t TK, int E, int K);
+
 /* As smoe_up_projection_forward with x and W1 given in the quantised form above:
  *   xq (T, H) bytes + x_scales (H/128, T); w1q (E, N1, H) bytes contiguous + w1_scales (H/128, E*N1)
  *   z (TK, N1) bf16 or NULL; y1 (TK, I) bf16 or NULL;

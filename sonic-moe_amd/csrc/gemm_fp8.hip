@@ -79,6 +79,7 @@ struct Fp8Params {
   const uint32_t* p_scales;
   int64_t p_rows;    // rows of the P scale table (T or TK)
   const int32_t* gidx;
+  int scales_grouped;  // the P scale table is in grouped row order although the data rows are gathered
   const uint8_t* Q;
   int64_t q_stride_e, q_stride_row;  // bytes
   const uint32_t* q_scales;
@@ -288,8 +289,9 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
     if (r0 < C::BM) {
       int m = row0 + r0 + lane;
       m = m < row_end ? m : row_end - 1;
-      s_rsrc[j] = make_buffer_resource(p.gidx ? p.p_scales : p.p_scales + row0);
-      s_voff[j] = (p.gidx ? (uint32_t)p.gidx[m] : (uint32_t)(m - row0)) * 4u;
+      const bool by_index = p.gidx != nullptr && !p.scales_grouped;
+      s_rsrc[j] = make_buffer_resource(by_index ? p.p_scales : p.p_scales + row0);
+      s_voff[j] = (by_index ? (uint32_t)p.gidx[m] : (uint32_t)(m - row0)) * 4u;
 #ifdef SMOE_PROBE_SCALES_CONTIG
       s_voff[j] = (uint32_t)lane * 4u;
 #endif
@@ -467,7 +469,7 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_stream_kernel(const Fp8Params 
     for (int i = 0; i <= PI; i++) {
       int m = t.row0 + (i < PI ? (wave * PI + i) * C::KRPI + ln / C::KPR : wave * 32 + (ln & 31));
       m = m < t.row_end ? m : t.row_end - 1;
-      rows[i] = p.gidx ? p.gidx[m] : m - t.row0;
+      rows[i] = p.gidx && (i < PI || !p.scales_grouped) ? p.gidx[m] : m - t.row0;
     }
   };
   // Operands and scale tables are fetched through buffer resources: a lane keeps one 32-bit byte offset per load
@@ -480,10 +482,8 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_stream_kernel(const Fp8Params 
   const uint32_t ps_step = (uint32_t)p.p_rows * 4u, qs_step = (uint32_t)p.q_rows * 4u;
   auto point_p = [&](const int(&rows)[PI + 1], const StreamTile& t) {
     const int ln = opaque_lane();
-    if (!p.gidx) {
-      p_rsrc = make_buffer_resource(p.P + (int64_t)t.row0 * p.p_stride);
-      ps_rsrc = make_buffer_resource(p.p_scales + t.row0);
-    }
+    if (!p.gidx) p_rsrc = make_buffer_resource(p.P + (int64_t)t.row0 * p.p_stride);
+    if (!p.gidx || p.scales_grouped) ps_rsrc = make_buffer_resource(p.p_scales + t.row0);
 #pragma unroll
     for (int i = 0; i < PI; i++) {
       const int r = (wave * PI + i) * C::KRPI + ln / C::KPR;
@@ -804,6 +804,43 @@ extern "C" int smoe_mx_quantize(const void* src, int64_t src_stride, int64_t R, 
   return SMOE_OK;
 }
 
+// ---- scale words of a gathered token operand in grouped row order ---------------------------------------------------
+// The GEMM kernels fetch one scale word per tile row and stage.  Through the gather index that is one cache line per
+// row (64 scattered 4-byte reads per load instruction); from a table in grouped order it is two lines per 64 rows.
+// dst[g][m] = src[g][gidx[m]] for the KB 128-element blocks of the contraction.
+__global__ __launch_bounds__(256) void gather_scale_rows_kernel(const uint32_t* __restrict__ src, int64_t src_rows,
+                                                                const int32_t* __restrict__ gidx,
+                                                                uint32_t* __restrict__ dst, int64_t TK, int KB) {
+  const int64_t m = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (m >= TK) return;
+  const int64_t r = gidx[m];
+  for (int g = 0; g < KB; g++) dst[(int64_t)g * TK + m] = src[(int64_t)g * src_rows + r];
+}
+
+static size_t grouped_scales_offset(int64_t TK, int E) { return (tile_map_bytes(TK, E) + 255) / 256 * 256; }
+
+// Points p at a grouped copy of its token operand's scale table in the workspace behind the tile map, if the workspace
+// is large enough for it (smoe_fp8_gemm_workspace_bytes); otherwise the kernels go through the gather index.
+static int group_token_scales(Fp8Params& p, void* workspace, size_t workspace_bytes, int64_t TK, int E,
+                              hipStream_t st) {
+  const int KB = p.Kdim / 128;
+  const size_t at = grouped_scales_offset(TK, E);
+  if (p.gidx == nullptr || workspace_bytes < at + (size_t)KB * TK * sizeof(uint32_t)) return SMOE_OK;
+  uint32_t* dst = (uint32_t*)((char*)workspace + at);
+  hipLaunchKernelGGL(gather_scale_rows_kernel, dim3((unsigned)ceil_div(TK, 256)), dim3(256), 0, st, p.p_scales,
+                     p.p_rows, p.gidx, dst, TK, KB);
+  SMOE_LAUNCH_CHECK();
+  p.p_scales = dst;
+  p.p_rows = TK;
+  p.scales_grouped = 1;
+  return SMOE_OK;
+}
+
+extern "C" size_t smoe_fp8_gemm_workspace_bytes(int64_t TK, int E, int K) {
+  if (TK < 0 || E < 1 || K < 128) return 0;
+  return grouped_scales_offset(TK, E) + (size_t)(K / 128) * TK * sizeof(uint32_t);
+}
+
 static int check_fp8(int64_t TK, int Kdim, int N, int E, const void* ws, size_t ws_bytes, const char* who) {
   SMOE_REQUIRE(TK >= 0 && TK < (1ll << 31), SMOE_ERR_INVALID, "%s: TK out of range", who);
   SMOE_REQUIRE(E >= 1, SMOE_ERR_INVALID, "%s: E must be >= 1", who);
@@ -857,6 +894,8 @@ extern "C" int smoe_up_projection_forward_fp8(const void* xq, const void* x_scal
   p.yq_scales = (uint32_t*)y1q_scales;
   p.yq_rows = TK;
   p.I = I;
+  rc = group_token_scales(p, workspace, workspace_bytes, TK, E, (hipStream_t)stream);
+  if (rc) return rc;
   return launch_fp8_up(activation, p, off, workspace, TK, E, (hipStream_t)stream);
 }
 
@@ -935,6 +974,8 @@ extern "C" int smoe_down_projection_backward_fp8(const void* doutq, const void* 
   p.sidx = s_scatter_idx;
   p.ds_partial = ds_partial;
   hipStream_t st = (hipStream_t)stream;
+  rc = group_token_scales(p, workspace, workspace_bytes, TK, E, st);
+  if (rc) return rc;
   rc = launch_fp8_dz(activation, p, off, workspace, TK, E, st);
   if (rc) return rc;
   return launch_ds_finalize(ds_partial, p.ds_cols, s_scatter_idx, ds, TK, st);

@@ -31,6 +31,7 @@ _SIGNATURES = {
     "smoe_routing_metadata_static_capacity": (c_size_t, []),
     "smoe_routing_metadata_static": (c_int, [_P, _P, _L, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P]),
     "smoe_gemm_workspace_bytes": (c_size_t, [_L, _I]),
+    "smoe_fp8_gemm_workspace_bytes": (c_size_t, [_L, _I, _I]),
     "smoe_up_projection_forward": (
         c_int,
         [_P, _P, _L, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],

@@ -13,8 +13,9 @@ from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
 from ..utils import expert_major_strides
 
 
-def _gemm_workspace(TK: int, E: int, device, stream_id: int) -> torch.Tensor:
-    """Tile-map scratch of one grouped-GEMM launch.  It comes from PyTorch's caching allocator, which orders its reuse
+def _gemm_workspace(TK: int, E: int, device, stream_id: int, fp8_gathered_k: int = 0) -> torch.Tensor:
+    """Tile-map scratch of one grouped-GEMM launch (`fp8_gathered_k`: contraction size of an fp8 operator with a gathered
+    token operand, whose workspace also holds the gathered rows' scale words).  It comes from PyTorch's caching allocator, which orders its reuse
     on the CURRENT stream, and the routing / combine kernels around the GEMM run on the current stream as well: a
     GEMM launched on any other stream would race with both, so that is refused."""
     current = _lib.current_stream_handle()
@@ -24,7 +25,10 @@ def _gemm_workspace(TK: int, E: int, device, stream_id: int) -> torch.Tensor:
             "torch.cuda.current_stream().cuda_stream (a MoE module keeps the stream it was constructed under in "
             "`.stream_id`; set it again when calling the module under another stream)"
         )
-    n = _lib.lib().smoe_gemm_workspace_bytes(TK, E)
+    if fp8_gathered_k:
+        n = _lib.lib().smoe_fp8_gemm_workspace_bytes(TK, E, fp8_gathered_k)
+    else:
+        n = _lib.lib().smoe_gemm_workspace_bytes(TK, E)
     return torch.empty(max(n, 16), dtype=torch.uint8, device=device)
 
 

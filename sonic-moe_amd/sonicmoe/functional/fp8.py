@@ -151,7 +151,7 @@ def _up_projection_forward_fp8(
     N1 = 2 * I if is_glu_activation else I
     assert w1q.shape == (E * N1, H) and x_scales.shape == (H // 128, T) and w1_scales.shape == (H // 128, E * N1)
     assert z is None or (z.shape == (TK, N1) and z.is_contiguous())
-    ws = _gemm_workspace(TK, E, xq.device, stream_id)
+    ws = _gemm_workspace(TK, E, xq.device, stream_id, fp8_gathered_k=H)
     rc = _lib.lib().smoe_up_projection_forward_fp8(
         _lib.ptr(xq),
         _lib.ptr(x_scales),
@@ -288,7 +288,7 @@ def _down_projection_backward_fp8(
     assert ds.dtype == torch.float32 and ds.numel() == TK and topk_scores.dtype == torch.float32
     ncols = _lib.lib().smoe_dz_partial_cols(I)
     ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
-    ws = _gemm_workspace(TK, E, z.device, stream_id)
+    ws = _gemm_workspace(TK, E, z.device, stream_id, fp8_gathered_k=H)
     rc = _lib.lib().smoe_down_projection_backward_fp8(
         _lib.ptr(doutq),
         _lib.ptr(dout_scales),

@@ -73,6 +73,9 @@ def test_argument_checks_return_status_codes(lib):
     assert lib.smoe_switch_loss_workspace_bytes(32768, 128) == 256 * 128 * 4
     # workspace size queries are pure host functions
     assert lib.smoe_gemm_workspace_bytes(262144, 128) > 0
+    # the fp8 operators with a gathered token operand: tile map + (K / 128) * TK scale words in grouped order
+    assert lib.smoe_fp8_gemm_workspace_bytes(262144, 128, 4096) >= lib.smoe_gemm_workspace_bytes(262144, 128) + 32 * 262144 * 4
+    assert lib.smoe_fp8_gemm_workspace_bytes(262144, 128, 64) == 0
     assert lib.smoe_routing_metadata_workspace_bytes(262144, 128) == 2 * 128 * 256 * 4
     assert lib.smoe_dz_partial_cols(1024) >= 4
 

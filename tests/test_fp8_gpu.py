@@ -57,8 +57,20 @@ def _problem(dev, T, H, I, E, K, seed, activation="swiglu", skew=0.0, empty=()):
     (2048, 1024, 512, 16, 4, "geglu", False, 0.5, ()),
     (1024, 512, 384, 4, 2, "gelu", True, 0.0, ()),         # not gated: z has I columns
 ])
-def test_fp8_forward_operators(dev, T, H, I, E, K, activation, with_bias, skew, empty):
+@pytest.mark.parametrize("kernel", ["stream", "stream_few_workgroups", "tile_per_workgroup", "stream_small_workspace",
+                                    "tile_per_workgroup_small_workspace"])
+def test_fp8_forward_operators(dev, tuning, monkeypatch, kernel, T, H, I, E, K, activation, with_bias, skew, empty):
+    """Both kernels behind the fp8 forward operators: the tile stream (default; with 8 workgroups every workgroup walks
+    through several tiles and tile switches) and the one-tile-per-workgroup kernel; each also with the workspace that has
+    no room for the gathered rows' scale words (the kernels then fetch them through the gather index)."""
     from sonicmoe.functional import fp8
+
+    tuning("gemm_stream", 0 if kernel.startswith("tile_per_workgroup") else 1)
+    if kernel == "stream_few_workgroups":
+        tuning("gemm_stream_grid", 8)
+    if kernel.endswith("small_workspace"):
+        full = fp8._gemm_workspace
+        monkeypatch.setattr(fp8, "_gemm_workspace", lambda TK, E, device, stream_id, fp8_gathered_k=0: full(TK, E, device, stream_id))
 
     glu, N1, w1, w2, b1, b2, x, md, meta = _problem(dev, T, H, I, E, K, T + H, activation, skew, empty)
     if not with_bias:
@@ -137,9 +149,15 @@ def test_transposing_quantiser_bit_exact(dev, E, R, C):
     (1024, 512, 384, 4, 2, "gelu", 0.0, ()),         # not gated: z and dz have I columns
     (1024, 512, 192, 4, 2, "reglu", 0.0, ()),        # I is not a multiple of 128 (N1 is)
 ])
-def test_fp8_backward_operators(dev, T, H, I, E, K, activation, skew, empty):
-    """dz / y1s / ds from quantised dout and W2^T, dz quantised in the epilogue, dx from that and W1^T."""
+@pytest.mark.parametrize("workspace", ["grouped_scales", "tile_map_only"])
+def test_fp8_backward_operators(dev, monkeypatch, workspace, T, H, I, E, K, activation, skew, empty):
+    """dz / y1s / ds from quantised dout and W2^T, dz quantised in the epilogue, dx from that and W1^T; with and without
+    room in the workspace for dout's scale words in grouped order."""
     from sonicmoe.functional import backward, fp8
+
+    if workspace == "tile_map_only":
+        full = fp8._gemm_workspace
+        monkeypatch.setattr(fp8, "_gemm_workspace", lambda TK, E, device, stream_id, fp8_gathered_k=0: full(TK, E, device, stream_id))
 
     glu, N1, w1, w2, _, _, x, md, meta = _problem(dev, T, H, I, E, K, 3 * T + H, activation, skew, empty)
     TK = T * K
