@@ -143,7 +143,7 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
                         2.0 * T * H * E, T * H * 2 + T * E * 2 + T * K * 8))
         if gemms_only:
             ops = [o for o in ops if o[2] and "router_gemm" not in o[0]]
-        if H % 128 == 0 and I % 128 == 0 and only is None and not gemms_only:
+        if H % 128 == 0 and I % 128 == 0 and (only is None or only.startswith("fp8:")) and not gemms_only:
             # fp8 forward (config 5 = this shape with block-scaled e4m3 operands): quantisers and the two fp8 GEMMs
             from sonicmoe.functional import fp8
 
@@ -202,9 +202,13 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
 SINGLE_KERNEL_OPS = {
     "up_projection_forward": "varlen_m_stream_kernel<up-projection forward>",
     "down_projection_forward": "varlen_m_stream_kernel<down-projection forward>",
-    "down_projection_backward(dz only)": "varlen_m_kernel<dz>",
+    "down_projection_backward(dz only)": "varlen_m_stream_kernel<dz>",
     "up_projection_backward(dW1 only)": "varlen_k_kernel<dW1>",
     "up_projection_backward(dx only)": "varlen_m_stream_kernel<dx_expanded>",
+    "fp8:up_projection_forward(+quantised y1)": "fp8_stream_kernel<up-projection forward>",
+    "fp8:down_projection_forward": "fp8_stream_kernel<down-projection forward>",
+    "fp8:down_projection_backward(dz, +quantised dz)": "fp8_varlen_m_kernel<dz>",
+    "fp8:up_projection_backward(dx)": "fp8_stream_kernel<dx_expanded>",
 }
 
 
@@ -473,7 +477,7 @@ def main():
     rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, t["x"], t["wr"], t["w1"], t["w2"], t["dout"],
                                                                     max(5, a.steps // 2))
     # dominant kernel = the single grouped-GEMM launch with the largest average duration
-    single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS]
+    single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS and not r["op"].startswith("fp8:")]
     roofline = None
     if single:
         dom = max(single, key=lambda r: r["ms"])

@@ -58,6 +58,8 @@ const char* smoe_last_error(void);
  *   "gemm_stream"          SMOE_GEMM_STREAM          1: token-grouped GEMMs run as tile streams (default); 0: one tile
  *                                                    per workgroup
  *   "gemm_stream_grid"     SMOE_GEMM_STREAM_GRID     workgroups of a tile-stream launch; 0 = one per compute unit
+ *   "dz_stream"            SMOE_DZ_STREAM            1 (default) the bf16 dz kernel is a tile stream too; 0 one tile per
+ *                                                    workgroup for dz alone
  *   "varlen_k_tile_order"  SMOE_VARLEN_K_TILE_ORDER  2 blocked (default), 0 round-robin, 1 whole experts per XCD */
 int smoe_set_tuning(const char* name, int value);
 

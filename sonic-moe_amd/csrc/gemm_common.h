@@ -819,7 +819,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
   constexpr int ZSW = ZL < 16 ? ZL - 1 : 15;  // row swizzle of the staged z chunks
   constexpr int NB = TM / BR, RB = BR / FR;   // batches of BR rows; fragment rows per batch
   static_assert(BR % FR == 0 && ZN >= 1 && YN >= 1, "a batch is whole fragment rows and whole load instructions");
-  static_assert(PF == 1 || PF == 2, "one or two batches of z are prefetched");
+  static_assert(PF >= 1 && PF <= 4, "one to four batches of z are prefetched");
   char* ybuf = zbuf + BR * ZB;
   const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
   const int zlimit = ZW * a.N;
@@ -834,8 +834,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
       dst[it] = *(const u32x4*)(a.zin + (int64_t)m * a.zin_stride + zcol_c);
     }
   };
-  fetch_z(0, zreg[0]);
-  if constexpr (NB > 1 && PF > 1) fetch_z(1, zreg[1]);
+  static_for<(PF < NB ? PF : NB)>([&](auto i_c) { fetch_z(decltype(i_c)::value, zreg[decltype(i_c)::value]); });
   ring_idle();  // the staging areas lie in the ring: every wave must be done reading it
   static_for<NB>([&](auto blk_c) {
     constexpr int blk = decltype(blk_c)::value;

@@ -170,7 +170,10 @@ def test_tile_streams(dev, tuning, grid, T, H, I, E, K, skew, empty):
     ds = torch.empty(TK, dtype=torch.float32, device=dev)
     bwd._down_projection_backward(dout, zb, w2.permute(1, 2, 0), dw2, dz2, ds, None, None, s_flat, off, None, gidx, sidx,
                                   stream, True, "swiglu")
-    _, _, _, dw2_ref = M.down_projection_backward(dout, zb, w2, s_flat, off, gidx, sidx, round_dtype=torch.bfloat16)
+    dz_ref, _, ds_ref, dw2_ref = M.down_projection_backward(dout, zb, w2, s_flat, off, gidx, sidx,
+                                                            round_dtype=torch.bfloat16)
+    assert rel_l2(dz2, dz_ref) < TOL      # the dz kernel is a tile stream as well
+    assert rel_l2(ds, ds_ref) < 2e-3
     assert rel_l2(dw2.permute(2, 0, 1), dw2_ref) < TOL
     for e in empty:
         assert bool((dw2[..., e] == 0).all())
@@ -183,7 +186,8 @@ def test_tile_streams(dev, tuning, grid, T, H, I, E, K, skew, empty):
     assert torch.equal(z1, z) and torch.equal(y11, y1)
 
 
-@pytest.mark.parametrize("knob,value", [("gemm_stream", 0), ("varlen_k_tile_order", 0), ("varlen_k_tile_order", 1)])
+@pytest.mark.parametrize("knob,value", [("gemm_stream", 0), ("dz_stream", 0), ("varlen_k_tile_order", 0),
+                                        ("varlen_k_tile_order", 1)])
 def test_kernel_selection_knobs(dev, tuning, knob, value):
     """The alternative kernels / tile orders a tuning knob selects give the same results as the defaults
     (bit-identical: the arithmetic of a tile does not depend on who computes it or when)."""
@@ -197,6 +201,8 @@ def test_kernel_selection_knobs(dev, tuning, knob, value):
     off, gidx, sidx = (md[k] for k in ("expert_frequency_offset", "x_gather_idx", "s_scatter_idx"))
     stream = torch.cuda.current_stream().cuda_stream
     dz = torch.randn(TK, 2 * I, generator=g).to(torch.bfloat16).to(dev)
+    dout = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    s_flat = torch.from_numpy(scores).to(dev).view(-1)
 
     def run():
         z = torch.empty(TK, 2 * I, dtype=torch.bfloat16, device=dev)
@@ -207,12 +213,16 @@ def test_kernel_selection_knobs(dev, tuning, knob, value):
         dw1 = torch.empty(E, 2 * I, H, dtype=torch.bfloat16, device=dev).permute(1, 2, 0)
         dxe = torch.empty(TK, H, dtype=torch.bfloat16, device=dev)
         bwd._up_projection_backward(x, w1.permute(1, 2, 0), dxe, dw1, dz, None, off, None, gidx, sidx, True, stream)
-        return z, y1, y2, dw1, dxe
+        dz2 = torch.empty_like(z)
+        ds = torch.empty(TK, dtype=torch.float32, device=dev)
+        bwd._down_projection_backward(dout, z, w2.permute(1, 2, 0), None, dz2, ds, None, None, s_flat, off, None, gidx,
+                                      sidx, stream, True, "swiglu")
+        return z, y1, y2, dw1, dxe, dz2, ds
 
     base = run()
     tuning(knob, value)
     other = run()
-    for name, a, b in zip(["z", "y1", "y2", "dw1", "dx_expanded"], base, other):
+    for name, a, b in zip(["z", "y1", "y2", "dw1", "dx_expanded", "dz", "ds"], base, other):
         assert torch.equal(a, b), name
 
 
