@@ -2,6 +2,8 @@
 torch.autograd through the restated forward (fp64), special cases that reduce to library routines, closed forms."""
 
 import numpy as np
+import math
+
 import pytest
 import torch
 import torch.nn.functional as F
@@ -90,6 +92,17 @@ def test_activation_forms(activation):
     dz, y_again = M.activation_backward(z, dy, activation)
     torch.testing.assert_close(dz, gz, rtol=1e-10, atol=1e-12)
     torch.testing.assert_close(y_again, y, rtol=1e-12, atol=1e-12)
+
+
+def test_gelu_is_the_erf_form():
+    """Known answers: gelu(t) = t * Phi(t) with the normal distribution function (tables: Phi(1) = 0.8413447460685429,
+    Phi(2) = 0.9772498680518208, Phi(-0.5) = 0.3085375387259869).  The tanh approximation the reference's fused kernels
+    use (grouped_gemm.py:432-433) gives 0.841192 at t = 1: the two forms differ from the fourth digit on."""
+    t = torch.tensor([[1.0, 2.0, -0.5, 0.0]], dtype=D)
+    want = torch.tensor([[0.8413447460685429, 2 * 0.9772498680518208, -0.5 * 0.3085375387259869, 0.0]], dtype=D)
+    torch.testing.assert_close(M.activation_forward(t, "gelu"), want, rtol=1e-12, atol=1e-14)
+    tanh_form = 0.5 * (1.0 + math.tanh(math.sqrt(2.0 / math.pi) * (1.0 + 0.044715)))
+    assert abs(float(M.activation_forward(t, "gelu")[0, 0]) - tanh_form) > 1e-4
 
 
 @pytest.mark.parametrize("activation", ALL_ACTIVATIONS)
