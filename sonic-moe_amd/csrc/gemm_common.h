@@ -820,18 +820,37 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
   constexpr int NB = TM / BR, RB = BR / FR;   // batches of BR rows; fragment rows per batch
   static_assert(BR % FR == 0 && ZN >= 1 && YN >= 1, "a batch is whole fragment rows and whole load instructions");
   static_assert(PF >= 1 && PF <= 4, "one to four batches of z are prefetched");
+  // N is a multiple of 64 (checked by the entry points): a wave tile of at most 64 columns lies wholly inside or wholly
+  // outside the matrix, so the column test of the score-gradient sum is made once per row instead of once per value
+  constexpr bool COLS_WHOLE = 64 % TN == 0;
   char* ybuf = zbuf + BR * ZB;
   const int zr = lane / ZL, zc = lane % ZL, yr = lane / YL, yc = lane % YL;
   const int zlimit = ZW * a.N;
   const int zcol = ZW * a.n_base + zc * 8;  // first z column of this lane's 16-byte chunk
   const int zcol_c = zcol <= zlimit - 8 ? zcol : zlimit - 8;
+  // Global addresses are a wave-uniform anchor (the wave's first row; for the loads, which clamp rows behind the
+  // expert's end to its last row, the earlier of the two) plus a 32-bit byte offset whose per-lane part is fixed for the
+  // whole epilogue: an access costs at most two vector instructions of address arithmetic instead of a 64-bit
+  // multiply-add, and the epilogue is bound by its vector instructions (a wave evaluates the activation's derivative for
+  // TM x TN values per tile).
+  const int m_base = __builtin_amdgcn_readfirstlane(a.m_base), m_last = __builtin_amdgcn_readfirstlane(a.row_end) - 1;
+  const int m_anchor = m_base < m_last ? m_base : m_last;
+  const int rows_left = m_last + 1 - m_base;  // valid rows from the wave's first row on (may be <= 0)
+  const uint32_t zin_rb = (uint32_t)a.zin_stride * 2u, dz_rb = (uint32_t)a.dz_stride * 2u, y_rb = (uint32_t)a.y1s_stride * 2u;
+  const char* zin_anchor = (const char*)(a.zin + (int64_t)m_anchor * a.zin_stride);
+  char* dz_anchor = (char*)(a.dz + (int64_t)m_base * a.dz_stride);
+  char* y_anchor = (char*)(a.y1s + (int64_t)m_base * a.y1s_stride);
+  const uint32_t zin_lane = (uint32_t)zr * zin_rb + (uint32_t)zcol_c * 2u;
+  const uint32_t zin_max = (uint32_t)(m_last - m_anchor) * zin_rb + (uint32_t)zcol_c * 2u;
+  const uint32_t dz_lane = (uint32_t)zr * dz_rb + (uint32_t)zcol * 2u;
+  const uint32_t y_lane = (uint32_t)yr * y_rb + (uint32_t)(a.n_base + yc * 8) * 2u;
   u32x4 zreg[PF][ZN];
   auto fetch_z = [&](int blk, u32x4(&dst)[ZN]) {
 #pragma unroll
     for (int it = 0; it < ZN; it++) {
-      int m = a.m_base + blk * BR + it * ZR + zr;
-      m = m < a.row_end ? m : a.row_end - 1;
-      dst[it] = *(const u32x4*)(a.zin + (int64_t)m * a.zin_stride + zcol_c);
+      uint32_t off = zin_lane + (uint32_t)(blk * BR + it * ZR + (m_base - m_anchor)) * zin_rb;
+      off = off < zin_max ? off : zin_max;
+      dst[it] = *(const u32x4*)(zin_anchor + off);
     }
   };
   static_for<(PF < NB ? PF : NB)>([&](auto i_c) { fetch_z(decltype(i_c)::value, zreg[decltype(i_c)::value]); });
@@ -867,7 +886,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
             float f, fp;
             pointwise_grad<PW>(g, f, fp);
             const float y1v = f * u;
-            if (a.n_base + il + q < a.N) dsum += dy * y1v;
+            if (COLS_WHOLE || a.n_base + il + q < a.N) dsum += dy * y1v;
             const float sd = sc * dy;
             dzv[q] = pack_bf16x2(sd * u * fp, sd * f);
             ys[q] = sc * y1v;
@@ -882,7 +901,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
             const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
             float f, fp;
             pointwise_grad<PW>(t, f, fp);
-            if (a.n_base + il + q < a.N) dsum += dy * f;
+            if (COLS_WHOLE || a.n_base + il + q < a.N) dsum += dy * f;
             dzf[q] = sc * dy * fp;
             ys[q] = sc * f;
           }
@@ -891,6 +910,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
         u32x2 yv = {pack_bf16x2(ys[0], ys[1]), pack_bf16x2(ys[2], ys[3])};
         epi_park_y<YB>(ybuf, mrow, il * 2, yv);
       });
+      if (COLS_WHOLE && a.n_base >= a.N) dsum = 0.f;
       // the 64 / FR lanes that share a token row hold disjoint columns: add their partial sums
       dsum += __shfl_xor(dsum, 32, 64);
       if constexpr (FR == 16) dsum += __shfl_xor(dsum, 16, 64);
@@ -900,9 +920,10 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
     for (int it = 0; it < ZN; it++) {
       const int r = it * ZR + zr;
       const u32x4 v = *(const u32x4*)(zbuf + r * ZB + ((zc ^ (r & ZSW)) << 4));
-      const int mm = a.m_base + blk * BR + r;
-      const bool live = mm < a.row_end && zcol < zlimit;
-      if (live) *(u32x4*)(a.dz + (int64_t)mm * a.dz_stride + zcol) = v;
+      const int r0 = blk * BR + it * ZR;  // first row of this store instruction, relative to the wave's first row
+      const int mm = m_base + r0 + zr;
+      const bool live = zr < rows_left - r0 && zcol < zlimit;
+      if (live) *(u32x4*)(dz_anchor + (size_t)r0 * dz_rb + dz_lane) = v;
       if constexpr (QUANT) {
         // 32 columns = the 16-byte chunks of 4 consecutive lanes
         float x[8];
@@ -932,8 +953,8 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
     for (int it = 0; it < YN; it++) {
       const int r = it * YR + yr;
       const u32x4 v = *(const u32x4*)(ybuf + r * YB + ((yc ^ ((r >> 1) & (YL < 8 ? YL - 1 : 7))) << 4));
-      const int mm = a.m_base + blk * BR + r, col = a.n_base + yc * 8;
-      if (mm < a.row_end && col < a.N) *(u32x4*)(a.y1s + (int64_t)mm * a.y1s_stride + col) = v;
+      const int r0 = blk * BR + it * YR;
+      if (yr < rows_left - r0 && a.n_base + yc * 8 < a.N) *(u32x4*)(y_anchor + (size_t)r0 * y_rb + y_lane) = v;
     }
   });
 }
