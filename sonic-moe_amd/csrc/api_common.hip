@@ -21,7 +21,7 @@ void set_error(const char* fmt, ...) {
 
 namespace {
 std::once_flag g_tuning_once;
-Tuning g_tuning = {1, 0, 2, 1};
+Tuning g_tuning = {1, 0, 2, 1, 1};
 
 struct Knob {
   const char* name;
@@ -34,6 +34,7 @@ const Knob g_knobs[] = {
     {"gemm_stream_grid", "SMOE_GEMM_STREAM_GRID", &Tuning::gemm_stream_grid, 0, 1 << 30, 0},
     {"varlen_k_tile_order", "SMOE_VARLEN_K_TILE_ORDER", &Tuning::varlen_k_tile_order, 0, 2, 2},
     {"dz_stream", "SMOE_DZ_STREAM", &Tuning::dz_stream, 0, 1, 1},
+    {"gemm_asm", "SMOE_GEMM_ASM", &Tuning::gemm_asm, 0, 1, 1},
 };
 
 void read_tuning_env() {

@@ -50,6 +50,12 @@ SMOE_DEV i32x4 make_buffer_resource(const void* base) {
   r[3] = 0x00020000;                                                        // 32-bit untyped data
   return r;
 }
+// with a range limit: loads whose byte offset (per-lane + wave-uniform) reaches `bytes` are dropped by the hardware
+SMOE_DEV i32x4 make_buffer_resource(const void* base, uint32_t bytes) {
+  i32x4 r = make_buffer_resource(base);
+  r[2] = (int32_t)bytes;
+  return r;
+}
 SMOE_DEV void buffer_load16_to_lds(i32x4 rsrc, uint32_t voff, uint32_t soff, uint32_t lds_wave_base) {
   asm volatile("s_mov_b32 m0, %3\n\ts_nop 0\n\tbuffer_load_dwordx4 %0, %1, %2 offen lds"
                :
@@ -685,77 +691,125 @@ SMOE_DEV void forward_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::
   }
 }
 
-// The same epilogue 32 rows at a time, parked in a caller-chosen LDS region of 32 padded rows
+// One 32-row batch of that epilogue, parked in a caller-chosen LDS region of 32 padded rows
 // (32 * EpiLayout<TN>::ROW_BYTES bytes per wave): for kernels whose ring keeps running during the epilogue.
-template <class Mma, int TM, int TN, bool WITH_ACT, int ACT>
-SMOE_DEV void forward_epilogue_rows(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* region, int lane,
-                                    const FwdEpilogueArgs& a) {
+// frag(fn_c, sub_c) names the accumulator fragment (fn, sub) of the batch (sub = fragment row inside the batch);
+// m0 = first grouped row of the batch.
+template <class Mma, int TN, bool WITH_ACT, int ACT, class FragAt>
+SMOE_DEV void forward_epilogue_batch(FragAt&& frag, char* region, int lane, const FwdEpilogueArgs& a, int m0) {
   using AL = AccLayout<Mma>;
   constexpr int FR = Mma::FR, FN = TN / FR, QPF = AL::QPF, RB = 32 / FR;  // RB fragment rows make a 32-row batch
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
   using LZ = EpiLayout<TN>;
   using LY = EpiLayout<TN / 2>;
-  const bool with_bias = a.bias != nullptr;
   const int lrow = AL::row(lane);
-  static_for<TM / 32>([&](auto blk_c) {
-    constexpr int blk = decltype(blk_c)::value;
-    if (with_bias) {  // re-read per batch (a few cached words) rather than held in registers across the batches
+  if (a.bias != nullptr) {  // re-read per batch (a few cached words) rather than held in registers across the batches
+    static_for<FN * QPF>([&](auto q_c) {
+      constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+      int n = a.n_base + fn * FR + AL::col(rg, lane);
+      n = n <= a.N - 4 ? n : a.N - 4;
+      const u32x2 b = *(const u32x2*)(a.bias + n);
+      static_for<RB>([&](auto sub_c) {
+        auto& f = frag(std::integral_constant<int, fn>{}, sub_c);
+        f[4 * rg + 0] += bf16_lo(b[0]);
+        f[4 * rg + 1] += bf16_hi(b[0]);
+        f[4 * rg + 2] += bf16_lo(b[1]);
+        f[4 * rg + 3] += bf16_hi(b[1]);
+      });
+    });
+  }
+  if (!WITH_ACT || a.out0 != nullptr) {
+    static_for<RB>([&](auto sub_c) {
+      constexpr int sub = decltype(sub_c)::value;
       static_for<FN * QPF>([&](auto q_c) {
         constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-        int n = a.n_base + fn * FR + AL::col(rg, lane);
-        n = n <= a.N - 4 ? n : a.N - 4;
-        const u32x2 b = *(const u32x2*)(a.bias + n);
-        static_for<RB>([&](auto sub_c) {
-          constexpr int fm = blk * RB + decltype(sub_c)::value;
-          acc[fn][fm][4 * rg + 0] += bf16_lo(b[0]);
-          acc[fn][fm][4 * rg + 1] += bf16_hi(b[0]);
-          acc[fn][fm][4 * rg + 2] += bf16_lo(b[1]);
-          acc[fn][fm][4 * rg + 3] += bf16_hi(b[1]);
-        });
+        const auto& f = frag(std::integral_constant<int, fn>{}, sub_c);
+        u32x2 v = {pack_bf16x2(f[4 * rg + 0], f[4 * rg + 1]), pack_bf16x2(f[4 * rg + 2], f[4 * rg + 3])};
+        *(u32x2*)(region + (sub * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
       });
-    }
-    const int m0 = a.m_base + blk * 32;
-    if (!WITH_ACT || a.out0 != nullptr) {
+    });
+    epilogue_flush<32, TN>(region, lane, a.out0, a.out0_stride, m0, a.row_end, a.n_base, a.N);
+  }
+  if constexpr (WITH_ACT && GLU) {
+    if (a.out1 != nullptr) {
       static_for<RB>([&](auto sub_c) {
-        constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
+        constexpr int sub = decltype(sub_c)::value;
         static_for<FN * QPF>([&](auto q_c) {
           constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-          u32x2 v = {pack_bf16x2(acc[fn][fm][4 * rg + 0], acc[fn][fm][4 * rg + 1]),
-                     pack_bf16x2(acc[fn][fm][4 * rg + 2], acc[fn][fm][4 * rg + 3])};
+          const auto& f = frag(std::integral_constant<int, fn>{}, sub_c);
+          const float g0 = f[4 * rg + 0], u0 = f[4 * rg + 1];
+          const float g1 = f[4 * rg + 2], u1 = f[4 * rg + 3];
+          const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
+          *(uint32_t*)(region + (sub * FR + lrow) * LY::ROW_BYTES + (fn * FR + AL::col(rg, lane))) = v;
+        });
+      });
+      epilogue_flush<32, TN / 2>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base / 2, a.N / 2);
+    }
+  } else if constexpr (WITH_ACT) {
+    if (a.out1 != nullptr) {
+      static_for<RB>([&](auto sub_c) {
+        constexpr int sub = decltype(sub_c)::value;
+        static_for<FN * QPF>([&](auto q_c) {
+          constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
+          const auto& f = frag(std::integral_constant<int, fn>{}, sub_c);
+          u32x2 v = {pack_bf16x2(pointwise<PW>(f[4 * rg + 0]), pointwise<PW>(f[4 * rg + 1])),
+                     pack_bf16x2(pointwise<PW>(f[4 * rg + 2]), pointwise<PW>(f[4 * rg + 3]))};
           *(u32x2*)(region + (sub * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
         });
       });
-      epilogue_flush<32, TN>(region, lane, a.out0, a.out0_stride, m0, a.row_end, a.n_base, a.N);
+      epilogue_flush<32, TN>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base, a.N);
     }
-    if constexpr (WITH_ACT && GLU) {
-      if (a.out1 != nullptr) {
-        static_for<RB>([&](auto sub_c) {
-          constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
-          static_for<FN * QPF>([&](auto q_c) {
-            constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-            const float g0 = acc[fn][fm][4 * rg + 0], u0 = acc[fn][fm][4 * rg + 1];
-            const float g1 = acc[fn][fm][4 * rg + 2], u1 = acc[fn][fm][4 * rg + 3];
-            const uint32_t v = pack_bf16x2(pointwise<PW>(g0) * u0, pointwise<PW>(g1) * u1);
-            *(uint32_t*)(region + (sub * FR + lrow) * LY::ROW_BYTES + (fn * FR + AL::col(rg, lane))) = v;
-          });
-        });
-        epilogue_flush<32, TN / 2>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base / 2, a.N / 2);
-      }
-    } else if constexpr (WITH_ACT) {
-      if (a.out1 != nullptr) {
-        static_for<RB>([&](auto sub_c) {
-          constexpr int sub = decltype(sub_c)::value, fm = blk * RB + sub;
-          static_for<FN * QPF>([&](auto q_c) {
-            constexpr int fn = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-            u32x2 v = {pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 0]), pointwise<PW>(acc[fn][fm][4 * rg + 1])),
-                       pack_bf16x2(pointwise<PW>(acc[fn][fm][4 * rg + 2]), pointwise<PW>(acc[fn][fm][4 * rg + 3]))};
-            *(u32x2*)(region + (sub * FR + lrow) * LZ::ROW_BYTES + (fn * FR + AL::col(rg, lane)) * 2) = v;
-          });
-        });
-        epilogue_flush<32, TN>(region, lane, a.out1, a.out1_stride, m0, a.row_end, a.n_base, a.N);
-      }
-    }
+  }
+}
+
+// The whole wave tile, 32 rows at a time, from accumulators the compiler holds
+template <class Mma, int TM, int TN, bool WITH_ACT, int ACT>
+SMOE_DEV void forward_epilogue_rows(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* region, int lane,
+                                    const FwdEpilogueArgs& a) {
+  constexpr int RB = 32 / Mma::FR;
+  static_for<TM / 32>([&](auto blk_c) {
+    constexpr int blk = decltype(blk_c)::value;
+    forward_epilogue_batch<Mma, TN, WITH_ACT, ACT>(
+        [&](auto fn_c, auto sub_c) -> typename Mma::Acc& {
+          return acc[decltype(fn_c)::value][blk * RB + decltype(sub_c)::value];
+        },
+        region, lane, a, a.m_base + blk * 32);
+  });
+}
+
+// ---- accumulators of the hand-scheduled loop -------------------------------------------------------------------------
+// The tile loop of tile_loop_gen.h leaves its results in the accumulation registers a[0:255], which the compiler does
+// not know about: they are read out four at a time, in program order (volatile), while the epilogue runs.
+template <int R>
+SMOE_DEV f32x4 agpr_read4() {
+  f32x4 r;
+  asm volatile(
+      "v_accvgpr_read_b32 %0, a[%4]\n\tv_accvgpr_read_b32 %1, a[%5]\n\tv_accvgpr_read_b32 %2, a[%6]\n\t"
+      "v_accvgpr_read_b32 %3, a[%7]"
+      : "=v"(r[0]), "=v"(r[1]), "=v"(r[2]), "=v"(r[3])
+      : "n"(R), "n"(R + 1), "n"(R + 2), "n"(R + 3));
+  return r;
+}
+
+// forward epilogue of a wave tile whose FN x FM fragments of 16 x 16 sit in a[4 * (fn * FM + fm) ..]
+template <class Mma, int TM, int TN, bool WITH_ACT, int ACT>
+SMOE_DEV void forward_epilogue_rows_agpr(char* region, int lane, const FwdEpilogueArgs& a) {
+  static_assert(Mma::ACC_REGS == 4, "four accumulator registers per fragment");
+  constexpr int FR = Mma::FR, FN = TN / FR, FM = TM / FR, RB = 32 / FR;
+  static_for<TM / 32>([&](auto blk_c) {
+    constexpr int blk = decltype(blk_c)::value;
+    f32x4 loc[FN][RB];
+    static_for<RB>([&](auto sub_c) {
+      constexpr int sub = decltype(sub_c)::value;
+      static_for<FN>([&](auto fn_c) {
+        constexpr int fn = decltype(fn_c)::value;
+        loc[fn][sub] = agpr_read4<4 * (fn * FM + blk * RB + sub)>();
+      });
+    });
+    forward_epilogue_batch<Mma, TN, WITH_ACT, ACT>(
+        [&](auto fn_c, auto sub_c) -> f32x4& { return loc[decltype(fn_c)::value][decltype(sub_c)::value]; }, region,
+        lane, a, a.m_base + blk * 32);
   });
 }
 
@@ -776,6 +830,8 @@ struct DzEpilogueArgs {
   const int32_t* sidx;
   float* ds_partial;  // (rows, ds_cols) fp32: this wave writes column ds_col, sum_i dy1 * y1 over its columns
   int ds_cols, ds_col;
+  int ds_pad_col1;  // 1 + a second column of this wave's rows that is written as zero (0: none): the table's pitch is
+                    // fixed by the widest kernel, a kernel with fewer waves per tile fills the columns it has no sum for
   int m_base, row_end;  // first grouped row of this wave's tile, end of the expert's rows
   int n_base, N;        // first dy1 column of this wave's tile, number of dy1 columns (I)
   // with QUANT: dz once more as e4m3 bytes (rows, ZW * N) with one power-of-two scale per 32 columns, the operand format
@@ -806,9 +862,10 @@ SMOE_DEV int mx_scale_exponent(float amax) {
   return k < 0 ? 0 : (k > 254 ? 254 : k);
 }
 
-template <class Mma, int TM, int TN, int ACT, int PF = 2, bool QUANT = false, int BR = 32, class RingIdle>
-SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* zbuf, int lane,
-                          const DzEpilogueArgs& a, RingIdle&& ring_idle) {
+// frag(fn_c, fm_c) hands out the accumulator fragment (fn, fm) of the wave tile, by reference or by value; every
+// fragment is asked for once per register group, in the order the batches consume them.
+template <class Mma, int TM, int TN, int ACT, int PF = 2, bool QUANT = false, int BR = 32, class FragAt, class RingIdle>
+SMOE_DEV void dz_epilogue_at(FragAt&& frag, char* zbuf, int lane, const DzEpilogueArgs& a, RingIdle&& ring_idle) {
   using AL = AccLayout<Mma>;
   constexpr bool GLU = act_is_glu(ACT);
   constexpr int PW = act_pointwise(ACT);
@@ -876,12 +933,13 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
         const int zbyte = il * 2 * ZW;                // their z bytes inside the staged row
         char* zaddr = zbuf + mrow * ZB + (((zbyte >> 4) ^ (mrow & ZSW)) << 4) + (zbyte & 15);
         float ys[4];
+        const auto& dyf = frag(std::integral_constant<int, fn>{}, std::integral_constant<int, fm>{});
         if constexpr (GLU) {
           const u32x4 zz = *(const u32x4*)zaddr;
           u32x4 dzv;
 #pragma unroll
           for (int q = 0; q < 4; q++) {
-            const float dy = acc[fn][fm][4 * rg + q];
+            const float dy = dyf[4 * rg + q];
             const float g = bf16_lo(zz[q]), u = bf16_hi(zz[q]);
             float f, fp;
             pointwise_grad<PW>(g, f, fp);
@@ -897,7 +955,7 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
           float dzf[4];
 #pragma unroll
           for (int q = 0; q < 4; q++) {
-            const float dy = acc[fn][fm][4 * rg + q];
+            const float dy = dyf[4 * rg + q];
             const float t = (q & 1) ? bf16_hi(zz[q >> 1]) : bf16_lo(zz[q >> 1]);
             float f, fp;
             pointwise_grad<PW>(t, f, fp);
@@ -914,7 +972,10 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
       // the 64 / FR lanes that share a token row hold disjoint columns: add their partial sums
       dsum += __shfl_xor(dsum, 32, 64);
       if constexpr (FR == 16) dsum += __shfl_xor(dsum, 16, 64);
-      if (mvalid && lane < FR) a.ds_partial[(int64_t)m * a.ds_cols + a.ds_col] = dsum;
+      if (mvalid && lane < FR) {
+        a.ds_partial[(int64_t)m * a.ds_cols + a.ds_col] = dsum;
+        if (a.ds_pad_col1 > 0) a.ds_partial[(int64_t)m * a.ds_cols + a.ds_pad_col1 - 1] = 0.f;
+      }
     });
 #pragma unroll
     for (int it = 0; it < ZN; it++) {
@@ -959,6 +1020,15 @@ SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], 
   });
 }
 
+// accumulators the compiler holds
+template <class Mma, int TM, int TN, int ACT, int PF = 2, bool QUANT = false, int BR = 32, class RingIdle>
+SMOE_DEV void dz_epilogue(typename Mma::Acc (&acc)[TN / Mma::FR][TM / Mma::FR], char* zbuf, int lane,
+                          const DzEpilogueArgs& a, RingIdle&& ring_idle) {
+  dz_epilogue_at<Mma, TM, TN, ACT, PF, QUANT, BR>(
+      [&](auto fn_c, auto fm_c) -> const typename Mma::Acc& { return acc[decltype(fn_c)::value][decltype(fm_c)::value]; },
+      zbuf, lane, a, ring_idle);
+}
+
 // ---- tuning knobs ----------------------------------------------------------------------------------------------
 // Read from the environment ONCE, at the first launch that asks (variable = "SMOE_" + the upper-cased field name);
 // smoe_set_tuning() overrides a knob afterwards (tests walk through the alternative kernels with it).
@@ -967,6 +1037,7 @@ struct Tuning {
   int gemm_stream_grid;     // workgroups of the tile-stream kernels; 0 (default) = one per compute unit
   int varlen_k_tile_order;  // 2 blocked (default), 0 single tiles round-robin over the XCDs, 1 whole experts per XCD
   int dz_stream;            // 1: dz runs as a tile stream too (with gemm_stream); 0: one tile per workgroup
+  int gemm_asm;             // 1: the tile streams run on the hand-scheduled four-wavefront loop (tile_loop_gen.h)
 };
 const Tuning& tuning();
 

@@ -334,8 +334,8 @@ static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st) {
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
               void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* order,
-              const int32_t* gidx, const int32_t* sidx, int64_t TK, int H, int I, int E, int activation,
-              void* workspace, hipStream_t st);
+              const int32_t* gidx, const int32_t* sidx, int64_t T, int64_t TK, int H, int I, int E,
+              int activation, void* workspace, hipStream_t st);
 int launch_dx(const void* dz, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row, void* dx_expanded,
               const int32_t* off, const int32_t* order, int64_t TK, int H, int N1, int E, void* workspace,
               hipStream_t st);
@@ -374,14 +374,13 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
                "down_projection_backward: null pointer");
   SMOE_REQUIRE(TK == 0 || !db2 || (scores && s_scatter_idx), SMOE_ERR_INVALID,
                "down_projection_backward: db2 needs scores and s_scatter_idx");
-  (void)T;
   SMOE_REQUIRE_ALIGNED("down_projection_backward", dout, z, w2, b2, dw2, db2, dz, y1s);
   SMOE_REQUIRE(stride8(w2_stride_e) && stride8(w2_stride_row) && stride8(dw2_stride_e) && stride8(dw2_stride_row),
                SMOE_ERR_UNSUPPORTED, "down_projection_backward: weight strides must be multiples of 8 elements");
   hipStream_t st = (hipStream_t)stream;
   if (TK > 0 && dz) {
     rc = launch_dz(dout, z, w2, w2_stride_e, w2_stride_row, dz, y1s, ds_partial, scores, off, expert_schedule_order,
-                   x_gather_idx, s_scatter_idx, TK, H, I, E, activation, workspace, st);
+                   x_gather_idx, s_scatter_idx, T, TK, H, I, E, activation, workspace, st);
     if (rc) return rc;
     rc = launch_ds_finalize(ds_partial, smoe_dz_partial_cols(I), s_scatter_idx, ds, TK, st);
     if (rc) return rc;

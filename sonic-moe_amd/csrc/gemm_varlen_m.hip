@@ -6,6 +6,7 @@
 //   down-proj activation grad P = dout rows gathered,              Q = W2[e] (MN-major)  -> dz, y1s, ds partials
 //   up-proj activation grad  P = dz rows,                          Q = W1[e] (MN-major)  -> dx_expanded
 #include "gemm_common.h"
+#include "tile_loop_gen.h"
 
 namespace smoe {
 
@@ -482,6 +483,235 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
       S_total, acc, issue_p, issue_q, load, issued_p, issued_q, first_boundary, tile_end);
 }
 
+// ---- the tile stream on the hand-scheduled loop ----------------------------------------------------------------------
+// Four wavefronts (one per SIMD) as 2 x 2 wave tiles of 128 x 128; the contraction of a tile is the single assembly
+// statement of tile_loop_gen.h, which leaves the tile in a[0:255].  This kernel does what happens once per tile: picks
+// the tiles, forms the per-lane source offsets of the current and the next tile for the two load streams (the streams
+// run across tile boundaries), and runs the epilogue out of the accumulation registers.  Source offsets are 32-bit byte
+// offsets from the token tensor's start and from the expert's weight matrix (the host checks that they fit).
+typedef int32_t i32x2 __attribute__((ext_vector_type(2)));
+typedef int32_t i32x8 __attribute__((ext_vector_type(8)));
+typedef int32_t i32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int DS_COLS_PER_TILE = 4;  // pitch of the score-gradient partials per 256-column tile
+
+template <class C, int ROLE, int ACT>
+__global__ __launch_bounds__(C::NT) void varlen_m_asm_kernel(const VarlenMParams p) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  using Mma = typename C::Mma;
+  constexpr int BN = C::BN, FN = C::FN, BK = C::BK;
+  static_assert(C::NW == 4 && C::WM == 2 && C::FM == SMOE_TL_FM && FN == SMOE_TL_FN && C::P_INSTR == SMOE_TL_P_INSTR &&
+                    C::Q_INSTR == SMOE_TL_Q_INSTR && Mma::FR == 16 && BK == 64,
+                "the generated loop is written for this tile shape");
+  const uint32_t smem_base = lds_address(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave % C::WM, wn = wave / C::WM;
+
+  const StreamTiles tiles(p.tm, p.off, p.n_tiles, BN);
+  int64_t vb = blockIdx.x;
+  StreamTile cur = tiles.at(vb);
+  if (!cur.valid) return;
+  StreamTile nxt = tiles.at(vb += gridDim.x);
+  bool more = nxt.valid;  // a tile follows the current one
+  if (!more) nxt = cur;   // the streams always run on: past the last tile they re-read it into slots nobody reads
+  StreamTile nn = tiles.at(vb += gridDim.x);
+  bool more2 = nn.valid;
+  if (!more2) nn = nxt;
+
+  auto opaque_lane = [&]() {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
+  // source rows of a tile's token operand: token indices (gathered) or the grouped rows themselves
+  auto token_rows = [&](const StreamTile& t, int(&rows)[C::P_INSTR]) {
+    const int ln = opaque_lane();
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) {
+      int m = t.row0 + (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
+      m = m < t.row_end ? m : t.row_end - 1;
+      rows[i] = p.gidx ? p.gidx[m] : m;
+    }
+  };
+  const uint32_t p_row_bytes = (uint32_t)p.p_stride * 2u, q_row_bytes = (uint32_t)p.q_stride_row * 2u;
+  auto point_p = [&](const int(&rows)[C::P_INSTR]) {
+    const int ln = opaque_lane();
+    i32x8 v;
+#pragma unroll
+    for (int i = 0; i < C::P_INSTR; i++) {
+      const int r = (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
+      v[i] = (int32_t)((uint32_t)rows[i] * p_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK, C::FR>(r)) << 4));
+    }
+    return v;
+  };
+  auto point_q = [&](const StreamTile& t) {
+    const int ln = opaque_lane();
+    i32x8 v;
+#pragma unroll
+    for (int i = 0; i < C::Q_INSTR; i++) {
+      if constexpr (!C::QMN) {
+        const int r = (wave * C::Q_INSTR + i) * C::KRPI + ln / C::KPR;
+        int n = t.n0 + r;
+        n = n < p.N ? n : p.N - 1;
+        v[i] = (int32_t)((uint32_t)n * q_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK, C::FR>(r)) << 4));
+      } else {
+        const int kl = (wave * C::Q_INSTR + i) * C::RPI + ln / C::LPR;
+        const int phys16 = ln % C::LPR;
+        const int log32 = (phys16 >> 1) ^ mnswz(kl);
+        int n = t.n0 + ((log32 << 1) | (phys16 & 1)) * 8;
+        n = n <= p.N - 8 ? n : p.N - 8;
+        v[i] = (int32_t)((uint32_t)kl * q_row_bytes + (uint32_t)n * 2u);
+      }
+    }
+    return v;
+  };
+  // base (48 bits) of an expert's weight matrix, as the first two words of a buffer resource
+  auto q_base = [&](const StreamTile& t) {
+    const uint64_t b = (uint64_t)(p.Q + (int64_t)t.e * p.q_stride_e);
+    i32x2 r;
+    r[0] = __builtin_amdgcn_readfirstlane((uint32_t)b);
+    r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32) & 0xffffu);
+    return r;
+  };
+  // extents: what the streams may touch (anything beyond is dropped by the range check instead of faulting)
+  const uint32_t p_bytes = (uint32_t)(p.p_rows * p.p_stride * 2);
+  const uint32_t q_bytes = C::QMN ? (uint32_t)(p.Kdim - 1) * q_row_bytes + (uint32_t)p.N * 2u
+                                  : (uint32_t)(p.N - 1) * q_row_bytes + (uint32_t)p.Kdim * 2u;
+  const i32x4 p_rsrc = make_buffer_resource(p.P, p_bytes);
+  i32x4 q_rsrc = make_buffer_resource(p.Q + (int64_t)cur.e * p.q_stride_e, q_bytes);
+
+  i32x8 pv, qv, pvn, qvn;
+  i32x2 qnb;
+  int rows_nn[C::P_INSTR];  // token rows of nn: requested one tile ahead of the offsets made from them
+  {
+    int rows[C::P_INSTR];
+    token_rows(cur, rows);
+    pv = point_p(rows);
+    qv = point_q(cur);
+    token_rows(nxt, rows);
+    pvn = point_p(rows);
+    qvn = point_q(nxt);
+    qnb = q_base(nxt);
+    token_rows(nn, rows_nn);
+  }
+
+  const int S_total = p.Kdim / BK;
+  int p_off_a[C::KSL];
+  int q_off_a[C::QMN ? 2 * FN : C::KSL];
+  fragment_offsets<C>(wm, wn, lane, p_off_a, q_off_a);
+  i32x2 poff = {p_off_a[0], p_off_a[1]};
+
+  constexpr int Q_RING = C::P_SLOTS * C::P_STAGE;
+  const uint32_t q_step = C::QMN ? (uint32_t)BK * q_row_bytes : (uint32_t)BK * 2u;
+  const uint32_t lds_p = smem_base, lds_q = smem_base + Q_RING, wave_lds = (uint32_t)wave * (C::P_INSTR * 1024);
+  const uint32_t p_end = (uint32_t)S_total * (BK * 2u), q_end = (uint32_t)S_total * q_step;
+  const uint32_t n_mid = (uint32_t)S_total - 2u;
+  // the first tile's stage 0 and the weight stage after it; the loop's entry requests P(1) and Q(2) into the "vacated"
+  // slots 0 / 0 and finds stage 0 in the slots after them
+  uint32_t p_soff = 0, q_soff = 0, p_fill = lds_p, q_fill = lds_q;
+  static_for<C::P_INSTR>([&](auto i_c) {
+    constexpr int i = decltype(i_c)::value;
+    buffer_load16_to_lds(p_rsrc, (uint32_t)pv[i], 0u, lds_p + C::P_STAGE + wave_lds + i * 1024);
+  });
+  static_for<2>([&](auto s_c) {
+    constexpr int s = decltype(s_c)::value;
+    static_for<C::Q_INSTR>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      buffer_load16_to_lds(q_rsrc, (uint32_t)qv[i], (uint32_t)s * q_step, lds_q + (1 + s) * C::Q_STAGE + wave_lds + i * 1024);
+    });
+  });
+  p_soff = BK * 2u;
+  q_soff = 2u * q_step;
+  wait_vmem_all();
+
+  constexpr int PARK = ROLE == ROLE_DZ ? DzStaging<C::TN, ACT, 16>::BYTES : 32 * EpiLayout<C::TN>::ROW_BYTES;
+  static_assert((C::NW / 2) * PARK <= C::P_STAGE && (C::NW / 2) * PARK <= C::Q_STAGE, "parking must fit into a ring slot");
+
+  for (;;) {
+    if constexpr (!C::QMN) {
+      i32x2 qoff = {q_off_a[0], q_off_a[1]};
+      SMOE_TILE_LOOP_KK(pv, qv, q_rsrc, p_soff, q_soff, p_fill, q_fill, pvn, qvn, poff, qoff, p_rsrc, qnb, p_end, q_end,
+                        q_step, n_mid, lds_p, lds_q, wave_lds);
+    } else {
+      i32x16 qoff;
+#pragma unroll
+      for (int i = 0; i < 2 * FN; i++) qoff[i] = q_off_a[i];
+      SMOE_TILE_LOOP_KM(pv, qv, q_rsrc, p_soff, q_soff, p_fill, q_fill, pvn, qvn, poff, qoff, p_rsrc, qnb, p_end, q_end,
+                        q_step, n_mid, lds_p, lds_q, wave_lds);
+    }
+    // Offsets of the tile after next, from the rows requested a tile ago.  Formed here, in front of the epilogue's
+    // stores: the wait for those rows then finds only loads outstanding.
+    const i32x8 pvn_new = point_p(rows_nn);
+    const i32x8 qvn_new = point_q(nn);
+    const i32x2 qnb_new = q_base(nn);
+
+    // waves 0, 1 park in the vacated token slot, waves 2, 3 in the vacated weight slot
+    char* region = smem + ((wave < C::NW / 2 ? p_fill : q_fill) - smem_base) + (wave & (C::NW / 2 - 1)) * PARK;
+    if constexpr (ROLE == ROLE_DZ) {
+      DzEpilogueArgs da = {};
+      da.zin = p.zin;
+      da.zin_stride = p.zin_stride;
+      da.dz = p.out0;
+      da.dz_stride = p.out0_stride;
+      da.y1s = p.out1;
+      da.y1s_stride = p.out1_stride;
+      da.scores = p.scores;
+      da.sidx = p.sidx;
+      da.ds_partial = p.ds_partial;
+      da.ds_cols = p.ds_cols;
+      // the table has the pitch of the eight-wave kernels (four columns per tile): two sums, two zeros
+      da.ds_col = (cur.n0 / BN) * DS_COLS_PER_TILE + wn;
+      da.ds_pad_col1 = da.ds_col + C::WN + 1;
+      da.m_base = cur.row0 + wm * C::TM;
+      da.row_end = cur.row_end;
+      da.n_base = cur.n0 + wn * C::TN;
+      da.N = p.N;
+      dz_epilogue_at<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) ? 2 : 1, false, 16>(
+          [&](auto fn_c, auto fm_c) { return agpr_read4<SMOE_TL_ACC(decltype(fn_c)::value, decltype(fm_c)::value)>(); },
+          region, opaque_lane(), da, [] {});
+    } else {
+      FwdEpilogueArgs ea;
+      ea.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
+      ea.out0 = p.out0;
+      ea.out0_stride = p.out0_stride;
+      ea.out1 = p.out1;
+      ea.out1_stride = p.out1_stride;
+      ea.m_base = cur.row0 + wm * C::TM;
+      ea.row_end = cur.row_end;
+      ea.n_base = cur.n0 + wn * C::TN;
+      ea.N = p.N;
+      forward_epilogue_rows_agpr<Mma, C::TM, C::TN, ROLE == ROLE_UP_FWD, ACT>(region, opaque_lane(), ea);
+    }
+    if (!more) break;
+    cur = nxt;
+    nxt = nn;
+    more = more2;
+    nn = tiles.at(vb += gridDim.x);
+    more2 = nn.valid;
+    if (!more2) nn = nxt;
+    token_rows(nn, rows_nn);
+    pvn = pvn_new;
+    qvn = qvn_new;
+    qnb = qnb_new;
+    wait_lds_all();  // this wave has read its parked rows back; the loop's entry barrier then frees the two slots
+  }
+  wait_vmem_all();  // the streams ran ahead into ring slots nobody reads any more: let those loads land before the end
+}
+
+// the four-wavefront shape of the hand-scheduled loop: 2 x 2 wave tiles of 128 x 128
+template <bool QMN>
+using AsmCfg = Cfg<256, 256, 2, 2, QMN, 64, 2>;
+
+// 32-bit byte offsets: the tile streams address the token operand from the tensor's start when it is gathered (all of
+// them on the hand-scheduled loop) and the weight operand from the expert's matrix
+static bool offsets_fit32(const VarlenMParams& p, bool qmn, bool all_rows) {
+  const int64_t lim = 0xffffffffll;
+  if ((p.gidx != nullptr || all_rows) && p.p_rows * p.p_stride * 2 > lim) return false;
+  const int64_t q_rows = qmn ? p.Kdim : p.N;
+  return p.q_stride_row > 0 && q_rows * p.q_stride_row * 2 <= lim;
+}
+
 template <class C, int ROLE, int ACT>
 static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace, int64_t TK, int E, hipStream_t st) {
   static LdsLimitOnce lds_limit;
@@ -490,23 +720,19 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
     const int rc_attr = lds_limit.ensure((const void*)kern, C::SMEM);
     if (rc_attr) return rc_attr;
   }
+  if (p.gidx == nullptr) p.p_rows = TK;
   p.tm = carve_tile_map(workspace, TK, E, C::BM);
   int rc = launch_build_tile_map(off, p.order, E, C::BM, p.tm, st);
   if (rc) return rc;
   p.n_tiles = (int)ceil_div(p.N, C::BN);
+  static_assert(C::WN == DS_COLS_PER_TILE, "pitch of the score-gradient partials");
   if (ROLE == ROLE_DZ) p.ds_cols = p.n_tiles * C::WN;
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
   {
     const Tuning& tune = tuning();
-    // the tile-stream kernel addresses a gathered token operand with 32-bit byte offsets from the tensor's start
-    const bool offsets_fit = p.gidx == nullptr || p.p_rows * p.p_stride * 2 <= 0xffffffffll;
-    if (tune.gemm_stream && (ROLE != ROLE_DZ || tune.dz_stream) && p.Kdim >= 3 * C::BK && offsets_fit) {
-      static LdsLimitOnce lds_limit_stream;
-      auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
-      const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
-      if (rc_s) return rc_s;
+    if (tune.gemm_stream && (ROLE != ROLE_DZ || tune.dz_stream) && p.Kdim >= 3 * C::BK && offsets_fit32(p, C::QMN, false)) {
       int cus = 0;
       const int rc_cu = device_compute_units(&cus);
       if (rc_cu) return rc_cu;
@@ -515,6 +741,21 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
       if (tune.gemm_stream_grid > 0) sgrid = ((int64_t)tune.gemm_stream_grid + 7) / 8 * 8;
       if (sgrid < 8) sgrid = 8;
       if (sgrid > grid) sgrid = grid;
+      using CA = AsmCfg<C::QMN>;
+      static_assert(CA::BM == C::BM && CA::BN == C::BN, "both shapes walk the same tile map");
+      if (tune.gemm_asm && offsets_fit32(p, C::QMN, true)) {
+        static LdsLimitOnce lds_limit_asm;
+        auto akern = varlen_m_asm_kernel<CA, ROLE, ACT>;
+        const int rc_a = lds_limit_asm.ensure((const void*)akern, CA::SMEM);
+        if (rc_a) return rc_a;
+        hipLaunchKernelGGL(akern, dim3((unsigned)sgrid), dim3(CA::NT), CA::SMEM, st, p);
+        SMOE_LAUNCH_CHECK();
+        return SMOE_OK;
+      }
+      static LdsLimitOnce lds_limit_stream;
+      auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
+      const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
+      if (rc_s) return rc_s;
       hipLaunchKernelGGL(skern, dim3((unsigned)sgrid), dim3(C::NT), C::SMEM, st, p);
       SMOE_LAUNCH_CHECK();
       return SMOE_OK;
@@ -640,14 +881,14 @@ namespace smoe {
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
               void* y1s, float* ds_partial, const float* scores, const int32_t* off, const int32_t* order,
-              const int32_t* gidx, const int32_t* sidx, int64_t TK, int H, int I, int E, int activation,
-              void* workspace, hipStream_t st) {
+              const int32_t* gidx, const int32_t* sidx, int64_t T, int64_t TK, int H, int I, int E,
+              int activation, void* workspace, hipStream_t st) {
   const int zw = act_is_glu(activation) ? 2 : 1;
   VarlenMParams p = {};
   p.P = (const uint16_t*)dout;
   p.p_stride = H;
   p.gidx = gidx;
-  p.p_rows = TK;  // an upper bound of the number of dout rows
+  p.p_rows = T;  // the range of gidx
   p.Q = (const uint16_t*)w2;  // W2[e] is (H, I): k = h rows, n = i contiguous
   p.q_stride_e = w2_stride_e;
   p.q_stride_row = w2_stride_row;

@@ -1,0 +1,358 @@
+"""Generator of the hand-scheduled main loop of the grouped GEMMs (gfx950, one wavefront per SIMD).
+
+    python sonic-moe_amd/csrc/gen_tile_loop.py            # rewrites csrc/tile_loop_gen.h
+
+The loop is ONE inline-assembly statement per output tile: every matrix instruction, LDS fragment read, direct-to-LDS
+load, wait and barrier of a 256 x 256 tile's contraction is placed here, in program order, for a workgroup of four
+wavefronts (2 x 2 wave tiles of 128 tokens x 128 features, 256 accumulator registers in a[0:255]).  The C++ kernel
+around it (varlen_m_asm_kernel in gemm_varlen_m.hip) owns everything that happens once per tile: which tile, the
+per-lane source offsets, the epilogue.
+
+Pipeline (stage = 64 of the contraction = two k-slices of 32; token operand P: ring of 2 LDS slots, weight operand Q:
+ring of 3):
+
+    entry    barrier (the epilogue of the previous tile parked rows in the two vacated slots); request the next stage of
+             either stream into those slots; read k-slice 0 of stage 0 into fragment set A
+    stage s  k-slice 0: 64 MFMAs on set A; between them the reads of k-slice 1 into set B, then the LDS addresses of
+                        stage s+1
+             wait until this wave's loads of stage s+1 have landed (vmcnt) and its reads have returned (lgkmcnt);
+             barrier: stage s+1 is complete in LDS and nobody reads the slots of stage s any more
+             k-slice 1: 64 MFMAs on set B; between them the reads of (s+1, k-slice 0) into set A and the loads
+                        P(s+2), Q(s+3) into the slots stage s has just vacated
+    last     k-slice 1 has nothing to read or request: the next tile's first stages were requested earlier (the streams
+             run across tile boundaries), its slots are left to the epilogue
+
+A stream that has requested the tile's last stage moves on to the next tile's offsets (pvn / qvn / next expert base).
+
+Everything about register numbers and LDS geometry the C++ side needs is emitted into the header as constants and as
+the operand list of the statement, so the two cannot drift apart; tests/test_tile_loop_gen.py replays the address
+arithmetic of this file on the host and checks the committed header against the generator.
+"""
+
+from __future__ import annotations
+
+import sys
+from pathlib import Path
+
+# ---- geometry (must match Cfg<256, 256, 2, 2, QMN, 64> in gemm_varlen_m.hip) ------------------------------------------
+BM = BN = 256
+BK = 64
+NW = 4
+TM = TN = 128
+FR = 16  # v_mfma_f32_16x16x32_bf16
+KSTEP = 32
+FM = TM // FR
+FN = TN // FR
+P_STAGE = BM * BK * 2
+Q_STAGE = BN * BK * 2
+P_SLOTS, Q_SLOTS = 2, 3
+P_INSTR = P_STAGE // 1024 // NW
+Q_INSTR = Q_STAGE // 1024 // NW
+KROW = BK * 2  # bytes per row of a K-major stage
+ROWB = BN * 2  # bytes per contraction row of an MN-major stage
+
+# ---- register map -----------------------------------------------------------------------------------------------------
+# accumulators: fragment (fn, fm) = a[4 * (fn * FM + fm) .. + 3]
+def acc_reg(fn: int, fm: int) -> int:
+    return 4 * (fn * FM + fm)
+
+
+V_SET = (0, 64)  # fragment sets A, B: 8 weight fragments of 4 registers, then 8 token fragments
+V_PV, V_QV, V_PVN, V_QVN = 128, 136, 144, 152  # per-lane source offsets of the two streams: current tile, next tile
+V_POFF = 160  # p_off[2]: fragment read offsets inside a slot, k-slice 0 / 1
+V_QOFF = 162  # K-major: q_off[2]; MN-major: q_off[16] (fragment fn, half h -> 2 * fn + h)
+V_PRA = 178  # read addresses of the stage being read (offset + slot), same shapes
+V_QRA = 180
+V_LAST = 195
+
+S_PRSRC, S_QRSRC, S_QNB = 40, 44, 48
+S_PSOFF, S_QSOFF, S_PEND, S_QEND, S_QSTEP, S_NMID = 50, 51, 52, 53, 54, 55
+S_PFILL, S_QFILL, S_LDSP, S_LDSQ, S_WLDS = 56, 57, 58, 59, 60
+S_PCUR, S_QCUR, S_PFW, S_QFW, S_CNT, S_T0 = 61, 62, 63, 64, 65, 66
+S_LAST = 66
+
+
+def qfrag(setno: int, q: int) -> int:
+    return V_SET[setno] + 4 * q
+
+
+def pfrag(setno: int, p: int) -> int:
+    return V_SET[setno] + 32 + 4 * p
+
+
+class Emitter:
+    def __init__(self) -> None:
+        self.lines: list[str] = []
+        self.nlabel = 0
+
+    def __call__(self, s: str) -> None:
+        self.lines.append(s)
+
+    def label(self, stem: str) -> str:
+        self.nlabel += 1
+        return f"L{stem}{self.nlabel}_%="
+
+
+def mfma(setno: int, idx: int, fresh: bool) -> str:
+    fn, fm = idx // FM, idx % FM
+    a = acc_reg(fn, fm)
+    q, p = qfrag(setno, fn), pfrag(setno, fm)
+    c = "0" if fresh else f"a[{a}:{a + 3}]"
+    return f"v_mfma_f32_16x16x32_bf16 a[{a}:{a + 3}], v[{q}:{q + 3}], v[{p}:{p + 3}], {c}"
+
+
+def fragment_reads(setno: int, ks: int, qmn: bool) -> list[str]:
+    """LDS reads of k-slice ks of the stage the read addresses point at, into fragment set setno."""
+    out = []
+    for q in range(FN):
+        r = qfrag(setno, q)
+        if not qmn:
+            out.append(f"ds_read_b128 v[{r}:{r + 3}], v{V_QRA + ks} offset:{q * FR * KROW}")
+        else:
+            off = ks * KSTEP * ROWB
+            out.append(f"ds_read_b64_tr_b16 v[{r}:{r + 1}], v{V_QRA + 2 * q} offset:{off}")
+            out.append(f"ds_read_b64_tr_b16 v[{r + 2}:{r + 3}], v{V_QRA + 2 * q + 1} offset:{off}")
+    for p in range(FM):
+        r = pfrag(setno, p)
+        out.append(f"ds_read_b128 v[{r}:{r + 3}], v{V_PRA + ks} offset:{p * FR * KROW}")
+    return out
+
+
+def n_qoff(qmn: bool) -> int:
+    return 2 * FN if qmn else 2
+
+
+def read_addresses(qmn: bool) -> list[str]:
+    """read address = offset inside a slot + LDS address of the slot the stream of stages is on (s_pcur / s_qcur)"""
+    out = [f"v_add_u32 v{V_PRA + k}, s{S_PCUR}, v{V_POFF + k}" for k in range(2)]
+    out += [f"v_add_u32 v{V_QRA + k}, s{S_QCUR}, v{V_QOFF + k}" for k in range(n_qoff(qmn))]
+    return out
+
+
+def next_slots() -> list[str]:
+    """the slots of the current stage become the ones to refill; move on to the slots of the next stage"""
+    return [
+        f"s_add_u32 s{S_PFW}, s{S_PCUR}, s{S_WLDS}",
+        f"s_add_u32 s{S_QFW}, s{S_QCUR}, s{S_WLDS}",
+        f"s_mov_b32 s{S_PFILL}, s{S_PCUR}",
+        f"s_mov_b32 s{S_QFILL}, s{S_QCUR}",
+        # P: two slots, toggle
+        f"s_sub_u32 s{S_T0}, s{S_PCUR}, s{S_LDSP}",
+        f"s_xor_b32 s{S_T0}, s{S_T0}, {P_STAGE}",
+        f"s_add_u32 s{S_PCUR}, s{S_T0}, s{S_LDSP}",
+        # Q: three slots, rotate
+        f"s_add_u32 s{S_QCUR}, s{S_QCUR}, {Q_STAGE}",
+        f"s_sub_u32 s{S_T0}, s{S_QCUR}, s{S_LDSQ}",
+        f"s_cmp_ge_u32 s{S_T0}, {Q_SLOTS * Q_STAGE}",
+        f"s_cselect_b32 s{S_T0}, {Q_SLOTS * Q_STAGE}, 0",
+        f"s_sub_u32 s{S_QCUR}, s{S_QCUR}, s{S_T0}",
+    ]
+
+
+def load_pair(which: str, i: int) -> tuple[str, str]:
+    """(set M0, direct-to-LDS load) of this wave's i-th load of a stage of stream `which`"""
+    if which == "p":
+        return (f"s_add_u32 m0, s{S_PFW}, {i * 1024}",
+                f"buffer_load_dwordx4 v{V_PV + i}, s[{S_PRSRC}:{S_PRSRC + 3}], s{S_PSOFF} offen lds")
+    return (f"s_add_u32 m0, s{S_QFW}, {i * 1024}",
+            f"buffer_load_dwordx4 v{V_QV + i}, s[{S_QRSRC}:{S_QRSRC + 3}], s{S_QSOFF} offen lds")
+
+
+def advance_stream(em: Emitter, which: str) -> list[str]:
+    """a stage of the stream has been requested: move along the contraction; behind the tile's last stage switch to
+    the next tile's offsets"""
+    lab = em.label("adv")
+    if which == "p":
+        out = [f"s_add_u32 s{S_PSOFF}, s{S_PSOFF}, {KROW}", f"s_cmp_lg_u32 s{S_PSOFF}, s{S_PEND}",
+               f"s_cbranch_scc1 {lab}"]
+        out += [f"v_mov_b32 v{V_PV + i}, v{V_PVN + i}" for i in range(P_INSTR)]
+        out += [f"s_mov_b32 s{S_PSOFF}, 0", f"{lab}:"]
+    else:
+        out = [f"s_add_u32 s{S_QSOFF}, s{S_QSOFF}, s{S_QSTEP}", f"s_cmp_lg_u32 s{S_QSOFF}, s{S_QEND}",
+               f"s_cbranch_scc1 {lab}"]
+        out += [f"v_mov_b32 v{V_QV + i}, v{V_QVN + i}" for i in range(Q_INSTR)]
+        out += [f"s_mov_b32 s{S_QRSRC}, s{S_QNB}", f"s_mov_b32 s{S_QRSRC + 1}, s{S_QNB + 1}",
+                f"s_mov_b32 s{S_QSOFF}, 0", f"{lab}:"]
+    return out
+
+
+def schedule(qmn: bool) -> dict:
+    """Where the non-matrix instructions of a stage go: index = the matrix instruction (0..63 of a k-slice) they follow."""
+    nreads = FM + (2 * FN if qmn else FN)
+    rstep = 1 if qmn else 2
+    k0_reads = [r * rstep for r in range(nreads)]  # reads of k-slice 1
+    k0_addr = max(k0_reads) + 2  # then the slot bookkeeping and the read addresses of the next stage
+    k1_reads = [r * rstep for r in range(nreads)]
+    # P first (its ring has one slot less, so its loads have the least time), one load per two matrix instructions;
+    # then Q, one per four
+    p_at = [1 + 2 * i for i in range(P_INSTR)]
+    q_at = [p_at[-1] + 4 + 4 * i for i in range(Q_INSTR)]
+    assert q_at[-1] + 2 < 64 and k0_addr + 4 + n_qoff(qmn) + 2 < 64
+    return dict(k0_reads=k0_reads, k0_addr=k0_addr, k1_reads=k1_reads, p_at=p_at, q_at=q_at)
+
+
+def emit_kslice(em: Emitter, setno: int, fresh: bool, extras: dict[int, list[str]]) -> None:
+    for line in extras.get(-1, []):
+        em(line)
+    for idx in range(FN * FM):
+        em(mfma(setno, idx, fresh))
+        for line in extras.get(idx, []):
+            em(line)
+
+
+def add_extra(extras: dict[int, list[str]], at: int, lines: list[str]) -> None:
+    extras.setdefault(at, []).extend(lines)
+
+
+def emit_stage(em: Emitter, qmn: bool, kind: str) -> None:
+    """kind: 'first' (accumulators start from zero, stores of the previous epilogue may be outstanding), 'mid', 'last'"""
+    sch = schedule(qmn)
+    # ---- k-slice 0 on set A (its reads were issued during the previous k-slice 1, or at the entry)
+    ex: dict[int, list[str]] = {-1: ["s_waitcnt lgkmcnt(0)"]}
+    for at, line in zip(sch["k0_reads"], fragment_reads(1, 1, qmn)):
+        add_extra(ex, at, [line])
+    if kind != "last":
+        # all reads that use the old addresses have been issued: derive the next stage's
+        slots = next_slots()
+        at = sch["k0_addr"]
+        for j in range(0, len(slots), 4):
+            add_extra(ex, at, slots[j:j + 4])
+            at += 1
+        for line in read_addresses(qmn):
+            add_extra(ex, at, [line])
+            at += 1
+    emit_kslice(em, 0, kind == "first", ex)
+    # stage s+1 has landed (only the weight stage after it may still be on its way); the reads of set B have returned
+    em(f"s_waitcnt vmcnt({0 if kind == 'first' else Q_INSTR}) lgkmcnt(0)")
+    em("s_barrier")
+    # ---- k-slice 1 on set B
+    ex = {}
+    if kind != "last":
+        for at, line in zip(sch["k1_reads"], fragment_reads(0, 0, qmn)):
+            add_extra(ex, at, [line])
+        for i, at in enumerate(sch["p_at"]):
+            m0, ld = load_pair("p", i)
+            add_extra(ex, at - 1, [m0])
+            add_extra(ex, at, [ld])
+        add_extra(ex, sch["p_at"][-1] + 1, advance_stream(em, "p"))
+        for i, at in enumerate(sch["q_at"]):
+            m0, ld = load_pair("q", i)
+            add_extra(ex, at - 1, [m0])
+            add_extra(ex, at, [ld])
+        add_extra(ex, sch["q_at"][-1] + 1, advance_stream(em, "q"))
+    emit_kslice(em, 1, False, ex)
+
+
+def emit_tile(qmn: bool) -> list[str]:
+    em = Emitter()
+    # ---- entry: refill the two slots the previous tile's last stage left (the epilogue parked rows there)
+    em("s_barrier")
+    em(f"s_add_u32 s{S_PFW}, s{S_PFILL}, s{S_WLDS}")
+    em(f"s_add_u32 s{S_QFW}, s{S_QFILL}, s{S_WLDS}")
+    for which, n in (("p", P_INSTR), ("q", Q_INSTR)):
+        for i in range(n):
+            m0, ld = load_pair(which, i)
+            em(m0)
+            em("s_nop 0")
+            em(ld)
+        for line in advance_stream(em, which):
+            em(line)
+    # stage 0 sits in the other token slot and in the weight slot after the vacated one
+    em(f"s_mov_b32 s{S_PCUR}, s{S_PFILL}")
+    em(f"s_mov_b32 s{S_QCUR}, s{S_QFILL}")
+    for line in next_slots()[4:]:
+        em(line)
+    for line in read_addresses(qmn):
+        em(line)
+    for line in fragment_reads(0, 0, qmn):
+        em(line)
+    em(f"s_mov_b32 s{S_CNT}, s{S_NMID}")
+    em("s_waitcnt lgkmcnt(0)")
+    emit_stage(em, qmn, "first")
+    top = em.label("stage")
+    em(f"{top}:")
+    emit_stage(em, qmn, "mid")
+    em(f"s_sub_u32 s{S_CNT}, s{S_CNT}, 1")
+    em(f"s_cmp_lg_u32 s{S_CNT}, 0")
+    em(f"s_cbranch_scc1 {top}")
+    emit_stage(em, qmn, "last")
+    # the slots of the last stage are the ones the epilogue may use and the next entry refills
+    em(f"s_mov_b32 s{S_PFILL}, s{S_PCUR}")
+    em(f"s_mov_b32 s{S_QFILL}, s{S_QCUR}")
+    # matrix results must not be read by the instructions that follow for 18 cycles
+    em("s_nop 15")
+    em("s_nop 7")
+    return em.lines
+
+
+# ---- the statement ------------------------------------------------------------------------------------------------------
+def vrange(lo: int, n: int) -> str:
+    return f"v{lo}" if n == 1 else f"v[{lo}:{lo + n - 1}]"
+
+
+def srange(lo: int, n: int) -> str:
+    return f"s{lo}" if n == 1 else f"s[{lo}:{lo + n - 1}]"
+
+
+def statement(name: str, qmn: bool) -> str:
+    lines = emit_tile(qmn)
+    nq = n_qoff(qmn)
+    outs = [
+        (vrange(V_PV, P_INSTR), "pv"), (vrange(V_QV, Q_INSTR), "qv"), (srange(S_QRSRC, 4), "qrsrc"),
+        (srange(S_PSOFF, 1), "psoff"), (srange(S_QSOFF, 1), "qsoff"), (srange(S_PFILL, 1), "pfill"),
+        (srange(S_QFILL, 1), "qfill"),
+    ]
+    ins = [
+        (vrange(V_PVN, P_INSTR), "pvn"), (vrange(V_QVN, Q_INSTR), "qvn"), (vrange(V_POFF, 2), "poff"),
+        (vrange(V_QOFF, nq), "qoff"), (srange(S_PRSRC, 4), "prsrc"), (srange(S_QNB, 2), "qnb"),
+        (srange(S_PEND, 1), "pend"), (srange(S_QEND, 1), "qend"), (srange(S_QSTEP, 1), "qstep"),
+        (srange(S_NMID, 1), "nmid"), (srange(S_LDSP, 1), "ldsp"), (srange(S_LDSQ, 1), "ldsq"),
+        (srange(S_WLDS, 1), "wlds"),
+    ]
+    clob = [f"v{i}" for i in range(0, 128)]
+    clob += [f"v{i}" for i in range(V_PRA, V_PRA + 2)]
+    clob += [f"v{i}" for i in range(V_QRA, V_QRA + nq)]
+    clob += [f"a{i}" for i in range(256)]
+    clob += [f"s{i}" for i in range(S_PCUR, S_LAST + 1)]
+    clob += ["scc", "memory"]
+    params = ", ".join(n for _, n in outs + ins)
+    body = [f"#define {name}({params}) \\", "  asm volatile( \\"]
+    for ln in lines:
+        body.append(f'    "{ln}\\n\\t" \\')
+    body.append("    : " + ", ".join(f'"+{{{r}}}"({n})' for r, n in outs) + " \\")
+    body.append("    : " + ", ".join(f'"{{{r}}}"({n})' for r, n in ins) + " \\")
+    # clobber list, a few per line
+    cl = [", ".join(f'"{c}"' for c in clob[i:i + 16]) for i in range(0, len(clob), 16)]
+    body.append("    : " + ", \\\n      ".join(cl) + ")")
+    return "\n".join(body)
+
+
+def header() -> str:
+    parts = [
+        "// GENERATED by gen_tile_loop.py - do not edit; regenerate with `python sonic-moe_amd/csrc/gen_tile_loop.py`.",
+        "// The hand-scheduled contraction loop of one 256 x 256 output tile for four wavefronts (one per SIMD): see the",
+        "// generator for the pipeline.  Operands are bound to fixed registers so that the text can name them.",
+        "#pragma once",
+        f"#define SMOE_TL_FM {FM}",
+        f"#define SMOE_TL_FN {FN}",
+        f"#define SMOE_TL_P_INSTR {P_INSTR}",
+        f"#define SMOE_TL_Q_INSTR {Q_INSTR}",
+        "// accumulator fragment (fn, fm) lives in a[SMOE_TL_ACC(fn, fm) .. + 3]",
+        f"#define SMOE_TL_ACC(fn, fm) (4 * ((fn) * {FM} + (fm)))",
+        "",
+        statement("SMOE_TILE_LOOP_KK", False),
+        "",
+        statement("SMOE_TILE_LOOP_KM", True),
+        "",
+    ]
+    return "\n".join(parts)
+
+
+OUT = Path(__file__).resolve().parent / "tile_loop_gen.h"
+
+if __name__ == "__main__":
+    text = header()
+    if len(sys.argv) > 1 and sys.argv[1] == "--check":
+        sys.exit(0 if OUT.exists() and OUT.read_text() == text else 1)
+    OUT.write_text(text)
+    print(OUT, len(text.splitlines()), "lines")

@@ -186,11 +186,12 @@ def test_tile_streams(dev, tuning, grid, T, H, I, E, K, skew, empty):
     assert torch.equal(z1, z) and torch.equal(y11, y1)
 
 
-@pytest.mark.parametrize("knob,value", [("gemm_stream", 0), ("dz_stream", 0), ("varlen_k_tile_order", 0),
-                                        ("varlen_k_tile_order", 1)])
+@pytest.mark.parametrize("knob,value", [("gemm_stream", 0), ("gemm_asm", 0), ("dz_stream", 0),
+                                        ("varlen_k_tile_order", 0), ("varlen_k_tile_order", 1)])
 def test_kernel_selection_knobs(dev, tuning, knob, value):
     """The alternative kernels / tile orders a tuning knob selects give the same results as the defaults
-    (bit-identical: the arithmetic of a tile does not depend on who computes it or when)."""
+    (bit-identical: the arithmetic of a tile does not depend on who computes it or when; the score gradient is a sum of
+    per-wave partial sums over the wave tile's columns, so kernels with different wave tiles agree to fp32 rounding)."""
     fwd, bwd = _ops()
     T, H, I, E, K = 4096, 1024, 512, 32, 8
     _, w1, w2 = make_weights(E, H, I, dev, seed=31)
@@ -223,7 +224,10 @@ def test_kernel_selection_knobs(dev, tuning, knob, value):
     tuning(knob, value)
     other = run()
     for name, a, b in zip(["z", "y1", "y2", "dw1", "dx_expanded", "dz", "ds"], base, other):
-        assert torch.equal(a, b), name
+        if name == "ds":
+            assert torch.allclose(a, b, rtol=1e-5, atol=1e-5), name
+        else:
+            assert torch.equal(a, b), name
 
 
 @pytest.mark.parametrize("stream_kernels", [1, 0])
