@@ -68,8 +68,8 @@ V_LAST = 195
 S_PRSRC, S_QRSRC, S_QNB = 40, 44, 48
 S_PSOFF, S_QSOFF, S_PEND, S_QEND, S_QSTEP, S_NMID = 50, 51, 52, 53, 54, 55
 S_PFILL, S_QFILL, S_LDSP, S_LDSQ, S_WLDS = 56, 57, 58, 59, 60
-S_PCUR, S_QCUR, S_PFW, S_QFW, S_CNT, S_T0 = 61, 62, 63, 64, 65, 66
-S_LAST = 66
+S_PCUR, S_QCUR, S_PFW, S_QFW, S_CNT, S_T0, S_QFWN = 61, 62, 63, 64, 65, 66, 67
+S_LAST = 67
 
 
 def qfrag(setno: int, q: int) -> int:
@@ -129,11 +129,12 @@ def read_addresses(qmn: bool) -> list[str]:
     return out
 
 
-def next_slots() -> list[str]:
-    """the slots of the current stage become the ones to refill; move on to the slots of the next stage"""
+def next_slots(qfw: int = S_QFW) -> list[str]:
+    """the slots of the current stage become the ones to refill; move on to the slots of the next stage.  qfw: where
+    this wave's weight fill address goes (loads into the previous weight slot may still be due: they use S_QFW)"""
     return [
         f"s_add_u32 s{S_PFW}, s{S_PCUR}, s{S_WLDS}",
-        f"s_add_u32 s{S_QFW}, s{S_QCUR}, s{S_WLDS}",
+        f"s_add_u32 s{qfw}, s{S_QCUR}, s{S_WLDS}",
         f"s_mov_b32 s{S_PFILL}, s{S_PCUR}",
         f"s_mov_b32 s{S_QFILL}, s{S_QCUR}",
         # P: two slots, toggle
@@ -176,19 +177,42 @@ def advance_stream(em: Emitter, which: str) -> list[str]:
     return out
 
 
+# Placement of the non-matrix instructions of a stage (index = the matrix instruction, 0..63 of a k-slice, they follow).
+# Loads issued in bursts are slower than loads issued evenly (measured: the same 16 loads of a stage bunched into the
+# first 30 matrix instructions of k-slice 1 cost 5 % of the kernel against loads 4 apart), so they are spread as far as
+# the ring allows: the token operand's over the first half of k-slice 1 (its ring has a slot less, so its loads have the
+# least time to land), the weight operand's over the rest of k-slice 1 and, Q_TAIL of them, over k-slice 0 of the NEXT
+# stage (the slot they fill was vacated at the same barrier; in program order they still follow the token loads, so the
+# counted wait is unchanged).
+SCHED = dict(
+    read_step_kk=2,  # K-major weights: one fragment read per this many matrix instructions
+    read_step_km=1,  # MN-major weights (two transpose reads per weight fragment)
+    p_first=2,
+    p_step=6,
+    q_first=50,
+    q_step=6,
+    q_tail=8,        # weight-operand loads of a stage issued during the next stage's k-slice 0 ...
+    q_tail_first=2,  # ... from this matrix instruction on,
+    q_tail_step=7,   # ... this far apart
+)
+
+
 def schedule(qmn: bool) -> dict:
-    """Where the non-matrix instructions of a stage go: index = the matrix instruction (0..63 of a k-slice) they follow."""
     nreads = FM + (2 * FN if qmn else FN)
-    rstep = 1 if qmn else 2
+    rstep = SCHED["read_step_km"] if qmn else SCHED["read_step_kk"]
     k0_reads = [r * rstep for r in range(nreads)]  # reads of k-slice 1
-    k0_addr = max(k0_reads) + 2  # then the slot bookkeeping and the read addresses of the next stage
     k1_reads = [r * rstep for r in range(nreads)]
-    # P first (its ring has one slot less, so its loads have the least time), one load per two matrix instructions;
-    # then Q, one per four
-    p_at = [1 + 2 * i for i in range(P_INSTR)]
-    q_at = [p_at[-1] + 4 + 4 * i for i in range(Q_INSTR)]
-    assert q_at[-1] + 2 < 64 and k0_addr + 4 + n_qoff(qmn) + 2 < 64
-    return dict(k0_reads=k0_reads, k0_addr=k0_addr, k1_reads=k1_reads, p_at=p_at, q_at=q_at)
+    nt = SCHED["q_tail"]
+    p_at = [SCHED["p_first"] + SCHED["p_step"] * i for i in range(P_INSTR)]
+    q_at = [SCHED["q_first"] + SCHED["q_step"] * i for i in range(Q_INSTR - nt)]
+    q_tail_at = [SCHED["q_tail_first"] + SCHED["q_tail_step"] * i for i in range(nt)]
+    # the slot bookkeeping and the read addresses of the next stage follow the last read (the tail loads keep their own
+    # copy of the fill address)
+    k0_addr = max(k0_reads) + 2
+    assert p_at[0] >= 1 and (not q_at or (q_at[0] > p_at[-1] + 1 and q_at[-1] + 2 < 64))
+    assert not q_tail_at or q_tail_at[0] >= 1
+    assert k0_addr + 4 + n_qoff(qmn) + 2 < 64 and (not q_tail_at or q_tail_at[-1] + 1 < 63)
+    return dict(k0_reads=k0_reads, k0_addr=k0_addr, k1_reads=k1_reads, p_at=p_at, q_at=q_at, q_tail_at=q_tail_at)
 
 
 def emit_kslice(em: Emitter, setno: int, fresh: bool, extras: dict[int, list[str]]) -> None:
@@ -205,15 +229,24 @@ def add_extra(extras: dict[int, list[str]], at: int, lines: list[str]) -> None:
 
 
 def emit_stage(em: Emitter, qmn: bool, kind: str) -> None:
-    """kind: 'first' (accumulators start from zero, stores of the previous epilogue may be outstanding), 'mid', 'last'"""
+    """kind: 'first' (accumulators start from zero, stores of the previous epilogue may be outstanding; the entry has
+    requested whole stages, so no loads are left over), 'mid', 'last' (requests nothing new)"""
     sch = schedule(qmn)
+    nt = len(sch["q_tail_at"])
     # ---- k-slice 0 on set A (its reads were issued during the previous k-slice 1, or at the entry)
     ex: dict[int, list[str]] = {-1: ["s_waitcnt lgkmcnt(0)"]}
     for at, line in zip(sch["k0_reads"], fragment_reads(1, 1, qmn)):
         add_extra(ex, at, [line])
+    if kind != "first" and nt:
+        # the rest of the weight stage whose first loads went out during the previous k-slice 1
+        for j, at in enumerate(sch["q_tail_at"]):
+            m0, ld = load_pair("q", Q_INSTR - nt + j)
+            add_extra(ex, at - 1, [m0])
+            add_extra(ex, at, [ld])
+        add_extra(ex, sch["q_tail_at"][-1] + 1, advance_stream(em, "q"))
     if kind != "last":
-        # all reads that use the old addresses have been issued: derive the next stage's
-        slots = next_slots()
+        # all reads that use the old slots have been issued: derive the next stage's
+        slots = next_slots(S_QFWN)
         at = sch["k0_addr"]
         for j in range(0, len(slots), 4):
             add_extra(ex, at, slots[j:j + 4])
@@ -221,6 +254,8 @@ def emit_stage(em: Emitter, qmn: bool, kind: str) -> None:
         for line in read_addresses(qmn):
             add_extra(ex, at, [line])
             at += 1
+    if kind != "last":
+        add_extra(ex, FN * FM - 1, [f"s_mov_b32 s{S_QFW}, s{S_QFWN}"])
     emit_kslice(em, 0, kind == "first", ex)
     # stage s+1 has landed (only the weight stage after it may still be on its way); the reads of set B have returned
     em(f"s_waitcnt vmcnt({0 if kind == 'first' else Q_INSTR}) lgkmcnt(0)")
@@ -239,7 +274,8 @@ def emit_stage(em: Emitter, qmn: bool, kind: str) -> None:
             m0, ld = load_pair("q", i)
             add_extra(ex, at - 1, [m0])
             add_extra(ex, at, [ld])
-        add_extra(ex, sch["q_at"][-1] + 1, advance_stream(em, "q"))
+        if nt == 0:
+            add_extra(ex, sch["q_at"][-1] + 1, advance_stream(em, "q"))
     emit_kslice(em, 1, False, ex)
 
 
