@@ -7,6 +7,7 @@
 //   dW1[e] (2I, H): R = dz rows,              S = x rows gathered
 //   dW2[e] (H, I) : R = dout rows gathered,   S = y1s rows
 #include "gemm_common.h"
+#include "tile_loop_gen.h"
 
 namespace smoe {
 
@@ -23,6 +24,7 @@ struct VarlenKParams {
   int tiles_a, tiles_b;
   int E;
   const int32_t* order;  // nullable: position i of the tile order works on expert order[i]
+  int64_t gather_rows;  // rows of the gathered operand's tensor (the range of gidx)
   int uniform_rows;  // off == nullptr: group e is rows [e * uniform_rows, min((e + 1) * uniform_rows, total_rows))
   int64_t total_rows;
   int xcd_chunked;  // tile order: 2 blocked, 1 contiguous tile range per XCD (probe: unbalanced on skewed experts), 0 round-robin
@@ -294,6 +296,110 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
                                p.NA, b0 + wb * C::TB, p.NB);
 }
 
+
+// ---- the same GEMM on the hand-scheduled loop ------------------------------------------------------------------------
+// Four wavefronts as 2 x 2 wave tiles of 128 x 128; the contraction is the weight-gradient statement of
+// tile_loop_gen.h (prologue + loop), which fetches the gather indices, forms the gathered operand's addresses and
+// leaves the tile in a[0:255].  Rows past the expert's end cost no code: the operand read in place has a buffer
+// resource that ends at the expert's last row, the gathered one gets index -1, and either way the range check of the
+// direct-to-LDS load writes zeros.  Experts with fewer than three stages of rows run three (the extra ones are all
+// zeros), so one pipeline shape serves every expert, the empty ones included.
+typedef int32_t ki32x8 __attribute__((ext_vector_type(8)));
+typedef int32_t ki32x16 __attribute__((ext_vector_type(16)));
+
+template <bool RG, bool SG>
+__global__ __launch_bounds__(256) void varlen_k_asm_kernel(const VarlenKParams p) {
+  static_assert(RG != SG, "exactly one operand is gathered");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  typedef Bf16Mma Mma;
+  constexpr int BA = 256, BB = 256, TA = 128, TB = 128, BK = 64, ROWB = 512, NINSTR = SMOE_TL_P_INSTR;
+  constexpr int FA = TA / 16, FB = TB / 16;
+  static_assert(FA == SMOE_TL_FM && FB == SMOE_TL_FN && Mma::FR == 16, "the generated loop is written for this tile shape");
+  const uint32_t smem_base = lds_address(smem);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wa = wave % 2, wb = wave / 2;
+
+  int e, ta, tb;
+  if (!decode_tile(p, (int64_t)blockIdx.x, e, ta, tb)) return;
+  if (p.order != nullptr) e = p.order[e];
+  const int a0 = ta * BA, b0 = tb * BB;
+  const int row_begin = p.off[e], row_end = p.off[e + 1];
+  const int S = (row_end - row_begin + BK - 1) / BK;
+  const uint32_t n_mid = (uint32_t)(S < 3 ? 3 : S) - 2u;
+
+  const uint32_t r_row_bytes = (uint32_t)p.r_stride * 2u, s_row_bytes = (uint32_t)p.s_stride * 2u;
+  // per-lane source offsets of the 8 loads of a stage: load i of this wave covers the token rows 2 i, 2 i + 1 of the
+  // wave's 16 (lanes 0-31 / 32-63) and 16 bytes per lane of the 512 the tile takes of a row
+  ki32x8 pv, qv;
+#pragma unroll
+  for (int i = 0; i < NINSTR; i++) {
+    const int kl = (wave * NINSTR + i) * 2 + lane / 32;
+    const int phys16 = lane % 32;
+    const int log32 = (phys16 >> 1) ^ mnswz(kl);
+    const int c = ((log32 << 1) | (phys16 & 1)) * 8;
+    int a = a0 + c, b = b0 + c;
+    a = a <= p.NA - 8 ? a : p.NA - 8;
+    b = b <= p.NB - 8 ? b : p.NB - 8;
+    pv[i] = (int32_t)((RG ? 0u : (uint32_t)kl * r_row_bytes) + (uint32_t)a * 2u);
+    qv[i] = (int32_t)((SG ? 0u : (uint32_t)kl * s_row_bytes) + (uint32_t)b * 2u);
+  }
+  // transpose-read addresses inside a slot: fragment f, half h -> 2 f + h
+  ki32x16 pra, qra;
+  {
+    const int grp = lane >> 4, i16 = lane & 15;
+    const int kk = 8 * grp + (i16 >> 2);
+#pragma unroll
+    for (int f = 0; f < 8; f++) {
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const int k = kk + 4 * h;
+        pra[f * 2 + h] = k * ROWB + ((((wa * TA) / 16 + f) ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+        qra[f * 2 + h] = k * ROWB + ((((wb * TB) / 16 + f) ^ mnswz(k)) << 5) + ((i16 & 3) << 3);
+      }
+    }
+  }
+  const int32_t half = lane >> 5;
+  // extents: the operand read in place ends at the expert's last row, the gathered one at its tensor's end
+  const i32x4 p_rsrc = make_buffer_resource(p.R, RG ? (uint32_t)(p.gather_rows * p.r_stride * 2) : (uint32_t)row_end * r_row_bytes);
+  const i32x4 q_rsrc = make_buffer_resource(p.S, SG ? (uint32_t)(p.gather_rows * p.s_stride * 2) : (uint32_t)row_end * s_row_bytes);
+  const i32x4 g_rsrc = make_buffer_resource(p.gidx, (uint32_t)(p.total_rows * 4));
+  uint32_t p_soff = RG ? (uint32_t)(row_begin + wave * 16) * 4u : (uint32_t)row_begin * r_row_bytes;
+  uint32_t q_soff = SG ? (uint32_t)(row_begin + wave * 16) * 4u : (uint32_t)row_begin * s_row_bytes;
+  const uint32_t p_step = RG ? r_row_bytes : (uint32_t)BK * r_row_bytes;
+  const uint32_t q_step = SG ? s_row_bytes : (uint32_t)BK * s_row_bytes;
+  int32_t rows_left = row_end - (row_begin + wave * 16);
+  const uint32_t lds_p = smem_base, lds_q = smem_base + 2 * 32768, wave_lds = (uint32_t)wave * (NINSTR * 1024);
+  uint32_t p_fill = lds_p, q_fill = lds_q;
+  if constexpr (SG) {
+    SMOE_TILE_PROLOGUE_MM_QG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc,
+                             p_step, q_step, n_mid, lds_p, lds_q, wave_lds);
+    SMOE_TILE_LOOP_MM_QG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc, p_step,
+                         q_step, n_mid, lds_p, lds_q, wave_lds);
+  } else {
+    SMOE_TILE_PROLOGUE_MM_PG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc,
+                             p_step, q_step, n_mid, lds_p, lds_q, wave_lds);
+    SMOE_TILE_LOOP_MM_PG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc, p_step,
+                         q_step, n_mid, lds_p, lds_q, wave_lds);
+  }
+  // epilogue out of the accumulation registers, 32 rows at a time through the two slots the last stage vacated
+  constexpr int PARK = 32 * EpiLayout<TB>::ROW_BYTES;
+  static_assert(2 * PARK <= 32768, "parking must fit into a ring slot");
+  char* region = smem + ((wave < 2 ? p_fill : q_fill) - smem_base) + (wave & 1) * PARK;
+  FwdEpilogueArgs ea;
+  ea.bias = nullptr;
+  ea.out0 = p.out + (int64_t)e * p.out_stride_e;
+  ea.out0_stride = p.out_stride_row;
+  ea.out1 = nullptr;
+  ea.out1_stride = 0;
+  ea.m_base = a0 + wa * TA;
+  ea.row_end = p.NA;
+  ea.n_base = b0 + wb * TB;
+  ea.N = p.NB;
+  forward_epilogue_rows_agpr<Mma, TA, TB, false, SMOE_ACT_SWIGLU>(region, lane, ea);
+  wait_vmem_all();  // the streams ran on into ring slots nobody reads: let those (empty) loads land before the end
+}
+
 template <class C>
 static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   static LdsLimitOnce lds_limit;
@@ -321,6 +427,24 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   // the kernel forms source addresses as row * (row stride in bytes, 32 bits) + column pointer
   SMOE_REQUIRE(p.r_stride > 0 && p.r_stride < (1ll << 31) && p.s_stride > 0 && p.s_stride < (1ll << 31),
                SMOE_ERR_UNSUPPORTED, "weight-grad gemm: operand row stride out of range");
+  if constexpr (C::R_GATHER != C::S_GATHER && C::BA == 256 && C::BB == 256) {
+    // the hand-scheduled loop addresses both operands with 32-bit byte offsets (the streams run a few stages past the
+    // expert's end before they stop) and tells rows past the end by a wrapped offset
+    const int64_t lim = (1ll << 32) - (1ll << 16);
+    const int64_t r_rows = C::R_GATHER ? p.gather_rows : p.total_rows + 8 * C::BK;
+    const int64_t s_rows = C::S_GATHER ? p.gather_rows : p.total_rows + 8 * C::BK;
+    const bool fits = p.off != nullptr && p.gidx != nullptr && p.gather_rows > 0 && (r_rows + 1) * p.r_stride * 2 < lim &&
+                      (s_rows + 1) * p.s_stride * 2 < lim && (p.total_rows + 8 * C::BK) * 4 < lim;
+    if (tuning().gemm_asm && fits) {
+      static LdsLimitOnce lds_limit_asm;
+      auto akern = varlen_k_asm_kernel<C::R_GATHER, C::S_GATHER>;
+      const int rc_a = lds_limit_asm.ensure((const void*)akern, 160 * 1024);
+      if (rc_a) return rc_a;
+      hipLaunchKernelGGL(akern, dim3((unsigned)grid), dim3(256), 160 * 1024, st, p);
+      SMOE_LAUNCH_CHECK();
+      return SMOE_OK;
+    }
+  }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
@@ -411,6 +535,7 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
   p.E = E;
   p.order = expert_schedule_order;
   p.total_rows = TK;
+  p.gather_rows = T;
   return launch_varlen_k_variant<true, false>(p, st);
 }
 
@@ -429,7 +554,7 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
                "up_projection_backward: nothing to compute (dw1, db1 and dx_expanded are all null)");
   SMOE_REQUIRE(TK == 0 || (dz && x_gather_idx && (!dw1 || x) && (!dx_expanded || w1)), SMOE_ERR_INVALID,
                "up_projection_backward: null pointer");
-  (void)T;
+  SMOE_REQUIRE(TK == 0 || !dw1 || T > 0, SMOE_ERR_INVALID, "up_projection_backward: T must be positive");
   SMOE_REQUIRE_ALIGNED("up_projection_backward", x, w1, dz, dw1, db1, dx_expanded);
   SMOE_REQUIRE(stride8(w1_stride_e) && stride8(w1_stride_row) && stride8(dw1_stride_e) && stride8(dw1_stride_row),
                SMOE_ERR_UNSUPPORTED, "up_projection_backward: weight strides must be multiples of 8 elements");
@@ -455,6 +580,7 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     p.E = E;
     p.order = expert_schedule_order;
     p.total_rows = TK;
+    p.gather_rows = T;
     rc = launch_varlen_k_variant<false, true>(p, st);
     if (rc) return rc;
   }

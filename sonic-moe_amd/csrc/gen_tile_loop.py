@@ -330,6 +330,278 @@ def srange(lo: int, n: int) -> str:
     return f"s{lo}" if n == 1 else f"s[{lo}:{lo + n - 1}]"
 
 
+# ======================================================================================================================
+# Weight-gradient loop ("MM"): dW[e][a][b] = sum over the expert's token rows m of R[row(m)][a] * S[row(m)][b].
+# Both operands are token-major in memory, so both LDS stages are [64 token rows][256 columns] and both fragment kinds
+# come from transpose reads.  P = R (output rows a), Q = S (output columns b).  One of the two is gathered through the
+# index array (x resp. dout rows), the other is read in place (dz resp. y1s rows of the expert):
+#   in place   per-lane byte offset fixed for the tile, the stage is a wave-uniform offset; the buffer resource ends at
+#              the expert's last row, so rows past it are dropped by the range check and read as zeros
+#   gathered   a wave's 16 token rows of a stage come with one scalar buffer load of 16 indices (range-checked against
+#              the index array), requested right behind the previous stage's loads; entries past the expert's end are
+#              replaced by -1, whose byte offset wraps to just below 4 GiB: out of range, zeros
+# Same pipeline, ring and waits as above; one tile per statement, no hand-over to a next tile: past the tile's last
+# stage the streams request rows past the expert's end, i.e. nothing.
+MV_PV, MV_QV = 128, 136          # in place: per-lane byte offsets of the 8 loads; gathered: the column part only
+MV_PRA, MV_QRA = 144, 160        # 16 + 16 fragment read addresses: slot-relative outside the statement
+MV_T, MV_HALF = 176, 178         # two scratch offsets; 1 in the upper half-wave (a load covers two token rows)
+MV_LAST = 178
+MS_PRSRC, MS_QRSRC, MS_GRSRC = 40, 44, 48
+MS_PSOFF, MS_QSOFF, MS_PSTEP, MS_QSTEP, MS_RLEFT, MS_NMID = 52, 53, 54, 55, 56, 57
+MS_PFILL, MS_QFILL, MS_LDSP, MS_LDSQ, MS_WLDS = 58, 59, 60, 61, 62
+MS_PCUR, MS_QCUR, MS_PFW, MS_QFW, MS_QFWN, MS_CNT, MS_T0, MS_T1, MS_DP, MS_DQ = 63, 64, 65, 66, 67, 68, 69, 70, 71, 72
+MS_A0, MS_A1 = 73, 74            # scratch of the gathered operand's address arithmetic
+MS_TOK = 76
+MS_LAST = MS_TOK + 15
+RPW = 2 * P_INSTR  # token rows a wave requests per stage and operand
+
+
+def mm_regs(which: str):
+    if which == "p":
+        return dict(v=MV_PV, rsrc=MS_PRSRC, soff=MS_PSOFF, step=MS_PSTEP, fw=MS_PFW)
+    return dict(v=MV_QV, rsrc=MS_QRSRC, soff=MS_QSOFF, step=MS_QSTEP, fw=MS_QFW)
+
+
+def mm_fragment_reads(setno: int, ks: int) -> list[str]:
+    out = []
+    off = ks * KSTEP * ROWB
+    for base, frag, n in ((MV_QRA, qfrag, FN), (MV_PRA, pfrag, FM)):
+        for f in range(n):
+            r = frag(setno, f)
+            out.append(f"ds_read_b64_tr_b16 v[{r}:{r + 1}], v{base + 2 * f} offset:{off}")
+            out.append(f"ds_read_b64_tr_b16 v[{r + 2}:{r + 3}], v{base + 2 * f + 1} offset:{off}")
+    return out
+
+
+def mm_next_slots() -> list[str]:
+    """as next_slots; leaves the distance to the next stage's slots in MS_DP / MS_DQ for the read addresses"""
+    return [
+        f"s_add_u32 s{MS_PFW}, s{MS_PCUR}, s{MS_WLDS}",
+        f"s_add_u32 s{MS_QFWN}, s{MS_QCUR}, s{MS_WLDS}",
+        f"s_mov_b32 s{MS_PFILL}, s{MS_PCUR}",
+        f"s_mov_b32 s{MS_QFILL}, s{MS_QCUR}",
+        f"s_sub_u32 s{MS_T0}, s{MS_PCUR}, s{MS_LDSP}",
+        f"s_xor_b32 s{MS_T0}, s{MS_T0}, {P_STAGE}",
+        f"s_add_u32 s{MS_T0}, s{MS_T0}, s{MS_LDSP}",
+        f"s_sub_u32 s{MS_DP}, s{MS_T0}, s{MS_PCUR}",
+        f"s_mov_b32 s{MS_PCUR}, s{MS_T0}",
+        f"s_add_u32 s{MS_T0}, s{MS_QCUR}, {Q_STAGE}",
+        f"s_sub_u32 s{MS_T1}, s{MS_T0}, s{MS_LDSQ}",
+        f"s_cmp_ge_u32 s{MS_T1}, {Q_SLOTS * Q_STAGE}",
+        f"s_cselect_b32 s{MS_T1}, {Q_SLOTS * Q_STAGE}, 0",
+        f"s_sub_u32 s{MS_T0}, s{MS_T0}, s{MS_T1}",
+        f"s_sub_u32 s{MS_DQ}, s{MS_T0}, s{MS_QCUR}",
+        f"s_mov_b32 s{MS_QCUR}, s{MS_T0}",
+    ]
+
+
+def mm_move_read_addresses() -> list[str]:
+    out = [f"v_add_u32 v{MV_PRA + k}, s{MS_DP}, v{MV_PRA + k}" for k in range(2 * FM)]
+    out += [f"v_add_u32 v{MV_QRA + k}, s{MS_DQ}, v{MV_QRA + k}" for k in range(2 * FN)]
+    return out
+
+
+def mm_ragged_fix(em: Emitter) -> list[str]:
+    """index run just arrived: entries for rows past the expert's end become -1; account for the 64 rows of the stage"""
+    lab = em.label("run")
+    out = [f"s_cmp_ge_i32 s{MS_RLEFT}, {RPW}", f"s_cbranch_scc1 {lab}"]
+    for j in range(RPW):
+        out += [f"s_cmp_gt_i32 s{MS_RLEFT}, {j}", f"s_cselect_b32 s{MS_TOK + j}, s{MS_TOK + j}, -1"]
+    out += [f"{lab}:", f"s_sub_i32 s{MS_RLEFT}, s{MS_RLEFT}, {BK}"]
+    return out
+
+
+def mm_load(which: str, i: int, gathered: bool) -> tuple[list[str], list[str], list[str]]:
+    """this wave's i-th load of a stage of stream `which`: what goes two, one and no matrix instructions ahead of it"""
+    r = mm_regs(which)
+    m0 = f"s_add_u32 m0, s{r['fw']}, {i * 1024}"
+    if not gathered:
+        return [], [m0], [f"buffer_load_dwordx4 v{r['v'] + i}, s[{r['rsrc']}:{r['rsrc'] + 3}], s{r['soff']} offen lds"]
+    vt = MV_T + (i & 1)
+    pre2 = [f"s_mul_i32 s{MS_A0}, s{MS_TOK + 2 * i}, s{r['step']}",
+            f"s_mul_i32 s{MS_A1}, s{MS_TOK + 2 * i + 1}, s{r['step']}",
+            f"s_sub_u32 s{MS_A1}, s{MS_A1}, s{MS_A0}"]
+    pre1 = [f"v_mul_lo_u32 v{vt}, v{MV_HALF}, s{MS_A1}",
+            f"v_add3_u32 v{vt}, v{vt}, s{MS_A0}, v{r['v'] + i}", m0]
+    return pre2, pre1, [f"buffer_load_dwordx4 v{vt}, s[{r['rsrc']}:{r['rsrc'] + 3}], 0 offen lds"]
+
+
+def mm_after_issue(which: str, gathered: bool) -> list[str]:
+    r = mm_regs(which)
+    if not gathered:
+        return [f"s_add_u32 s{r['soff']}, s{r['soff']}, s{r['step']}"]
+    return [f"s_buffer_load_dwordx16 s[{MS_TOK}:{MS_TOK + 15}], s[{MS_GRSRC}:{MS_GRSRC + 3}], s{r['soff']}",
+            f"s_add_u32 s{r['soff']}, s{r['soff']}, {4 * BK}"]
+
+
+def mm_issue_now(em: Emitter, which: str, gathered: bool) -> None:
+    """a whole stage of stream `which` into the slot its fill address names, outside the matrix-instruction stream"""
+    if gathered:
+        em("s_waitcnt lgkmcnt(0)")
+        for ln in mm_ragged_fix(em):
+            em(ln)
+    for i in range(P_INSTR):
+        pre2, pre1, ld = mm_load(which, i, gathered)
+        for ln in pre2 + pre1:
+            em(ln)
+        em("s_nop 0")
+        for ln in ld:
+            em(ln)
+    for ln in mm_after_issue(which, gathered):
+        em(ln)
+
+
+MM_SCHED = dict(read_step=1, p_first=3, p_step=7, q_tail_first=3, q_tail_step=7)
+
+
+def mm_emit_stage(em: Emitter, gp: bool, gq: bool, kind: str) -> None:
+    rs = MM_SCHED["read_step"]
+    nreads = 2 * (FN + FM)
+    reads_at = [r * rs for r in range(nreads)]
+    p_at = [MM_SCHED["p_first"] + MM_SCHED["p_step"] * i for i in range(P_INSTR)]
+    q_at = [MM_SCHED["q_tail_first"] + MM_SCHED["q_tail_step"] * i for i in range(Q_INSTR)]
+    assert p_at[0] >= 2 and q_at[0] >= 2 and p_at[-1] + 1 < 63 and q_at[-1] + 1 < 63
+    # ---- k-slice 0 on set A
+    ex: dict[int, list[str]] = {-1: ["s_waitcnt lgkmcnt(0)"]}
+    for at, line in zip(reads_at, mm_fragment_reads(1, 1)):
+        add_extra(ex, at, [line])
+    if kind != "first":
+        # the weight-side stage Q(s+2) goes into the slot the previous stage vacated
+        if gq:
+            add_extra(ex, -1, mm_ragged_fix(em))
+        for j, at in enumerate(q_at):
+            pre2, pre1, ld = mm_load("q", j, gq)
+            add_extra(ex, at - 2, pre2)
+            add_extra(ex, at - 1, pre1)
+            add_extra(ex, at, ld)
+        add_extra(ex, q_at[-1] + 1, mm_after_issue("q", gq))
+    if kind != "last":
+        slots = mm_next_slots()
+        at = max(reads_at) + 1
+        for j in range(0, len(slots), 4):
+            add_extra(ex, at, slots[j:j + 4])
+            at += 1
+        moves = mm_move_read_addresses()
+        per = -(-len(moves) // (FN * FM - 1 - at))  # spread over what is left of the k-slice
+        for j in range(0, len(moves), per):
+            add_extra(ex, at, moves[j:j + per])
+            at += 1
+        assert at <= FN * FM - 1
+        add_extra(ex, FN * FM - 1, [f"s_mov_b32 s{MS_QFW}, s{MS_QFWN}"])
+    emit_kslice(em, 0, kind == "first", ex)
+    em(f"s_waitcnt vmcnt({0 if kind == 'first' else Q_INSTR}) lgkmcnt(0)")
+    em("s_barrier")
+    # ---- k-slice 1 on set B
+    ex = {}
+    if kind != "last":
+        for at, line in zip(reads_at, mm_fragment_reads(0, 0)):
+            add_extra(ex, at, [line])
+        if gp:
+            add_extra(ex, -1, mm_ragged_fix(em))
+        for i, at in enumerate(p_at):
+            pre2, pre1, ld = mm_load("p", i, gp)
+            add_extra(ex, at - 2, pre2)
+            add_extra(ex, at - 1, pre1)
+            add_extra(ex, at, ld)
+        add_extra(ex, p_at[-1] + 1, mm_after_issue("p", gp))
+    emit_kslice(em, 1, False, ex)
+
+
+def mm_emit_prologue(gp: bool, gq: bool) -> list[str]:
+    """before the first statement of a tile: P(0) into token slot 1, Q(0), Q(1) into weight slots 1, 2 (the statement's
+    entry then requests P(1), Q(2) into the slots 0 / 0 it is told are vacant)"""
+    em = Emitter()
+    if gp or gq:
+        r = mm_regs("p" if gp else "q")
+        em(f"s_buffer_load_dwordx16 s[{MS_TOK}:{MS_TOK + 15}], s[{MS_GRSRC}:{MS_GRSRC + 3}], s{r['soff']}")
+        em(f"s_add_u32 s{r['soff']}, s{r['soff']}, {4 * BK}")
+    em(f"s_add_u32 s{MS_PFW}, s{MS_LDSP}, s{MS_WLDS}")
+    em(f"s_add_u32 s{MS_PFW}, s{MS_PFW}, {P_STAGE}")
+    mm_issue_now(em, "p", gp)
+    em(f"s_add_u32 s{MS_QFW}, s{MS_LDSQ}, s{MS_WLDS}")
+    em(f"s_add_u32 s{MS_QFW}, s{MS_QFW}, {Q_STAGE}")
+    mm_issue_now(em, "q", gq)
+    em(f"s_add_u32 s{MS_QFW}, s{MS_QFW}, {Q_STAGE}")
+    mm_issue_now(em, "q", gq)
+    em("s_waitcnt vmcnt(0) lgkmcnt(0)")
+    return em.lines
+
+
+def mm_emit_tile(gp: bool, gq: bool) -> list[str]:
+    em = Emitter()
+    em("s_barrier")
+    em(f"s_add_u32 s{MS_PFW}, s{MS_PFILL}, s{MS_WLDS}")
+    em(f"s_add_u32 s{MS_QFW}, s{MS_QFILL}, s{MS_WLDS}")
+    mm_issue_now(em, "p", gp)
+    mm_issue_now(em, "q", gq)
+    # stage 0 sits in the other token slot and in the weight slot after the vacated one; the read addresses come in
+    # slot-relative and leave slot-relative
+    em(f"s_mov_b32 s{MS_PCUR}, s{MS_PFILL}")
+    em(f"s_mov_b32 s{MS_QCUR}, s{MS_QFILL}")
+    for line in mm_next_slots()[4:]:
+        em(line)
+    em(f"s_mov_b32 s{MS_DP}, s{MS_PCUR}")
+    em(f"s_mov_b32 s{MS_DQ}, s{MS_QCUR}")
+    for line in mm_move_read_addresses():
+        em(line)
+    for line in mm_fragment_reads(0, 0):
+        em(line)
+    em(f"s_mov_b32 s{MS_CNT}, s{MS_NMID}")
+    em("s_waitcnt lgkmcnt(0)")
+    mm_emit_stage(em, gp, gq, "first")
+    top = em.label("stage")
+    em(f"{top}:")
+    mm_emit_stage(em, gp, gq, "mid")
+    em(f"s_sub_u32 s{MS_CNT}, s{MS_CNT}, 1")
+    em(f"s_cmp_lg_u32 s{MS_CNT}, 0")
+    em(f"s_cbranch_scc1 {top}")
+    mm_emit_stage(em, gp, gq, "last")
+    em(f"s_mov_b32 s{MS_PFILL}, s{MS_PCUR}")
+    em(f"s_mov_b32 s{MS_QFILL}, s{MS_QCUR}")
+    em(f"s_sub_u32 s{MS_DP}, 0, s{MS_PCUR}")
+    em(f"s_sub_u32 s{MS_DQ}, 0, s{MS_QCUR}")
+    for line in mm_move_read_addresses():
+        em(line)
+    # the index run requested behind the last loads must not land in registers the compiler owns again
+    em("s_waitcnt lgkmcnt(0)")
+    em("s_nop 15")
+    em("s_nop 7")
+    return em.lines
+
+
+def mm_operands():
+    outs = [
+        (vrange(MV_PRA, 2 * FM), "pra"), (vrange(MV_QRA, 2 * FN), "qra"), (srange(MS_PSOFF, 1), "psoff"),
+        (srange(MS_QSOFF, 1), "qsoff"), (srange(MS_RLEFT, 1), "rleft"), (srange(MS_PFILL, 1), "pfill"),
+        (srange(MS_QFILL, 1), "qfill"),
+    ]
+    ins = [
+        (vrange(MV_PV, P_INSTR), "pv"), (vrange(MV_QV, Q_INSTR), "qv"), (vrange(MV_HALF, 1), "half"),
+        (srange(MS_PRSRC, 4), "prsrc"), (srange(MS_QRSRC, 4), "qrsrc"), (srange(MS_GRSRC, 4), "grsrc"),
+        (srange(MS_PSTEP, 1), "pstep"), (srange(MS_QSTEP, 1), "qstep"), (srange(MS_NMID, 1), "nmid"),
+        (srange(MS_LDSP, 1), "ldsp"), (srange(MS_LDSQ, 1), "ldsq"), (srange(MS_WLDS, 1), "wlds"),
+    ]
+    return outs, ins
+
+
+def mm_statement(name: str, lines: list[str], with_matrix: bool) -> str:
+    outs, ins = mm_operands()
+    clob = [f"v{i}" for i in range(MV_T, MV_T + 2)]
+    if with_matrix:
+        clob += [f"v{i}" for i in range(0, 128)] + [f"a{i}" for i in range(256)]
+    clob += [f"s{i}" for i in range(MS_PCUR, MS_A1 + 1)] + [f"s{i}" for i in range(MS_TOK, MS_TOK + 16)]
+    clob += ["scc", "memory"]
+    params = ", ".join(n for _, n in outs + ins)
+    body = [f"#define {name}({params}) \\", "  asm volatile( \\"]
+    for ln in lines:
+        body.append(f'    "{ln}\\n\\t" \\')
+    body.append("    : " + ", ".join(f'"+{{{r}}}"({n})' for r, n in outs) + " \\")
+    body.append("    : " + ", ".join(f'"{{{r}}}"({n})' for r, n in ins) + " \\")
+    cl = [", ".join(f'"{c}"' for c in clob[i:i + 16]) for i in range(0, len(clob), 16)]
+    body.append("    : " + ", \\\n      ".join(cl) + ")")
+    return "\n".join(body)
+
+
 def statement(name: str, qmn: bool) -> str:
     lines = emit_tile(qmn)
     nq = n_qoff(qmn)
@@ -379,6 +651,15 @@ def header() -> str:
         statement("SMOE_TILE_LOOP_KK", False),
         "",
         statement("SMOE_TILE_LOOP_KM", True),
+        "",
+        "// weight-gradient loop: token operand in place, weight-side operand gathered (dW1) and the other way round (dW2)",
+        mm_statement("SMOE_TILE_PROLOGUE_MM_QG", mm_emit_prologue(False, True), False),
+        "",
+        mm_statement("SMOE_TILE_LOOP_MM_QG", mm_emit_tile(False, True), True),
+        "",
+        mm_statement("SMOE_TILE_PROLOGUE_MM_PG", mm_emit_prologue(True, False), False),
+        "",
+        mm_statement("SMOE_TILE_LOOP_MM_PG", mm_emit_tile(True, False), True),
         "",
     ]
     return "\n".join(parts)

@@ -36,6 +36,7 @@ LDS_BYTES = 160 * 1024
 PIECE = 1024
 NPIECE = LDS_BYTES // PIECE
 P_STREAM, Q_STREAM = 0, 1
+ZERO = -3  # identity of a value a range-checked load replaced by zero
 
 
 def kswz(row):  # kswz<64, 16> of gemm_common.h
@@ -94,6 +95,10 @@ class Wave:
         self.mfma_count = 0
         self.acc_seen = {}
         self.tile = None  # (expert, row0, row_end, n0) the matrix instructions work on
+        self.ldsp_reg = G.S_LDSP  # register that holds the LDS address of the token operand's ring
+        self.oob_zero = False  # loads beyond the extent write zeros (the weight-gradient loop relies on it)
+        self.smem_out = set()  # scalar registers a scalar load in flight will write
+        self.expect = None  # callable(wave, fn, fm, stage, ks) -> (want_q, want_p); default: the varlen-M operands
 
     # ---- memory side
     def issue_load(self, voff_reg, rsrc, soff_reg):
@@ -106,8 +111,10 @@ class Wave:
             raise SimError(f"load through unknown resource s{rsrc}")
         base = self.s[rsrc] | ((self.s[rsrc + 1] & 0xffff) << 32)
         extent = self.s[rsrc + 2] & 0xffffffff
-        off = (self.v[voff_reg] + self.s[soff_reg]) & 0xffffffff
-        if (off + 16 > extent).any():
+        soff = self.s[soff_reg] if soff_reg is not None else 0
+        off = (self.v[voff_reg] + soff) & 0xffffffff
+        oob = off + 16 > extent
+        if oob.any() and not self.oob_zero:
             raise SimError(f"wave {self.w}: load offset {int(off.max())} + 16 beyond extent {extent} (stream {stream})")
         if (off % 16).any():
             raise SimError("unaligned global piece")
@@ -115,7 +122,7 @@ class Wave:
             raise SimError(f"wave {self.w}: M0 = {self.m0}")
         piece = self.m0 // PIECE
         ring_lo, ring_hi = (0, G.P_SLOTS * G.P_STAGE) if stream == P_STREAM else (G.P_SLOTS * G.P_STAGE, LDS_BYTES)
-        if not (ring_lo <= self.m0 - self.s[G.S_LDSP] < ring_hi):
+        if not (ring_lo <= self.m0 - self.s[self.ldsp_reg] < ring_hi):
             raise SimError(f"wave {self.w}: stream {stream} load lands outside its ring (M0 = {self.m0})")
         if lds.pending[piece] is not None:
             raise SimError(f"piece {piece} requested twice")
@@ -126,7 +133,9 @@ class Wave:
         if piece in self.reads_out:
             raise SimError(f"wave {self.w} overwrites piece {piece} while its own read is in flight")
         elem = (base + off) // 2
-        tags = ((elem[:, None] + np.arange(8)[None, :]) | (stream << 60)).reshape(-1)
+        tags = (elem[:, None] + np.arange(8)[None, :]) | (stream << 60)
+        tags[oob] = ZERO
+        tags = tags.reshape(-1)
         lds.pending[piece] = self.w
         self.vmq.append((piece, tags))
 
@@ -193,6 +202,10 @@ class Wave:
         self.acc_seen[acc] = n_done + 1
         lane = np.arange(64)
         wm, wn = self.w % 2, self.w // 2
+        if self.expect is not None:
+            want_q, want_p = self.expect(self, fn, fm, stage, ks)
+            self._compare(qreg, preg, want_q, want_p, stage, ks, fn, fm)
+            return
         k = stage * G.BK + ks * G.KSTEP + 8 * (lane // 16)[:, None] + np.arange(8)[None, :]
         # weight fragment: feature row n
         n = n0 + wn * G.TN + fn * G.FR + lane % 16
@@ -207,6 +220,9 @@ class Wave:
         m = np.minimum(row0 + wm * G.TM + fm * G.FR + lane % 16, row_end - 1)
         row = prob.gidx[m] if prob.gidx is not None else m
         want_p = (row[:, None] * prob.p_stride + k) | (P_STREAM << 60)
+        self._compare(qreg, preg, want_q, want_p, stage, ks, fn, fm)
+
+    def _compare(self, qreg, preg, want_q, want_p, stage, ks, fn, fm):
         got_q = self.vt[qreg:qreg + 4].transpose(1, 0, 2).reshape(64, 8)
         got_p = self.vt[preg:preg + 4].transpose(1, 0, 2).reshape(64, 8)
         if not (got_q == want_q).all():
@@ -233,6 +249,11 @@ def _first(m):
 
 def asm_lines(qmn: bool) -> list[str]:
     return G.emit_tile(qmn)
+
+
+def _signed(x: int) -> int:
+    x &= 0xffffffff
+    return x - (1 << 32) if x & 0x80000000 else x
 
 
 def _sval(w: Wave, tok: str) -> int:
@@ -278,6 +299,7 @@ def run_wave(w: Wave, lines: list[str]):
                 assert int(m.group(1)) == 0
                 w.reads_out = []
                 w.regs_out = set()
+                w.smem_out = set()
         elif op in ("s_add_u32", "s_sub_u32", "s_xor_b32"):
             a, b = _sval(w, args[1]), _sval(w, args[2])
             r = a + b if op == "s_add_u32" else (a - b if op == "s_sub_u32" else a ^ b)
@@ -286,6 +308,31 @@ def run_wave(w: Wave, lines: list[str]):
                 w.m0 = r
             else:
                 w.s[int(args[0][1:])] = r
+        elif op == "s_mul_i32":
+            for a in args[1:]:
+                if a.startswith("s") and int(a[1:]) in w.smem_out:
+                    raise SimError("scalar register read while a scalar load into it is in flight")
+            w.s[int(args[0][1:])] = (_sval(w, args[1]) * _sval(w, args[2])) & 0xffffffff
+        elif op == "s_sub_i32":
+            w.s[int(args[0][1:])] = (_sval(w, args[1]) - _sval(w, args[2])) & 0xffffffff
+        elif op in ("s_cmp_ge_i32", "s_cmp_gt_i32"):
+            a, b = _signed(_sval(w, args[0])), _signed(_sval(w, args[1]))
+            w.scc = int(a >= b) if op == "s_cmp_ge_i32" else int(a > b)
+        elif op == "s_buffer_load_dwordx16":
+            dst = _first(_RE_SR.match(args[0]))
+            rs = _first(_RE_SR.match(args[1]))
+            off = _sval(w, args[2])
+            extent = w.s[rs + 2] & 0xffffffff
+            base = w.s[rs] | ((w.s[rs + 1] & 0xffff) << 32)
+            assert base == 0 and off % 4 == 0
+            for j in range(16):
+                o = off + 4 * j
+                w.s[dst + j] = int(w.prob.gidx_flat[o // 4]) & 0xffffffff if o + 4 <= extent else 0
+            w.smem_out = set(range(dst, dst + 16))
+        elif op == "v_mul_lo_u32":
+            w.v[int(args[0][1:])] = (w.v[int(args[1][1:])] * _sval(w, args[2])) & 0xffffffff
+        elif op == "v_add3_u32":
+            w.v[int(args[0][1:])] = (w.v[int(args[1][1:])] + _sval(w, args[2]) + w.v[int(args[3][1:])]) & 0xffffffff
         elif op == "s_mov_b32":
             w.s[int(args[0][1:])] = _sval(w, args[1])
         elif op == "s_cmp_lg_u32":
@@ -293,7 +340,9 @@ def run_wave(w: Wave, lines: list[str]):
         elif op == "s_cmp_ge_u32":
             w.scc = int(_sval(w, args[0]) >= _sval(w, args[1]))
         elif op == "s_cselect_b32":
-            w.s[int(args[0][1:])] = _sval(w, args[1]) if w.scc else _sval(w, args[2])
+            if any(a.startswith("s") and int(a[1:]) in w.smem_out for a in args[1:]):
+                raise SimError("scalar register read while a scalar load into it is in flight")
+            w.s[int(args[0][1:])] = (_sval(w, args[1]) if w.scc else _sval(w, args[2])) & 0xffffffff
         elif op == "s_cbranch_scc1":
             if w.scc:
                 pc = labels[args[0]]
@@ -312,7 +361,7 @@ def run_wave(w: Wave, lines: list[str]):
         elif op == "buffer_load_dwordx4":
             soff = args[2].split()[0]
             assert args[2].split()[1:] == ["offen", "lds"]
-            w.issue_load(int(args[0][1:]), _first(_RE_SR.match(args[1])), int(soff[1:]))
+            w.issue_load(int(args[0][1:]), _first(_RE_SR.match(args[1])), int(soff[1:]) if soff.startswith("s") else None)
         elif op == "v_mfma_f32_16x16x32_bf16":
             # operands: a[..], v[..], v[..], (0 | a[..]) - the vector ranges contain commas only between operands
             m = re.match(r"a\[(\d+):(\d+)\], v\[(\d+):(\d+)\], v\[(\d+):(\d+)\], (0|a\[(\d+):(\d+)\])$", rest)
@@ -491,3 +540,118 @@ def simulate(prob: Problem, lds_base: int = 0) -> dict:
     for w in waves:
         w.wait_vm(0)
     return dict(mfma=sum(w.mfma_count for w in waves), barriers=waves[0].nbarrier)
+
+
+# ---- weight-gradient loop --------------------------------------------------------------------------------------------
+@dataclass
+class ProblemMM:
+    gp: bool  # the token-side operand R is gathered (dW2); otherwise the weight-side operand S is (dW1)
+    NA: int
+    NB: int
+    r_stride: int
+    s_stride: int
+    gather_rows: int
+    gidx_flat: np.ndarray  # (total_rows,) grouped row -> row of the gathered tensor
+    row_begin: int
+    row_end: int
+    a0: int
+    b0: int
+
+    @property
+    def total_rows(self):
+        return len(self.gidx_flat)
+
+
+def simulate_mm(prob: ProblemMM) -> dict:
+    gp, gq = prob.gp, not prob.gp
+    pro, lines = G.mm_emit_prologue(gp, gq), G.mm_emit_tile(gp, gq)
+    lds = Lds()
+    waves = [Wave(w, lds, prob) for w in range(G.NW)]
+    S = -(-(prob.row_end - prob.row_begin) // G.BK)
+    S_eff = max(S, 3)
+    rrb, srb = prob.r_stride * 2, prob.s_stride * 2
+    lane = np.arange(64)
+
+    def clamp8(c, n):
+        return np.minimum(c - c % 8, n - 8) + c % 8
+
+    def expect(w, fn, fm, stage, ks):
+        wa, wb = w.w % 2, w.w // 2
+        m = prob.row_begin + stage * G.BK + ks * G.KSTEP + 8 * (lane // 16)[:, None] + np.arange(8)[None, :]
+        valid = m < prob.row_end
+        mc = np.minimum(m, prob.total_rows - 1)
+        b = clamp8(prob.b0 + wb * G.TN + fn * G.FR + lane % 16, prob.NB)
+        a = clamp8(prob.a0 + wa * G.TM + fm * G.FR + lane % 16, prob.NA)
+        rq = prob.gidx_flat[mc] if gq else mc
+        rp = prob.gidx_flat[mc] if gp else mc
+        want_q = np.where(valid, (rq * prob.s_stride + b[:, None]) | (Q_STREAM << 60), ZERO)
+        want_p = np.where(valid, (rp * prob.r_stride + a[:, None]) | (P_STREAM << 60), ZERO)
+        return want_q, want_p
+
+    for w in waves:
+        w.ldsp_reg = G.MS_LDSP
+        w.oob_zero = True
+        w.expect = expect
+        w.tile = (0, 0, 0, 0)
+        s = w.s
+        s[G.MS_PRSRC:G.MS_PRSRC + 4] = [0, 0, (prob.gather_rows if gp else prob.row_end) * rrb, 0x20000]
+        s[G.MS_QRSRC:G.MS_QRSRC + 4] = [0, 0, (prob.gather_rows if gq else prob.row_end) * srb, 0x20000]
+        s[G.MS_GRSRC:G.MS_GRSRC + 4] = [0, 0, prob.total_rows * 4, 0x20000]
+        pv, qv = [], []
+        for i in range(G.P_INSTR):
+            kl = (w.w * G.P_INSTR + i) * 2 + lane // 32
+            phys16 = lane % 32
+            log32 = (phys16 >> 1) ^ mnswz(kl)
+            c = ((log32 << 1) | (phys16 & 1)) * 8
+            a = np.minimum(prob.a0 + c, prob.NA - 8)
+            b = np.minimum(prob.b0 + c, prob.NB - 8)
+            pv.append((0 if gp else kl * rrb) + a * 2)
+            qv.append((0 if gq else kl * srb) + b * 2)
+        for i in range(G.P_INSTR):
+            w.v[G.MV_PV + i] = pv[i]
+            w.v[G.MV_QV + i] = qv[i]
+        wa, wb = w.w % 2, w.w // 2
+        grp, i16 = lane >> 4, lane & 15
+        kk = 8 * grp + (i16 >> 2)
+        for f in range(8):
+            for h in range(2):
+                k = kk + 4 * h
+                w.v[G.MV_PRA + 2 * f + h] = k * G.ROWB + ((((wa * G.TM) // 16 + f) ^ mnswz(k)) << 5) + ((i16 & 3) << 3)
+                w.v[G.MV_QRA + 2 * f + h] = k * G.ROWB + ((((wb * G.TN) // 16 + f) ^ mnswz(k)) << 5) + ((i16 & 3) << 3)
+        w.v[G.MV_HALF] = lane >> 5
+        first_run = (prob.row_begin + w.w * 16) * 4
+        s[G.MS_PSOFF] = first_run if gp else prob.row_begin * rrb
+        s[G.MS_QSOFF] = first_run if gq else prob.row_begin * srb
+        s[G.MS_PSTEP] = rrb if gp else G.BK * rrb
+        s[G.MS_QSTEP] = srb if gq else G.BK * srb
+        s[G.MS_RLEFT] = (prob.row_end - (prob.row_begin + w.w * 16)) & 0xffffffff
+        s[G.MS_NMID] = S_eff - 2
+        s[G.MS_LDSP], s[G.MS_LDSQ], s[G.MS_WLDS] = 0, G.P_SLOTS * G.P_STAGE, w.w * G.P_INSTR * 1024
+        s[G.MS_PFILL], s[G.MS_QFILL] = 0, G.P_SLOTS * G.P_STAGE
+        for _ in run_wave(w, pro):
+            raise SimError("barrier in the prologue")
+        if w.vmq or w.smem_out:
+            raise SimError("the prologue leaves operations in flight")
+    saved = [(w.v[G.MV_PRA:G.MV_PRA + 16].copy(), w.v[G.MV_QRA:G.MV_QRA + 16].copy()) for w in waves]
+    gens = [run_wave(w, lines) for w in waves]
+    alive = [True] * G.NW
+    while any(alive):
+        state = []
+        for i, g in enumerate(gens):
+            try:
+                next(g)
+                state.append("barrier")
+            except StopIteration:
+                alive[i] = False
+                state.append("done")
+        if len(set(state)) != 1:
+            raise SimError(f"waves disagree at a barrier: {state}")
+    for w, (pra, qra) in zip(waves, saved):
+        if len(w.acc_seen) != G.FN * G.FM or any(v != 2 * S_eff for v in w.acc_seen.values()):
+            raise SimError(f"wave {w.w}: accumulators saw {sorted(set(w.acc_seen.values()))} k-slices, want {2 * S_eff}")
+        if w.reads_out or w.smem_out:
+            raise SimError("LDS or scalar reads in flight at the end of the statement")
+        if not ((w.v[G.MV_PRA:G.MV_PRA + 16] == pra).all() and (w.v[G.MV_QRA:G.MV_QRA + 16] == qra).all()):
+            raise SimError("read addresses do not come back slot-relative")
+        w.wait_vm(0)
+    return dict(mfma=sum(w.mfma_count for w in waves), barriers=waves[0].nbarrier, stages=S_eff)
