@@ -297,53 +297,146 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
 }
 
 
-// ---- the same GEMM on the hand-scheduled loop ------------------------------------------------------------------------
-// Four wavefronts as 2 x 2 wave tiles of 128 x 128; the contraction is the weight-gradient statement of
-// tile_loop_gen.h (prologue + loop), which fetches the gather indices, forms the gathered operand's addresses and
-// leaves the tile in a[0:255].  Rows past the expert's end cost no code: the operand read in place has a buffer
-// resource that ends at the expert's last row, the gathered one gets index -1, and either way the range check of the
-// direct-to-LDS load writes zeros.  Experts with fewer than three stages of rows run three (the extra ones are all
-// zeros), so one pipeline shape serves every expert, the empty ones included.
+// ---- the same GEMM on the hand-scheduled loop, as a stream of tiles ---------------------------------------------------
+// Schedule.  The 32 tiles an XCD's 32 workgroups run side by side are one block (BA_T x BB_T tiles) of ONE expert's
+// output, as in the blocked order above - so all of them have the same length (the expert's token count) and a
+// persistent workgroup that takes tile i of every block of its XCD is balanced against its 31 neighbours by
+// construction.  Across the XCDs the blocks are dealt by cost: experts sorted by token count, largest first (or in the
+// caller's expert_schedule_order), their blocks laid out in that order and dealt to the XCDs in snake order
+// 0..7, 7..0, so every XCD gets one of the larger and one of the smaller blocks of each run of 16.  No queue, no
+// atomics: the table is built by one small kernel per launch and every workgroup knows its next tiles in advance,
+// which is what lets the load streams of the loop run across tile boundaries.
+//   table: int32 count[8] (rounds per XCD), then block[8][max_rounds] (block id = expert * blocks_per_expert + block)
+constexpr int SCHED_MAX_E = 4096;
+
+static inline size_t block_schedule_bytes(int64_t blocks_total) {
+  return (size_t)(8 + 8 * ((blocks_total + 7) / 8 + 1)) * sizeof(int32_t);
+}
+
+__global__ __launch_bounds__(1024) void build_block_schedule_kernel(const int32_t* __restrict__ off,
+                                                                    const int32_t* __restrict__ order, int E, int nb,
+                                                                    int max_rounds, int32_t* __restrict__ table) {
+  __shared__ int32_t cost[SCHED_MAX_E];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += 1024) cost[e] = off[e + 1] - off[e];
+  __syncthreads();
+  const int64_t total = (int64_t)E * nb;
+  for (int e = tid; e < E; e += 1024) {
+    int pos = 0;  // position of expert e in the schedule order
+    if (order != nullptr) {
+      for (int i = 0; i < E; i++) pos = order[i] == e ? i : pos;
+    } else {
+      const int c = cost[e];
+      for (int o = 0; o < E; o++) pos += (cost[o] > c || (cost[o] == c && o < e)) ? 1 : 0;
+    }
+    for (int j = 0; j < nb; j++) {
+      const int64_t seq = (int64_t)pos * nb + j;
+      const int r = (int)(seq & 15);
+      const int x = r < 8 ? r : 15 - r;
+      const int64_t round = 2 * (seq >> 4) + (r >= 8 ? 1 : 0);
+      table[8 + (int64_t)x * max_rounds + round] = e * nb + j;
+    }
+  }
+  if (tid < 8) {
+    const int rem = (int)(total & 15);
+    int n = (int)(2 * (total >> 4));
+    if (tid < (rem < 8 ? rem : 8)) n += 1;
+    if (rem > 8 && tid > 15 - rem) n += 1;
+    table[tid] = n;
+  }
+}
+
+// Four wavefronts as 2 x 2 wave tiles of 128 x 128; the contraction of a tile is the weight-gradient statement of
+// tile_loop_gen.h, which fetches the gather indices, forms the gathered operand's addresses, keeps both load streams
+// running into the next tile and leaves the tile in a[0:255].  Rows past the expert's end cost no code: the operand
+// read in place has a buffer resource that ends at the expert's last row, the gathered one gets index -1, and either
+// way the range check of the direct-to-LDS load writes zeros.  Experts with fewer than three stages of rows run three
+// (the extra ones read nothing), so one pipeline shape serves every expert, the empty ones included.
 typedef int32_t ki32x8 __attribute__((ext_vector_type(8)));
 typedef int32_t ki32x16 __attribute__((ext_vector_type(16)));
 
+struct BlockShape {
+  int nb, nbj, ba, bb;  // blocks per expert, blocks along b, tiles per block along a / b
+};
+
 template <bool RG, bool SG>
-__global__ __launch_bounds__(256) void varlen_k_asm_kernel(const VarlenKParams p) {
+__global__ __launch_bounds__(256) void varlen_k_stream_kernel(const VarlenKParams p, const BlockShape bs,
+                                                              const int32_t* table, int max_rounds) {
   static_assert(RG != SG, "exactly one operand is gathered");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   typedef Bf16Mma Mma;
   constexpr int BA = 256, BB = 256, TA = 128, TB = 128, BK = 64, ROWB = 512, NINSTR = SMOE_TL_P_INSTR;
-  constexpr int FA = TA / 16, FB = TB / 16;
-  static_assert(FA == SMOE_TL_FM && FB == SMOE_TL_FN && Mma::FR == 16, "the generated loop is written for this tile shape");
+  static_assert(TA / 16 == SMOE_TL_FM && TB / 16 == SMOE_TL_FN && Mma::FR == 16, "the generated loop is written for this tile shape");
   const uint32_t smem_base = lds_address(smem);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wa = wave % 2, wb = wave / 2;
 
-  int e, ta, tb;
-  if (!decode_tile(p, (int64_t)blockIdx.x, e, ta, tb)) return;
-  if (p.order != nullptr) e = p.order[e];
-  const int a0 = ta * BA, b0 = tb * BB;
-  const int row_begin = p.off[e], row_end = p.off[e + 1];
-  const int S = (row_end - row_begin + BK - 1) / BK;
-  const uint32_t n_mid = (uint32_t)(S < 3 ? 3 : S) - 2u;
+  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;  // workgroup b runs on XCD b % 8
+  const const_i32_ptr tab = (const_i32_ptr)table, off = (const_i32_ptr)p.off;
+  const int rounds = tab[xcd];
+  if (rounds == 0) return;
+  const const_i32_ptr blocks = tab + 8 + (int64_t)xcd * max_rounds;
+  struct Tile {
+    int e, row_begin, row_end, a0, b0;
+  };
+  // past the XCD's last round: an empty expert - every load out of range
+  auto tile_at = [&](int r) {
+    Tile t = {0, 0, 0, 0, 0};
+    if (r < rounds) {
+      const int B = blocks[r];
+      t.e = B / bs.nb;
+      const int blk = B - t.e * bs.nb;
+      t.a0 = ((blk / bs.nbj) * bs.ba + slot / bs.bb) * BA;
+      t.b0 = ((blk % bs.nbj) * bs.bb + slot % bs.bb) * BB;
+      t.row_begin = off[t.e];
+      t.row_end = off[t.e + 1];
+    }
+    return t;
+  };
+  auto stages_of = [&](const Tile& t) {
+    const int S = (t.row_end - t.row_begin + BK - 1) / BK;
+    return S < 3 ? 3 : S;
+  };
 
   const uint32_t r_row_bytes = (uint32_t)p.r_stride * 2u, s_row_bytes = (uint32_t)p.s_stride * 2u;
+  auto opaque_lane = [&]() {
+    int l = lane;
+    asm volatile("" : "+v"(l));
+    return l;
+  };
   // per-lane source offsets of the 8 loads of a stage: load i of this wave covers the token rows 2 i, 2 i + 1 of the
   // wave's 16 (lanes 0-31 / 32-63) and 16 bytes per lane of the 512 the tile takes of a row
-  ki32x8 pv, qv;
+  auto lane_offsets = [&](const Tile& t, ki32x8& pvv, ki32x8& qvv) {
+    const int ln = opaque_lane();
 #pragma unroll
-  for (int i = 0; i < NINSTR; i++) {
-    const int kl = (wave * NINSTR + i) * 2 + lane / 32;
-    const int phys16 = lane % 32;
-    const int log32 = (phys16 >> 1) ^ mnswz(kl);
-    const int c = ((log32 << 1) | (phys16 & 1)) * 8;
-    int a = a0 + c, b = b0 + c;
-    a = a <= p.NA - 8 ? a : p.NA - 8;
-    b = b <= p.NB - 8 ? b : p.NB - 8;
-    pv[i] = (int32_t)((RG ? 0u : (uint32_t)kl * r_row_bytes) + (uint32_t)a * 2u);
-    qv[i] = (int32_t)((SG ? 0u : (uint32_t)kl * s_row_bytes) + (uint32_t)b * 2u);
-  }
+    for (int i = 0; i < NINSTR; i++) {
+      const int kl = (wave * NINSTR + i) * 2 + ln / 32;
+      const int phys16 = ln % 32;
+      const int log32 = (phys16 >> 1) ^ mnswz(kl);
+      const int c = ((log32 << 1) | (phys16 & 1)) * 8;
+      int a = t.a0 + c, b = t.b0 + c;
+      a = a <= p.NA - 8 ? a : p.NA - 8;
+      b = b <= p.NB - 8 ? b : p.NB - 8;
+      pvv[i] = (int32_t)((RG ? 0u : (uint32_t)kl * r_row_bytes) + (uint32_t)a * 2u);
+      qvv[i] = (int32_t)((SG ? 0u : (uint32_t)kl * s_row_bytes) + (uint32_t)b * 2u);
+    }
+  };
+  auto first_offsets = [&](const Tile& t, int32_t& ps, int32_t& qs) {
+    const uint32_t run = (uint32_t)(t.row_begin + wave * 16) * 4u;
+    ps = (int32_t)(RG ? run : (uint32_t)t.row_begin * r_row_bytes);
+    qs = (int32_t)(SG ? run : (uint32_t)t.row_begin * s_row_bytes);
+  };
+
+  auto uniform = [](auto& v) {
+#pragma unroll
+    for (int k = 0; k < (int)(sizeof(v) / 4); k++) v[k] = __builtin_amdgcn_readfirstlane(v[k]);
+  };
+  Tile cur = tile_at(0), nxt = tile_at(1);
+  ki32x8 pv, qv, pvn, qvn;
+  lane_offsets(cur, pv, qv);
+  lane_offsets(nxt, pvn, qvn);
   // transpose-read addresses inside a slot: fragment f, half h -> 2 f + h
   ki32x16 pra, qra;
   {
@@ -361,47 +454,86 @@ __global__ __launch_bounds__(256) void varlen_k_asm_kernel(const VarlenKParams p
   }
   const int32_t half = lane >> 5;
   // extents: the operand read in place ends at the expert's last row, the gathered one at its tensor's end
-  const i32x4 p_rsrc = make_buffer_resource(p.R, RG ? (uint32_t)(p.gather_rows * p.r_stride * 2) : (uint32_t)row_end * r_row_bytes);
-  const i32x4 q_rsrc = make_buffer_resource(p.S, SG ? (uint32_t)(p.gather_rows * p.s_stride * 2) : (uint32_t)row_end * s_row_bytes);
+  i32x4 p_rsrc = make_buffer_resource(p.R, RG ? (uint32_t)(p.gather_rows * p.r_stride * 2) : (uint32_t)cur.row_end * r_row_bytes);
+  i32x4 q_rsrc = make_buffer_resource(p.S, SG ? (uint32_t)(p.gather_rows * p.s_stride * 2) : (uint32_t)cur.row_end * s_row_bytes);
   const i32x4 g_rsrc = make_buffer_resource(p.gidx, (uint32_t)(p.total_rows * 4));
-  uint32_t p_soff = RG ? (uint32_t)(row_begin + wave * 16) * 4u : (uint32_t)row_begin * r_row_bytes;
-  uint32_t q_soff = SG ? (uint32_t)(row_begin + wave * 16) * 4u : (uint32_t)row_begin * s_row_bytes;
-  const uint32_t p_step = RG ? r_row_bytes : (uint32_t)BK * r_row_bytes;
-  const uint32_t q_step = SG ? s_row_bytes : (uint32_t)BK * s_row_bytes;
-  int32_t rows_left = row_end - (row_begin + wave * 16);
-  const uint32_t lds_p = smem_base, lds_q = smem_base + 2 * 32768, wave_lds = (uint32_t)wave * (NINSTR * 1024);
-  uint32_t p_fill = lds_p, q_fill = lds_q;
-  if constexpr (SG) {
-    SMOE_TILE_PROLOGUE_MM_QG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc,
-                             p_step, q_step, n_mid, lds_p, lds_q, wave_lds);
-    SMOE_TILE_LOOP_MM_QG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc, p_step,
-                         q_step, n_mid, lds_p, lds_q, wave_lds);
-  } else {
-    SMOE_TILE_PROLOGUE_MM_PG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc,
-                             p_step, q_step, n_mid, lds_p, lds_q, wave_lds);
-    SMOE_TILE_LOOP_MM_PG(pra, qra, p_soff, q_soff, rows_left, p_fill, q_fill, pv, qv, half, p_rsrc, q_rsrc, g_rsrc, p_step,
-                         q_step, n_mid, lds_p, lds_q, wave_lds);
+  const uint32_t lds_p = smem_base, lds_q = smem_base + 2 * 32768;
+  ki32x8 state = {}, next = {}, geo = {};
+  {
+    int32_t ps, qs;
+    first_offsets(cur, ps, qs);
+    state[SMOE_MM_PSOFF] = ps;
+    state[SMOE_MM_QSOFF] = qs;
   }
-  // epilogue out of the accumulation registers, 32 rows at a time through the two slots the last stage vacated
+  state[SMOE_MM_RLEFT] = cur.row_end - (cur.row_begin + wave * 16);
+  state[SMOE_MM_PFILL] = (int32_t)lds_p;
+  state[SMOE_MM_QFILL] = (int32_t)lds_q;
+  geo[SMOE_MM_PSTEP] = (int32_t)(RG ? r_row_bytes : (uint32_t)BK * r_row_bytes);
+  geo[SMOE_MM_QSTEP] = (int32_t)(SG ? s_row_bytes : (uint32_t)BK * s_row_bytes);
+  geo[SMOE_MM_LDSP] = (int32_t)lds_p;
+  geo[SMOE_MM_LDSQ] = (int32_t)lds_q;
+  geo[SMOE_MM_WLDS] = wave * (NINSTR * 1024);
+  if constexpr (SG) {
+    SMOE_TILE_PROLOGUE_MM_QG(pra, qra, pv, qv, p_rsrc, q_rsrc, state, pvn, qvn, half, g_rsrc, next, geo);
+  } else {
+    SMOE_TILE_PROLOGUE_MM_PG(pra, qra, pv, qv, p_rsrc, q_rsrc, state, pvn, qvn, half, g_rsrc, next, geo);
+  }
+  uniform(state);
+  uniform(p_rsrc);
+  uniform(q_rsrc);
+  // the prologue has requested one token-side stage and two weight-side stages of the first tile
+  state[SMOE_MM_PLEFT] = stages_of(cur) - 1;
+  state[SMOE_MM_QLEFT] = stages_of(cur) - 2;
+
   constexpr int PARK = 32 * EpiLayout<TB>::ROW_BYTES;
   static_assert(2 * PARK <= 32768, "parking must fit into a ring slot");
-  char* region = smem + ((wave < 2 ? p_fill : q_fill) - smem_base) + (wave & 1) * PARK;
-  FwdEpilogueArgs ea;
-  ea.bias = nullptr;
-  ea.out0 = p.out + (int64_t)e * p.out_stride_e;
-  ea.out0_stride = p.out_stride_row;
-  ea.out1 = nullptr;
-  ea.out1_stride = 0;
-  ea.m_base = a0 + wa * TA;
-  ea.row_end = p.NA;
-  ea.n_base = b0 + wb * TB;
-  ea.N = p.NB;
-  forward_epilogue_rows_agpr<Mma, TA, TB, false, SMOE_ACT_SWIGLU>(region, lane, ea);
+  for (int r = 0;; r++) {
+    geo[SMOE_MM_NMID] = stages_of(cur) - 2;
+    {
+      int32_t ps, qs;
+      first_offsets(nxt, ps, qs);
+      next[SMOE_MM_PSOFFN] = ps;
+      next[SMOE_MM_QSOFFN] = qs;
+    }
+    next[SMOE_MM_PEXTN] = (int32_t)((uint32_t)nxt.row_end * r_row_bytes);
+    next[SMOE_MM_QEXTN] = (int32_t)((uint32_t)nxt.row_end * s_row_bytes);
+    next[SMOE_MM_RLEFTN] = nxt.row_end - (nxt.row_begin + wave * 16);
+    next[SMOE_MM_SNEXT] = stages_of(nxt);
+    if constexpr (SG) {
+      SMOE_TILE_LOOP_MM_QG(pra, qra, pv, qv, p_rsrc, q_rsrc, state, pvn, qvn, half, g_rsrc, next, geo);
+    } else {
+      SMOE_TILE_LOOP_MM_PG(pra, qra, pv, qv, p_rsrc, q_rsrc, state, pvn, qvn, half, g_rsrc, next, geo);
+    }
+    // (the compiler takes the scalar results of an assembly statement for per-lane values; say that they are uniform)
+    uniform(state);
+    uniform(p_rsrc);
+    uniform(q_rsrc);
+    // both streams are on nxt now; their next tile is the one after it
+    const Tile nn = tile_at(r + 2);
+    lane_offsets(nn, pvn, qvn);
+    // epilogue out of the accumulation registers, 32 rows at a time through the two slots the last stage vacated
+    char* region = smem + ((uint32_t)(wave < 2 ? state[SMOE_MM_PFILL] : state[SMOE_MM_QFILL]) - smem_base) + (wave & 1) * PARK;
+    FwdEpilogueArgs ea;
+    ea.bias = nullptr;
+    ea.out0 = p.out + (int64_t)cur.e * p.out_stride_e;
+    ea.out0_stride = p.out_stride_row;
+    ea.out1 = nullptr;
+    ea.out1_stride = 0;
+    ea.m_base = cur.a0 + wa * TA;
+    ea.row_end = p.NA;
+    ea.n_base = cur.b0 + wb * TB;
+    ea.N = p.NB;
+    forward_epilogue_rows_agpr<Mma, TA, TB, false, SMOE_ACT_SWIGLU>(region, opaque_lane(), ea);
+    if (r + 1 >= rounds) break;
+    cur = nxt;
+    nxt = nn;
+    wait_lds_all();  // this wave has read its parked rows back; the loop's entry barrier then frees the two slots
+  }
   wait_vmem_all();  // the streams ran on into ring slots nobody reads: let those (empty) loads land before the end
 }
 
 template <class C>
-static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
+static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st, void* workspace = nullptr, size_t workspace_bytes = 0) {
   static LdsLimitOnce lds_limit;
   auto kern = varlen_k_kernel<C>;
   {
@@ -428,21 +560,35 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
   SMOE_REQUIRE(p.r_stride > 0 && p.r_stride < (1ll << 31) && p.s_stride > 0 && p.s_stride < (1ll << 31),
                SMOE_ERR_UNSUPPORTED, "weight-grad gemm: operand row stride out of range");
   if constexpr (C::R_GATHER != C::S_GATHER && C::BA == 256 && C::BB == 256) {
-    // the hand-scheduled loop addresses both operands with 32-bit byte offsets (the streams run a few stages past the
-    // expert's end before they stop) and tells rows past the end by a wrapped offset
+    // The tile streams on the hand-scheduled loop: whole blocks of 32 tiles per expert, a schedule table in the
+    // workspace, and 32-bit byte offsets for both operands (the streams run a few stages past an expert's end before
+    // they stop; rows past the end are told by a wrapped offset).
     const int64_t lim = (1ll << 32) - (1ll << 16);
     const int64_t r_rows = C::R_GATHER ? p.gather_rows : p.total_rows + 8 * C::BK;
     const int64_t s_rows = C::S_GATHER ? p.gather_rows : p.total_rows + 8 * C::BK;
     const bool fits = p.off != nullptr && p.gidx != nullptr && p.gather_rows > 0 && (r_rows + 1) * p.r_stride * 2 < lim &&
                       (s_rows + 1) * p.s_stride * 2 < lim && (p.total_rows + 8 * C::BK) * 4 < lim;
-    if (tuning().gemm_asm && fits) {
-      static LdsLimitOnce lds_limit_asm;
-      auto akern = varlen_k_asm_kernel<C::R_GATHER, C::S_GATHER>;
-      const int rc_a = lds_limit_asm.ensure((const void*)akern, 160 * 1024);
-      if (rc_a) return rc_a;
-      hipLaunchKernelGGL(akern, dim3((unsigned)grid), dim3(256), 160 * 1024, st, p);
-      SMOE_LAUNCH_CHECK();
-      return SMOE_OK;
+    BlockShape bs;
+    bs.bb = p.tiles_b < 8 ? p.tiles_b : 8;
+    bs.ba = 32 / bs.bb;
+    const bool whole_blocks = 32 % bs.bb == 0 && p.tiles_b % bs.bb == 0 && p.tiles_a % bs.ba == 0;
+    if (tuning().gemm_asm && fits && whole_blocks && p.E <= SCHED_MAX_E && workspace != nullptr) {
+      bs.nbj = p.tiles_b / bs.bb;
+      bs.nb = (p.tiles_a / bs.ba) * bs.nbj;
+      const int64_t blocks_total = (int64_t)bs.nb * p.E;
+      if (block_schedule_bytes(blocks_total) <= workspace_bytes && blocks_total < (1ll << 30)) {
+        const int max_rounds = (int)((blocks_total + 7) / 8 + 1);
+        static LdsLimitOnce lds_limit_asm;
+        auto akern = varlen_k_stream_kernel<C::R_GATHER, C::S_GATHER>;
+        const int rc_a = lds_limit_asm.ensure((const void*)akern, 160 * 1024);
+        if (rc_a) return rc_a;
+        hipLaunchKernelGGL(build_block_schedule_kernel, dim3(1), dim3(1024), 0, st, p.off, p.order, p.E, bs.nb, max_rounds,
+                           (int32_t*)workspace);
+        SMOE_LAUNCH_CHECK();
+        hipLaunchKernelGGL(akern, dim3(256), dim3(256), 160 * 1024, st, p, bs, (const int32_t*)workspace, max_rounds);
+        SMOE_LAUNCH_CHECK();
+        return SMOE_OK;
+      }
     }
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
@@ -452,8 +598,9 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st) {
 
 // 256 x 256 output tile, 8 wavefronts as 2 x 4, 64 token rows per stage, double buffer
 template <bool RG, bool SG>
-static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st) {
-  return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 64, 2>>(p, st);
+static int launch_varlen_k_variant(const VarlenKParams& p, hipStream_t st, void* workspace = nullptr,
+                                   size_t workspace_bytes = 0) {
+  return launch_varlen_k<KCfg<256, 256, 2, 4, RG, SG, 64, 2>>(p, st, workspace, workspace_bytes);
 }
 
 int launch_dz(const void* dout, const void* z, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row, void* dz,
@@ -536,7 +683,8 @@ extern "C" int smoe_down_projection_backward(const void* dout, const void* z, co
   p.order = expert_schedule_order;
   p.total_rows = TK;
   p.gather_rows = T;
-  return launch_varlen_k_variant<true, false>(p, st);
+  // the schedule table may take the place of the tile map: the activation-gradient GEMM that used it ran before
+  return launch_varlen_k_variant<true, false>(p, st, workspace, workspace_bytes);
 }
 
 extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_t w1_stride_e, int64_t w1_stride_row,
@@ -581,7 +729,8 @@ extern "C" int smoe_up_projection_backward(const void* x, const void* w1, int64_
     p.order = expert_schedule_order;
     p.total_rows = TK;
     p.gather_rows = T;
-    rc = launch_varlen_k_variant<false, true>(p, st);
+    // the schedule table shares the workspace with the tile map the dx GEMM builds afterwards, in stream order
+    rc = launch_varlen_k_variant<false, true>(p, st, workspace, workspace_bytes);
     if (rc) return rc;
   }
   if (TK > 0 && dx_expanded) {

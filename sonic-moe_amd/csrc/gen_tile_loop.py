@@ -340,26 +340,37 @@ def srange(lo: int, n: int) -> str:
 #   gathered   a wave's 16 token rows of a stage come with one scalar buffer load of 16 indices (range-checked against
 #              the index array), requested right behind the previous stage's loads; entries past the expert's end are
 #              replaced by -1, whose byte offset wraps to just below 4 GiB: out of range, zeros
-# Same pipeline, ring and waits as above; one tile per statement, no hand-over to a next tile: past the tile's last
-# stage the streams request rows past the expert's end, i.e. nothing.
-MV_PV, MV_QV = 128, 136          # in place: per-lane byte offsets of the 8 loads; gathered: the column part only
-MV_PRA, MV_QRA = 144, 160        # 16 + 16 fragment read addresses: slot-relative outside the statement
-MV_T, MV_HALF = 176, 178         # two scratch offsets; 1 in the upper half-wave (a load covers two token rows)
-MV_LAST = 178
-MS_PRSRC, MS_QRSRC, MS_GRSRC = 40, 44, 48
-MS_PSOFF, MS_QSOFF, MS_PSTEP, MS_QSTEP, MS_RLEFT, MS_NMID = 52, 53, 54, 55, 56, 57
-MS_PFILL, MS_QFILL, MS_LDSP, MS_LDSQ, MS_WLDS = 58, 59, 60, 61, 62
-MS_PCUR, MS_QCUR, MS_PFW, MS_QFW, MS_QFWN, MS_CNT, MS_T0, MS_T1, MS_DP, MS_DQ = 63, 64, 65, 66, 67, 68, 69, 70, 71, 72
-MS_A0, MS_A1 = 73, 74            # scratch of the gathered operand's address arithmetic
-MS_TOK = 76
+# Same pipeline, ring and waits as above.  A tile has at least three stages (shorter experts are padded with stages
+# past their end, which read nothing); a stream that has requested its tile's last stage takes over the next tile's
+# offsets, extent, first stage and stage count, so the ring runs on across tiles of different length.
+MV_PV, MV_QV, MV_PVN, MV_QVN = 128, 136, 144, 152  # in place: per-lane byte offsets of the 8 loads; gathered: column part
+MV_PRA, MV_QRA = 160, 176        # 16 + 16 fragment read addresses: slot-relative outside the statement
+MV_T, MV_HALF = 192, 194         # two scratch offsets; 1 in the upper half-wave (a load covers two token rows)
+MV_LAST = 194
+MS_PRSRC, MS_QRSRC, MS_GRSRC = 24, 28, 32
+# state (in/out, one 8-tuple): offsets of the two streams, rows left at the next index run, stages left to request in
+# the streams' tiles, the slots to refill
+MS_ST = 36
+MS_PSOFF, MS_QSOFF, MS_RLEFT, MS_PLEFT, MS_QLEFT, MS_PFILL, MS_QFILL = 36, 37, 38, 39, 40, 41, 42
+# next tile (in, one 8-tuple): first offsets, extents of the operand read in place, rows at the first index run, stages
+MS_NX = 44
+MS_PSOFFN, MS_QSOFFN, MS_PEXTN, MS_QEXTN, MS_RLEFTN, MS_SNEXT = 44, 45, 46, 47, 48, 49
+# geometry (in, one 8-tuple)
+MS_GEO = 52
+MS_PSTEP, MS_QSTEP, MS_NMID, MS_LDSP, MS_LDSQ, MS_WLDS = 52, 53, 54, 55, 56, 57
+MS_PCUR, MS_QCUR, MS_PFW, MS_QFW, MS_QFWN, MS_CNT, MS_T0, MS_T1, MS_DP, MS_DQ = 60, 61, 62, 63, 64, 65, 66, 67, 68, 69
+MS_A0, MS_A1 = 70, 71            # scratch of the gathered operand's address arithmetic
+MS_TOK = 72
 MS_LAST = MS_TOK + 15
 RPW = 2 * P_INSTR  # token rows a wave requests per stage and operand
 
 
 def mm_regs(which: str):
     if which == "p":
-        return dict(v=MV_PV, rsrc=MS_PRSRC, soff=MS_PSOFF, step=MS_PSTEP, fw=MS_PFW)
-    return dict(v=MV_QV, rsrc=MS_QRSRC, soff=MS_QSOFF, step=MS_QSTEP, fw=MS_QFW)
+        return dict(v=MV_PV, vn=MV_PVN, rsrc=MS_PRSRC, soff=MS_PSOFF, soffn=MS_PSOFFN, extn=MS_PEXTN, step=MS_PSTEP,
+                    fw=MS_PFW, left=MS_PLEFT)
+    return dict(v=MV_QV, vn=MV_QVN, rsrc=MS_QRSRC, soff=MS_QSOFF, soffn=MS_QSOFFN, extn=MS_QEXTN, step=MS_QSTEP,
+                fw=MS_QFW, left=MS_QLEFT)
 
 
 def mm_fragment_reads(setno: int, ks: int) -> list[str]:
@@ -426,15 +437,35 @@ def mm_load(which: str, i: int, gathered: bool) -> tuple[list[str], list[str], l
     return pre2, pre1, [f"buffer_load_dwordx4 v{vt}, s[{r['rsrc']}:{r['rsrc'] + 3}], 0 offen lds"]
 
 
-def mm_after_issue(which: str, gathered: bool) -> list[str]:
+def mm_after_issue(em: Emitter, which: str, gathered: bool, hand_over: bool = True) -> list[str]:
+    """behind a stage's loads: move the stream along the rows; behind the tile's last stage take over the next tile"""
     r = mm_regs(which)
+    out = []
     if not gathered:
-        return [f"s_add_u32 s{r['soff']}, s{r['soff']}, s{r['step']}"]
+        out.append(f"s_add_u32 s{r['soff']}, s{r['soff']}, s{r['step']}")
+    if hand_over:
+        lab = em.label("next")
+        out += [f"s_sub_u32 s{r['left']}, s{r['left']}, 1", f"s_cmp_lg_u32 s{r['left']}, 0", f"s_cbranch_scc1 {lab}"]
+        out += [f"v_mov_b32 v{r['v'] + i}, v{r['vn'] + i}" for i in range(P_INSTR)]
+        out += [f"s_mov_b32 s{r['soff']}, s{r['soffn']}", f"s_mov_b32 s{r['left']}, s{MS_SNEXT}"]
+        if gathered:
+            out.append(f"s_mov_b32 s{MS_RLEFT}, s{MS_RLEFTN}")
+        else:
+            out.append(f"s_mov_b32 s{r['rsrc'] + 2}, s{r['extn']}")
+        out.append(f"{lab}:")
+    return out
+
+
+def mm_request_run(which: str) -> list[str]:
+    """request the 16 indices of the stage the gathered stream loads next.  Scalar loads share a counter with the LDS
+    reads and return out of order with them, so the next wait for fragment reads is a wait for this load as well: it is
+    issued right BEHIND such a wait, with a whole k-slice to land before the following one."""
+    r = mm_regs(which)
     return [f"s_buffer_load_dwordx16 s[{MS_TOK}:{MS_TOK + 15}], s[{MS_GRSRC}:{MS_GRSRC + 3}], s{r['soff']}",
             f"s_add_u32 s{r['soff']}, s{r['soff']}, {4 * BK}"]
 
 
-def mm_issue_now(em: Emitter, which: str, gathered: bool) -> None:
+def mm_issue_now(em: Emitter, which: str, gathered: bool, hand_over: bool = True) -> None:
     """a whole stage of stream `which` into the slot its fill address names, outside the matrix-instruction stream"""
     if gathered:
         em("s_waitcnt lgkmcnt(0)")
@@ -447,7 +478,7 @@ def mm_issue_now(em: Emitter, which: str, gathered: bool) -> None:
         em("s_nop 0")
         for ln in ld:
             em(ln)
-    for ln in mm_after_issue(which, gathered):
+    for ln in mm_after_issue(em, which, gathered, hand_over):
         em(ln)
 
 
@@ -465,6 +496,9 @@ def mm_emit_stage(em: Emitter, gp: bool, gq: bool, kind: str) -> None:
     ex: dict[int, list[str]] = {-1: ["s_waitcnt lgkmcnt(0)"]}
     for at, line in zip(reads_at, mm_fragment_reads(1, 1)):
         add_extra(ex, at, [line])
+    if gp:
+        # indices of the token-side stage this stage's k-slice 1 requests (the last stage: the next entry's)
+        add_extra(ex, -1, mm_request_run("p"))
     if kind != "first":
         # the weight-side stage Q(s+2) goes into the slot the previous stage vacated
         if gq:
@@ -474,7 +508,7 @@ def mm_emit_stage(em: Emitter, gp: bool, gq: bool, kind: str) -> None:
             add_extra(ex, at - 2, pre2)
             add_extra(ex, at - 1, pre1)
             add_extra(ex, at, ld)
-        add_extra(ex, q_at[-1] + 1, mm_after_issue("q", gq))
+        add_extra(ex, q_at[-1] + 1, mm_after_issue(em, "q", gq))
     if kind != "last":
         slots = mm_next_slots()
         at = max(reads_at) + 1
@@ -493,6 +527,9 @@ def mm_emit_stage(em: Emitter, gp: bool, gq: bool, kind: str) -> None:
     em("s_barrier")
     # ---- k-slice 1 on set B
     ex = {}
+    if gq:
+        # indices of the weight-side stage the next stage's k-slice 0 requests (the last stage: the next entry's)
+        add_extra(ex, -1, mm_request_run("q"))
     if kind != "last":
         for at, line in zip(reads_at, mm_fragment_reads(0, 0)):
             add_extra(ex, at, [line])
@@ -503,26 +540,34 @@ def mm_emit_stage(em: Emitter, gp: bool, gq: bool, kind: str) -> None:
             add_extra(ex, at - 2, pre2)
             add_extra(ex, at - 1, pre1)
             add_extra(ex, at, ld)
-        add_extra(ex, p_at[-1] + 1, mm_after_issue("p", gp))
+        add_extra(ex, p_at[-1] + 1, mm_after_issue(em, "p", gp))
     emit_kslice(em, 1, False, ex)
 
 
 def mm_emit_prologue(gp: bool, gq: bool) -> list[str]:
-    """before the first statement of a tile: P(0) into token slot 1, Q(0), Q(1) into weight slots 1, 2 (the statement's
-    entry then requests P(1), Q(2) into the slots 0 / 0 it is told are vacant)"""
+    """before the first statement of a workgroup: P(0) into token slot 1, Q(0), Q(1) into weight slots 1, 2 (the
+    statement's entry then requests P(1), Q(2) into the slots 0 / 0 it is told are vacant); leaves the index run of the
+    gathered stream's next stage requested and landed"""
     em = Emitter()
-    if gp or gq:
-        r = mm_regs("p" if gp else "q")
-        em(f"s_buffer_load_dwordx16 s[{MS_TOK}:{MS_TOK + 15}], s[{MS_GRSRC}:{MS_GRSRC + 3}], s{r['soff']}")
-        em(f"s_add_u32 s{r['soff']}, s{r['soff']}, {4 * BK}")
+    req = lambda which: [em(ln) for ln in mm_request_run(which)]
+    if gp:
+        req("p")
     em(f"s_add_u32 s{MS_PFW}, s{MS_LDSP}, s{MS_WLDS}")
     em(f"s_add_u32 s{MS_PFW}, s{MS_PFW}, {P_STAGE}")
-    mm_issue_now(em, "p", gp)
+    mm_issue_now(em, "p", gp, False)
+    if gp:
+        req("p")
+    if gq:
+        req("q")
     em(f"s_add_u32 s{MS_QFW}, s{MS_LDSQ}, s{MS_WLDS}")
     em(f"s_add_u32 s{MS_QFW}, s{MS_QFW}, {Q_STAGE}")
-    mm_issue_now(em, "q", gq)
+    mm_issue_now(em, "q", gq, False)
+    if gq:
+        req("q")
     em(f"s_add_u32 s{MS_QFW}, s{MS_QFW}, {Q_STAGE}")
-    mm_issue_now(em, "q", gq)
+    mm_issue_now(em, "q", gq, False)
+    if gq:
+        req("q")
     em("s_waitcnt vmcnt(0) lgkmcnt(0)")
     return em.lines
 
@@ -571,15 +616,13 @@ def mm_emit_tile(gp: bool, gq: bool) -> list[str]:
 
 def mm_operands():
     outs = [
-        (vrange(MV_PRA, 2 * FM), "pra"), (vrange(MV_QRA, 2 * FN), "qra"), (srange(MS_PSOFF, 1), "psoff"),
-        (srange(MS_QSOFF, 1), "qsoff"), (srange(MS_RLEFT, 1), "rleft"), (srange(MS_PFILL, 1), "pfill"),
-        (srange(MS_QFILL, 1), "qfill"),
+        (vrange(MV_PRA, 2 * FM), "pra"), (vrange(MV_QRA, 2 * FN), "qra"), (vrange(MV_PV, P_INSTR), "pv"),
+        (vrange(MV_QV, Q_INSTR), "qv"), (srange(MS_PRSRC, 4), "prsrc"), (srange(MS_QRSRC, 4), "qrsrc"),
+        (srange(MS_ST, 8), "state"),
     ]
     ins = [
-        (vrange(MV_PV, P_INSTR), "pv"), (vrange(MV_QV, Q_INSTR), "qv"), (vrange(MV_HALF, 1), "half"),
-        (srange(MS_PRSRC, 4), "prsrc"), (srange(MS_QRSRC, 4), "qrsrc"), (srange(MS_GRSRC, 4), "grsrc"),
-        (srange(MS_PSTEP, 1), "pstep"), (srange(MS_QSTEP, 1), "qstep"), (srange(MS_NMID, 1), "nmid"),
-        (srange(MS_LDSP, 1), "ldsp"), (srange(MS_LDSQ, 1), "ldsq"), (srange(MS_WLDS, 1), "wlds"),
+        (vrange(MV_PVN, P_INSTR), "pvn"), (vrange(MV_QVN, Q_INSTR), "qvn"), (vrange(MV_HALF, 1), "half"),
+        (srange(MS_GRSRC, 4), "grsrc"), (srange(MS_NX, 8), "next"), (srange(MS_GEO, 8), "geo"),
     ]
     return outs, ins
 
@@ -600,6 +643,17 @@ def mm_statement(name: str, lines: list[str], with_matrix: bool) -> str:
     cl = [", ".join(f'"{c}"' for c in clob[i:i + 16]) for i in range(0, len(clob), 16)]
     body.append("    : " + ", \\\n      ".join(cl) + ")")
     return "\n".join(body)
+
+
+def mm_layout_defines() -> list[str]:
+    """positions inside the three scalar 8-tuples, for the C++ side"""
+    names = dict(PSOFF=MS_PSOFF - MS_ST, QSOFF=MS_QSOFF - MS_ST, RLEFT=MS_RLEFT - MS_ST, PLEFT=MS_PLEFT - MS_ST,
+                 QLEFT=MS_QLEFT - MS_ST, PFILL=MS_PFILL - MS_ST, QFILL=MS_QFILL - MS_ST,
+                 PSOFFN=MS_PSOFFN - MS_NX, QSOFFN=MS_QSOFFN - MS_NX, PEXTN=MS_PEXTN - MS_NX, QEXTN=MS_QEXTN - MS_NX,
+                 RLEFTN=MS_RLEFTN - MS_NX, SNEXT=MS_SNEXT - MS_NX,
+                 PSTEP=MS_PSTEP - MS_GEO, QSTEP=MS_QSTEP - MS_GEO, NMID=MS_NMID - MS_GEO, LDSP=MS_LDSP - MS_GEO,
+                 LDSQ=MS_LDSQ - MS_GEO, WLDS=MS_WLDS - MS_GEO)
+    return [f"#define SMOE_MM_{k} {v}" for k, v in names.items()]
 
 
 def statement(name: str, qmn: bool) -> str:
@@ -652,7 +706,9 @@ def header() -> str:
         "",
         statement("SMOE_TILE_LOOP_KM", True),
         "",
-        "// weight-gradient loop: token operand in place, weight-side operand gathered (dW1) and the other way round (dW2)",
+        "// weight-gradient loop: token operand in place, weight-side operand gathered (dW1) and the other way round (dW2);",
+        "// state / next / geo are 8-tuples of scalars, SMOE_MM_* name their elements",
+        *mm_layout_defines(),
         mm_statement("SMOE_TILE_PROLOGUE_MM_QG", mm_emit_prologue(False, True), False),
         "",
         mm_statement("SMOE_TILE_LOOP_MM_QG", mm_emit_tile(False, True), True),

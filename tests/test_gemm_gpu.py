@@ -21,6 +21,9 @@ SHAPES = [
     (1500, 768, 192, 16, 4, 1.2, (3, 15)), # skewed, empty experts, N tails (2I=384, I=192 not multiples of 256)
     (4096, 1024, 512, 32, 8, 0.8, (0,)),
     (300, 64, 64, 4, 1, 0.0, ()),          # smallest supported H / I
+    # outputs that split into whole blocks of 32 tiles: the weight gradients run as tile streams on a block schedule;
+    # skewed experts of 0 .. ~20 stages, empty ones, a few rows only
+    (1536, 2048, 1024, 12, 2, 1.5, (2, 7)),
 ]
 
 

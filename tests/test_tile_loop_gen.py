@@ -88,28 +88,42 @@ def test_replay_catches_a_wrong_slot():
 
 
 # ---- weight-gradient loop ------------------------------------------------------------------------------------------------
-def _problem_mm(gp, rows, NA, NB, a0, b0, seed=0, before=37, after=90, ntok=500):
+def _problem_mm(gp, experts, NA, NB, seed=0, before=37, after=90, ntok=500, tiles_of=None):
+    """experts: row counts; the workgroup walks through one tile of every expert (a0, b0 vary), in order"""
     rng = np.random.default_rng(seed)
-    total = before + rows + after
+    total = before + sum(experts) + after
     gidx = rng.integers(0, ntok, size=total).astype(np.int64)
+    tiles, row = [], before
+    for i, n in enumerate(experts):
+        a0 = (i * 256) % (-(-NA // 256) * 256)
+        b0 = ((i + 1) * 256) % (-(-NB // 256) * 256)
+        tiles.append((row, row + n, a0, b0))
+        row += n
     return sim.ProblemMM(gp=gp, NA=NA, NB=NB, r_stride=NA + (8 if seed & 1 else 0), s_stride=NB, gather_rows=ntok,
-                         gidx_flat=gidx, row_begin=before, row_end=before + rows, a0=a0, b0=b0)
+                         gidx_flat=gidx, tiles=tiles)
 
 
 @pytest.mark.parametrize("gp", [False, True])
 @pytest.mark.parametrize("rows", [0, 1, 63, 64, 130, 192, 257, 448])
 def test_replay_weight_gradient_loop(gp, rows):
-    # experts of 0 .. 7 stages, with ragged last stages; the expert sits in the middle of the grouped rows
-    out = sim.simulate_mm(_problem_mm(gp, rows, 512, 768, 256, 512, seed=rows))
-    assert out["stages"] == max(3, -(-rows // 64)) and out["mfma"] == G.NW * 64 * 2 * out["stages"]
+    # one expert of 0 .. 7 stages with a ragged last stage, in the middle of the grouped rows
+    out = sim.simulate_mm(_problem_mm(gp, [rows], 512, 768, seed=rows))
+    assert out["mfma"] == G.NW * 64 * 2 * max(3, -(-rows // 64))
+
+
+@pytest.mark.parametrize("gp", [False, True])
+def test_replay_weight_gradient_stream(gp):
+    # a stream of tiles of different experts: long, empty, one row, ragged, exactly three stages, long
+    sim.simulate_mm(_problem_mm(gp, [300, 0, 1, 130, 192, 450, 64], 512, 768, seed=11))
+    sim.simulate_mm(_problem_mm(gp, [192, 192, 0, 0, 200], 768, 512, seed=12, before=0))
 
 
 @pytest.mark.parametrize("gp", [False, True])
 def test_replay_weight_gradient_edges(gp):
-    # the expert ends exactly at the end of the grouped rows (index loads run past the array: range-checked), ragged
-    # output tile in both directions (NA = 320, NB = 448: the last tiles have 64 resp. 192 valid columns)
-    sim.simulate_mm(_problem_mm(gp, 100, 320, 448, 256, 256, seed=5, after=0))
-    sim.simulate_mm(_problem_mm(gp, 300, 320, 448, 0, 256, seed=6, before=0, after=0))
+    # the last expert ends exactly at the end of the grouped rows (index loads run past the array: range-checked);
+    # ragged output tiles in both directions (NA = 320, NB = 448: the last tiles have 64 resp. 192 valid columns)
+    sim.simulate_mm(_problem_mm(gp, [100, 70], 320, 448, seed=5, after=0))
+    sim.simulate_mm(_problem_mm(gp, [300], 320, 448, seed=6, before=0, after=0))
 
 
 def test_replay_weight_gradient_catches_missing_fix():
@@ -118,6 +132,6 @@ def test_replay_weight_gradient_catches_missing_fix():
     G.mm_ragged_fix = lambda em: [f"s_sub_i32 s{G.MS_RLEFT}, s{G.MS_RLEFT}, {G.BK}"]
     try:
         with pytest.raises(sim.SimError):
-            sim.simulate_mm(_problem_mm(False, 100, 512, 512, 0, 0, seed=7))
+            sim.simulate_mm(_problem_mm(False, [100, 100], 512, 512, seed=7))
     finally:
         G.mm_ragged_fix = orig

@@ -96,6 +96,7 @@ class Wave:
         self.acc_seen = {}
         self.tile = None  # (expert, row0, row_end, n0) the matrix instructions work on
         self.ldsp_reg = G.S_LDSP  # register that holds the LDS address of the token operand's ring
+        self.rsrc_regs = (G.S_PRSRC, G.S_QRSRC)  # first registers of the two streams' buffer resources
         self.oob_zero = False  # loads beyond the extent write zeros (the weight-gradient loop relies on it)
         self.smem_out = set()  # scalar registers a scalar load in flight will write
         self.expect = None  # callable(wave, fn, fm, stage, ks) -> (want_q, want_p); default: the varlen-M operands
@@ -103,9 +104,9 @@ class Wave:
     # ---- memory side
     def issue_load(self, voff_reg, rsrc, soff_reg):
         lds = self.lds
-        if rsrc == G.S_PRSRC:
+        if rsrc == self.rsrc_regs[0]:
             stream = P_STREAM
-        elif rsrc == G.S_QRSRC:
+        elif rsrc == self.rsrc_regs[1]:
             stream = Q_STREAM
         else:
             raise SimError(f"load through unknown resource s{rsrc}")
@@ -552,10 +553,7 @@ class ProblemMM:
     s_stride: int
     gather_rows: int
     gidx_flat: np.ndarray  # (total_rows,) grouped row -> row of the gathered tensor
-    row_begin: int
-    row_end: int
-    a0: int
-    b0: int
+    tiles: list  # (row_begin, row_end, a0, b0) this workgroup walks through, in order
 
     @property
     def total_rows(self):
@@ -567,46 +565,73 @@ def simulate_mm(prob: ProblemMM) -> dict:
     pro, lines = G.mm_emit_prologue(gp, gq), G.mm_emit_tile(gp, gq)
     lds = Lds()
     waves = [Wave(w, lds, prob) for w in range(G.NW)]
-    S = -(-(prob.row_end - prob.row_begin) // G.BK)
-    S_eff = max(S, 3)
     rrb, srb = prob.r_stride * 2, prob.s_stride * 2
     lane = np.arange(64)
+    tiles = prob.tiles
+
+    def stages(tile):
+        return max(3, -(-(tile[1] - tile[0]) // G.BK))
 
     def clamp8(c, n):
         return np.minimum(c - c % 8, n - 8) + c % 8
 
     def expect(w, fn, fm, stage, ks):
+        row_begin, row_end, a0, b0 = w.tile
         wa, wb = w.w % 2, w.w // 2
-        m = prob.row_begin + stage * G.BK + ks * G.KSTEP + 8 * (lane // 16)[:, None] + np.arange(8)[None, :]
-        valid = m < prob.row_end
+        m = row_begin + stage * G.BK + ks * G.KSTEP + 8 * (lane // 16)[:, None] + np.arange(8)[None, :]
+        valid = m < row_end
         mc = np.minimum(m, prob.total_rows - 1)
-        b = clamp8(prob.b0 + wb * G.TN + fn * G.FR + lane % 16, prob.NB)
-        a = clamp8(prob.a0 + wa * G.TM + fm * G.FR + lane % 16, prob.NA)
+        b = clamp8(b0 + wb * G.TN + fn * G.FR + lane % 16, prob.NB)
+        a = clamp8(a0 + wa * G.TM + fm * G.FR + lane % 16, prob.NA)
         rq = prob.gidx_flat[mc] if gq else mc
         rp = prob.gidx_flat[mc] if gp else mc
         want_q = np.where(valid, (rq * prob.s_stride + b[:, None]) | (Q_STREAM << 60), ZERO)
         want_p = np.where(valid, (rp * prob.r_stride + a[:, None]) | (P_STREAM << 60), ZERO)
         return want_q, want_p
 
-    for w in waves:
-        w.ldsp_reg = G.MS_LDSP
-        w.oob_zero = True
-        w.expect = expect
-        w.tile = (0, 0, 0, 0)
-        s = w.s
-        s[G.MS_PRSRC:G.MS_PRSRC + 4] = [0, 0, (prob.gather_rows if gp else prob.row_end) * rrb, 0x20000]
-        s[G.MS_QRSRC:G.MS_QRSRC + 4] = [0, 0, (prob.gather_rows if gq else prob.row_end) * srb, 0x20000]
-        s[G.MS_GRSRC:G.MS_GRSRC + 4] = [0, 0, prob.total_rows * 4, 0x20000]
+    def lane_offsets(wv, tile):
+        row_begin, row_end, a0, b0 = tile
         pv, qv = [], []
         for i in range(G.P_INSTR):
-            kl = (w.w * G.P_INSTR + i) * 2 + lane // 32
+            kl = (wv * G.P_INSTR + i) * 2 + lane // 32
             phys16 = lane % 32
             log32 = (phys16 >> 1) ^ mnswz(kl)
             c = ((log32 << 1) | (phys16 & 1)) * 8
-            a = np.minimum(prob.a0 + c, prob.NA - 8)
-            b = np.minimum(prob.b0 + c, prob.NB - 8)
+            a = np.minimum(a0 + c, prob.NA - 8)
+            b = np.minimum(b0 + c, prob.NB - 8)
             pv.append((0 if gp else kl * rrb) + a * 2)
             qv.append((0 if gq else kl * srb) + b * 2)
+        return pv, qv
+
+    def first_offsets(wv, tile):
+        row_begin = tile[0]
+        run = (row_begin + wv * 16) * 4
+        return (run if gp else row_begin * rrb), (run if gq else row_begin * srb)
+
+    NULL = (0, 0, 0, 0)  # behind the last tile: an empty expert, every load out of range
+
+    def set_next(w, tile):
+        pvn, qvn = lane_offsets(w.w, tile)
+        for i in range(G.P_INSTR):
+            w.v[G.MV_PVN + i] = pvn[i]
+            w.v[G.MV_QVN + i] = qvn[i]
+        s = w.s
+        s[G.MS_PSOFFN], s[G.MS_QSOFFN] = first_offsets(w.w, tile)
+        s[G.MS_PEXTN], s[G.MS_QEXTN] = tile[1] * rrb, tile[1] * srb
+        s[G.MS_RLEFTN] = (tile[1] - (tile[0] + w.w * 16)) & 0xffffffff
+        s[G.MS_SNEXT] = stages(tile)
+
+    for w in waves:
+        w.ldsp_reg = G.MS_LDSP
+        w.rsrc_regs = (G.MS_PRSRC, G.MS_QRSRC)
+        w.oob_zero = True
+        w.expect = expect
+        t0 = tiles[0]
+        s = w.s
+        s[G.MS_PRSRC:G.MS_PRSRC + 4] = [0, 0, (prob.gather_rows if gp else t0[1]) * rrb, 0x20000]
+        s[G.MS_QRSRC:G.MS_QRSRC + 4] = [0, 0, (prob.gather_rows if gq else t0[1]) * srb, 0x20000]
+        s[G.MS_GRSRC:G.MS_GRSRC + 4] = [0, 0, prob.total_rows * 4, 0x20000]
+        pv, qv = lane_offsets(w.w, t0)
         for i in range(G.P_INSTR):
             w.v[G.MV_PV + i] = pv[i]
             w.v[G.MV_QV + i] = qv[i]
@@ -619,39 +644,61 @@ def simulate_mm(prob: ProblemMM) -> dict:
                 w.v[G.MV_PRA + 2 * f + h] = k * G.ROWB + ((((wa * G.TM) // 16 + f) ^ mnswz(k)) << 5) + ((i16 & 3) << 3)
                 w.v[G.MV_QRA + 2 * f + h] = k * G.ROWB + ((((wb * G.TN) // 16 + f) ^ mnswz(k)) << 5) + ((i16 & 3) << 3)
         w.v[G.MV_HALF] = lane >> 5
-        first_run = (prob.row_begin + w.w * 16) * 4
-        s[G.MS_PSOFF] = first_run if gp else prob.row_begin * rrb
-        s[G.MS_QSOFF] = first_run if gq else prob.row_begin * srb
+        s[G.MS_PSOFF], s[G.MS_QSOFF] = first_offsets(w.w, t0)
         s[G.MS_PSTEP] = rrb if gp else G.BK * rrb
         s[G.MS_QSTEP] = srb if gq else G.BK * srb
-        s[G.MS_RLEFT] = (prob.row_end - (prob.row_begin + w.w * 16)) & 0xffffffff
-        s[G.MS_NMID] = S_eff - 2
+        s[G.MS_RLEFT] = (t0[1] - (t0[0] + w.w * 16)) & 0xffffffff
         s[G.MS_LDSP], s[G.MS_LDSQ], s[G.MS_WLDS] = 0, G.P_SLOTS * G.P_STAGE, w.w * G.P_INSTR * 1024
         s[G.MS_PFILL], s[G.MS_QFILL] = 0, G.P_SLOTS * G.P_STAGE
         for _ in run_wave(w, pro):
             raise SimError("barrier in the prologue")
         if w.vmq or w.smem_out:
             raise SimError("the prologue leaves operations in flight")
+        # the prologue has requested one token stage and two weight stages of the first tile
+        s[G.MS_PLEFT], s[G.MS_QLEFT] = stages(t0) - 1, stages(t0) - 2
     saved = [(w.v[G.MV_PRA:G.MV_PRA + 16].copy(), w.v[G.MV_QRA:G.MV_QRA + 16].copy()) for w in waves]
-    gens = [run_wave(w, lines) for w in waves]
-    alive = [True] * G.NW
-    while any(alive):
-        state = []
-        for i, g in enumerate(gens):
-            try:
-                next(g)
-                state.append("barrier")
-            except StopIteration:
-                alive[i] = False
-                state.append("done")
-        if len(set(state)) != 1:
-            raise SimError(f"waves disagree at a barrier: {state}")
-    for w, (pra, qra) in zip(waves, saved):
-        if len(w.acc_seen) != G.FN * G.FM or any(v != 2 * S_eff for v in w.acc_seen.values()):
-            raise SimError(f"wave {w.w}: accumulators saw {sorted(set(w.acc_seen.values()))} k-slices, want {2 * S_eff}")
-        if w.reads_out or w.smem_out:
-            raise SimError("LDS or scalar reads in flight at the end of the statement")
-        if not ((w.v[G.MV_PRA:G.MV_PRA + 16] == pra).all() and (w.v[G.MV_QRA:G.MV_QRA + 16] == qra).all()):
-            raise SimError("read addresses do not come back slot-relative")
+    total_mfma = 0
+    for ti, tile in enumerate(tiles):
+        nxt = tiles[ti + 1] if ti + 1 < len(tiles) else NULL
+        for w in waves:
+            w.tile = tile
+            w.acc_seen = {}
+            w.s[G.MS_NMID] = stages(tile) - 2
+            set_next(w, nxt)
+        gens = [run_wave(w, lines) for w in waves]
+        alive = [True] * G.NW
+        while any(alive):
+            state = []
+            for i, g in enumerate(gens):
+                try:
+                    next(g)
+                    state.append("barrier")
+                except StopIteration:
+                    alive[i] = False
+                    state.append("done")
+            if len(set(state)) != 1:
+                raise SimError(f"waves disagree at a barrier: {state}")
+        for w, (pra, qra) in zip(waves, saved):
+            if len(w.acc_seen) != G.FN * G.FM or any(v != 2 * stages(tile) for v in w.acc_seen.values()):
+                raise SimError(f"wave {w.w}: accumulators saw {sorted(set(w.acc_seen.values()))} k-slices, want {2 * stages(tile)}")
+            if w.reads_out or w.smem_out:
+                raise SimError("LDS or scalar reads in flight at the end of the statement")
+            if not ((w.v[G.MV_PRA:G.MV_PRA + 16] == pra).all() and (w.v[G.MV_QRA:G.MV_QRA + 16] == qra).all()):
+                raise SimError("read addresses do not come back slot-relative")
+        total_mfma += G.NW * 64 * 2 * stages(tile)
+        # epilogue: parks rows in the two vacated slots
+        for w in waves:
+            slot = w.s[G.MS_PFILL] if w.w < 2 else w.s[G.MS_QFILL]
+            for piece in range(slot // PIECE, (slot + G.P_STAGE) // PIECE):
+                if lds.pending[piece] is not None:
+                    raise SimError(f"epilogue parks in piece {piece} with a load in flight")
+                for o in waves:
+                    if o.w != w.w and lds.last_read[o.w][piece] >= w.phase:
+                        raise SimError(f"epilogue of wave {w.w} parks in piece {piece} wave {o.w} may still read")
+                lds.tag[piece * 512:(piece + 1) * 512] = -2
+    for w in waves:
         w.wait_vm(0)
-    return dict(mfma=sum(w.mfma_count for w in waves), barriers=waves[0].nbarrier, stages=S_eff)
+    got = sum(w.mfma_count for w in waves)
+    if got != total_mfma:
+        raise SimError(f"{got} matrix instructions, want {total_mfma}")
+    return dict(mfma=got, barriers=waves[0].nbarrier)
