@@ -198,13 +198,54 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
     return rows
 
 
+def vendor_dense(cfg, dev, steps=5):
+    """The vendor library (hipBLASLt through torch.matmul) on the dense GEMM of the same shape as each grouped GEMM, same
+    process, warm, random bf16 data: what the machine's own best GEMM kernel does with these FLOPs when there is no
+    gather, no expert boundary and no fused epilogue.  The two weight-gradient GEMMs are E separate (N x tokens) @
+    (tokens x M) products with TK / E tokens each, launched back to back."""
+    T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
+    TK = T * K
+    bf = torch.bfloat16
+    res = {}
+
+    def rnd(*shape, scale=1.0):
+        return (torch.randn(*shape, device=dev, dtype=torch.float32) * scale).to(bf)
+
+    with torch.no_grad():
+        for name, (m, k, n) in {
+            "up_projection_forward": (TK, H, 2 * I),
+            "down_projection_forward": (TK, I, H),
+            "down_projection_backward(dz only)": (TK, H, I),
+            "up_projection_backward(dx only)": (TK, 2 * I, H),
+        }.items():
+            a, b = rnd(m, k), rnd(n, k, scale=0.02)
+            c = torch.empty(m, n, dtype=bf, device=dev)
+            ms, _ = time_region(lambda: torch.matmul(a, b.t(), out=c), steps, 2)
+            res[name] = round(2.0 * m * k * n / ms / 1e9, 1)
+            del a, b, c
+        tok = TK // E
+        for name, (n, m) in {"up_projection_backward(dW1 only)": (2 * I, H), "dW2": (H, I)}.items():
+            a, b = rnd(TK, n), rnd(TK, m)
+            c = torch.empty(E, n, m, dtype=bf, device=dev)
+
+            def per_expert():
+                for e in range(E):
+                    torch.matmul(a[e * tok:(e + 1) * tok].t(), b[e * tok:(e + 1) * tok], out=c[e])
+
+            ms, _ = time_region(per_expert, max(2, steps // 2), 1)
+            res[name] = round(2.0 * TK * n * m / ms / 1e9, 1)
+            del a, b, c
+    torch.cuda.empty_cache()
+    return res
+
+
 # operators that are one grouped-GEMM kernel launch (plus a ~5 us tile-map builder), and the kernel they launch
 SINGLE_KERNEL_OPS = {
-    "up_projection_forward": "varlen_m_stream_kernel<up-projection forward>",
-    "down_projection_forward": "varlen_m_stream_kernel<down-projection forward>",
-    "down_projection_backward(dz only)": "varlen_m_stream_kernel<dz>",
-    "up_projection_backward(dW1 only)": "varlen_k_kernel<dW1>",
-    "up_projection_backward(dx only)": "varlen_m_stream_kernel<dx_expanded>",
+    "up_projection_forward": "varlen_m_asm_kernel<up-projection forward>",
+    "down_projection_forward": "varlen_m_asm_kernel<down-projection forward>",
+    "down_projection_backward(dz only)": "varlen_m_asm_kernel<dz>",
+    "up_projection_backward(dW1 only)": "varlen_k_stream_kernel<dW1>",
+    "up_projection_backward(dx only)": "varlen_m_asm_kernel<dx_expanded>",
     "fp8:up_projection_forward(+quantised y1)": "fp8_stream_kernel<up-projection forward>",
     "fp8:down_projection_forward": "fp8_stream_kernel<down-projection forward>",
     "fp8:down_projection_backward(dz, +quantised dz)": "fp8_varlen_m_kernel<dz>",
@@ -476,6 +517,15 @@ def main():
 
     rows = [] if (a.no_breakdown or rounding) else kernel_breakdown(cfg, t["x"], t["wr"], t["w1"], t["w2"], t["dout"],
                                                                     max(5, a.steps // 2))
+    if rows and not a.no_other_configs:
+        # the vendor library's dense rate on each grouped GEMM's shape: a same-box, same-run ceiling per kernel
+        ceil = vendor_dense(cfg, dev)
+        for r in rows:
+            if r["op"] in ceil:
+                r["vendor_dense_tflops"] = ceil[r["op"]]
+            elif r["op"] == "down_projection_backward(dz+dW2)":
+                r["vendor_dense_tflops_dW2"] = ceil["dW2"]
+        log("vendor dense GEMM (hipBLASLt) on the same shapes: " + ", ".join(f"{k} {v:.0f}" for k, v in ceil.items()))
     # dominant kernel = the single grouped-GEMM launch with the largest average duration
     single = [r for r in rows if r["op"] in SINGLE_KERNEL_OPS and not r["op"].startswith("fp8:")]
     roofline = None

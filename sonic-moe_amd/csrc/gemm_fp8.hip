@@ -78,6 +78,7 @@ struct Fp8Params {
   int64_t p_stride;  // bytes
   const uint32_t* p_scales;
   int64_t p_rows;    // rows of the P scale table (T or TK)
+  int64_t data_rows; // rows of the P data operand = the range of gidx (0: the same as p_rows)
   const int32_t* gidx;
   int scales_grouped;  // the P scale table is in grouped row order although the data rows are gathered
   const uint8_t* Q;
@@ -128,6 +129,8 @@ struct Fp8Cfg {
   static_assert(STREAM_SMEM <= 160 * 1024, "LDS budget of a CU");
   static_assert(S_INSTR * NW * 64 == BM + BN, "the scale rows must split evenly over the wavefronts");
   static_assert(SMEM <= 160 * 1024, "LDS budget of a CU");
+  // smoe_dz_partial_cols() sizes the score-gradient partial sums for both the bf16 and the fp8 dz kernel
+  static_assert(BN == 256 && WN == 4, "the partial sums' pitch is four columns per 256-column tile");
 };
 
 // direct-to-LDS load of one 32-bit word per lane through a buffer resource: the wavefront's 64 words land at
@@ -292,9 +295,6 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
       const bool by_index = p.gidx != nullptr && !p.scales_grouped;
       s_rsrc[j] = make_buffer_resource(by_index ? p.p_scales : p.p_scales + row0);
       s_voff[j] = (by_index ? (uint32_t)p.gidx[m] : (uint32_t)(m - row0)) * 4u;
-#ifdef SMOE_PROBE_SCALES_CONTIG
-      s_voff[j] = (uint32_t)lane * 4u;
-#endif
       s_step[j] = (uint32_t)p.p_rows * 4u;
     } else {
       int n = n0 + r0 - C::BM + lane;
@@ -343,10 +343,8 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
       buffer_load16_to_lds(q_rsrc, q_voff[j], (uint32_t)s * C::BKB, base + C::P_STAGE + (wave * C::Q_INSTR + j) * 1024);
     } else {
       constexpr int j = i - C::P_INSTR - C::Q_INSTR;
-#ifndef SMOE_PROBE_NO_SCALE_LOADS
       buffer_load4_to_lds(s_rsrc[j], s_voff[j], (uint32_t)s * s_step[j],
                           base + C::P_STAGE + C::Q_STAGE + (wave * C::S_INSTR + j) * 256);
-#endif
     }
   };
   auto load = [&](int buf, int /*s*/, auto step_c, Fp8Frag(&qf)[FN], Fp8Frag(&pf)[C::NP]) {
@@ -359,11 +357,7 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
       const i32x4 lo = *(const i32x4*)(st + p_off[ks][0] + fm * 32 * C::BKB);
       const i32x4 hi = *(const i32x4*)(st + p_off[ks][1] + fm * 32 * C::BKB);
       pf[pp].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#ifdef SMOE_PROBE_NO_SCALE_READS
-      pf[pp].scale = 127;
-#else
       pf[pp].scale = (int)(*(const uint32_t*)(st + ps_off + fm * 32 * 4) >> shift);
-#endif
     }
     if constexpr (Fp8Mma::reads_q(step)) {
 #pragma unroll
@@ -371,11 +365,7 @@ __global__ __launch_bounds__(Fp8Cfg::NT) void fp8_varlen_m_kernel(const Fp8Param
         const i32x4 lo = *(const i32x4*)(st + q_off[ks][0] + fn * 32 * C::BKB);
         const i32x4 hi = *(const i32x4*)(st + q_off[ks][1] + fn * 32 * C::BKB);
         qf[fn].data = i32x8{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-#ifdef SMOE_PROBE_NO_SCALE_READS
-        qf[fn].scale = 127;
-#else
         qf[fn].scale = (int)(*(const uint32_t*)(st + qs_off + fn * 32 * 4) >> shift);
-#endif
       }
     }
   };
@@ -649,7 +639,8 @@ static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t
   if (DZ) p.ds_cols = p.n_tiles * C::WN;
   // the kernel addresses its operands with 32-bit byte offsets from a buffer base
   const int64_t lim = 1ll << 32;
-  SMOE_REQUIRE((p.gidx ? p.p_rows : (int64_t)C::BM) * p.p_stride < lim && (int64_t)p.N * p.q_stride_row < lim &&
+  const int64_t data_rows = p.data_rows ? p.data_rows : p.p_rows;
+  SMOE_REQUIRE((p.gidx ? data_rows : (int64_t)C::BM) * p.p_stride < lim && (int64_t)p.N * p.q_stride_row < lim &&
                    (int64_t)(p.Kdim / C::BKB) * (p.p_rows > p.q_rows ? p.p_rows : p.q_rows) * 4 < lim,
                SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: operand too large for 32-bit offsets");
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
@@ -657,7 +648,7 @@ static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t
   SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: too many tiles");
   const Tuning& tune = tuning();
   const int64_t lim24 = 1ll << 24;  // the tile-stream kernel forms its offsets with 24-bit multiplies
-  const bool fits24 = p.p_rows < lim24 && p.p_stride < lim24 && p.N < lim24 && p.q_stride_row < lim24;
+  const bool fits24 = data_rows < lim24 && p.p_rows < lim24 && p.p_stride < lim24 && p.N < lim24 && p.q_stride_row < lim24;
   if constexpr (!DZ) if (tune.gemm_stream && p.Kdim >= 2 * C::BKB && fits24) {
     static LdsLimitOnce lds_limit_stream;
     auto skern = fp8_stream_kernel<WITH_ACT, ACT>;
@@ -831,6 +822,7 @@ static int group_token_scales(Fp8Params& p, void* workspace, size_t workspace_by
                      p.p_rows, p.gidx, dst, TK, KB);
   SMOE_LAUNCH_CHECK();
   p.p_scales = dst;
+  if (p.data_rows == 0) p.data_rows = p.p_rows;  // the data operand keeps its T rows; only the scale table is regrouped
   p.p_rows = TK;
   p.scales_grouped = 1;
   return SMOE_OK;

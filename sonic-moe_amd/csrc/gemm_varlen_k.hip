@@ -568,10 +568,17 @@ static int launch_varlen_k(const VarlenKParams& pin, hipStream_t st, void* works
     const int64_t s_rows = C::S_GATHER ? p.gather_rows : p.total_rows + 8 * C::BK;
     const bool fits = p.off != nullptr && p.gidx != nullptr && p.gather_rows > 0 && (r_rows + 1) * p.r_stride * 2 < lim &&
                       (s_rows + 1) * p.s_stride * 2 < lim && (p.total_rows + 8 * C::BK) * 4 < lim;
-    BlockShape bs;
-    bs.bb = p.tiles_b < 8 ? p.tiles_b : 8;
-    bs.ba = 32 / bs.bb;
-    const bool whole_blocks = 32 % bs.bb == 0 && p.tiles_b % bs.bb == 0 && p.tiles_a % bs.ba == 0;
+    // a block is ba x bb tiles with ba * bb = 32, as square as the tile counts allow (fewest operand panels per block)
+    BlockShape bs = {0, 0, 0, 0};
+    bool whole_blocks = false;
+    for (int bb : {8, 4, 16, 2, 32, 1}) {
+      if (p.tiles_b % bb == 0 && p.tiles_a % (32 / bb) == 0) {
+        bs.bb = bb;
+        bs.ba = 32 / bb;
+        whole_blocks = true;
+        break;
+      }
+    }
     if (tuning().gemm_asm && fits && whole_blocks && p.E <= SCHED_MAX_E && workspace != nullptr) {
       bs.nbj = p.tiles_b / bs.bb;
       bs.nb = (p.tiles_a / bs.ba) * bs.nbj;

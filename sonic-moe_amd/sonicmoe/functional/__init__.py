@@ -231,12 +231,20 @@ def largest_first_schedule_order(expert_frequency_offset: torch.Tensor) -> torch
     return torch.argsort(counts, descending=True, stable=True).to(torch.int32)
 
 
-def _fp8_backward_requested(b1, b2) -> bool:
-    """The fp8-backward switch as it stands while the forward pass runs (the backward pass may run outside the block)."""
+def _fp8_backward_requested(b1, b2, w1=None, w2=None) -> bool:
+    """The fp8-backward switch as it stands while the forward pass runs (the backward pass may run outside the block).
+    What the fp8 backward cannot do is refused here, in forward, not in the middle of a backward pass: biases, and
+    weight shapes whose transposed quantised copies do not split into 128-element blocks.  (The fp8 kernels take the
+    experts in index order: an expert_schedule policy only reorders the bf16 weight-gradient GEMMs of such a step.)"""
     if not is_using_fp8_backward():
         return False
     if b1 is not None or b2 is not None:
         raise NotImplementedError("enable_fp8_backward: layers with biases are not supported")
+    if w1 is not None and (w1.size(0) % 128 != 0 or w1.size(1) % 128 != 0):
+        # the activation gradients contract over the up-projection's output columns (dx) and over H (dz): both are
+        # quantised in blocks along those indices
+        raise NotImplementedError(
+            f"enable_fp8_backward: up-projection width {w1.size(0)} and hidden size {w1.size(1)} must be multiples of 128")
     return True
 
 
@@ -376,7 +384,7 @@ class _ExpertsFunction(torch.autograd.Function):
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K,
                                 activation_type, stream_id, inference, order)
         ctx.order = order
-        ctx.fp8_backward = _fp8_backward_requested(b1, b2)
+        ctx.fp8_backward = _fp8_backward_requested(b1, b2, w1, w2)
         if not inference:
             ctx.save_for_backward(x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K_or_maxK, is_varlen_K, activation_type, stream_id, inference, b1 is not None)
@@ -426,8 +434,10 @@ class _TCLayerFunction(torch.autograd.Function):
             router_logits = torch.empty(T, E, dtype=x.dtype, device=x.device)
             colsum = torch.empty(router_fused_partials(T, E), E, dtype=torch.float32, device=x.device)
             _router_forward_fused(x, router_w.contiguous(), router_logits, scores, indices, colsum)
-            # picked up by switch_loss() when it is handed this very tensor (MoE.forward does that)
-            router_logits._smoe_softmax_colsum_partials = (colsum, router_logits._version)
+            # picked up by switch_loss() when it is handed this very tensor (MoE.forward does that).  Under torch.compile
+            # a tensor attribute does not survive tracing: the loss then takes its own pass over the logits.
+            if not torch.compiler.is_compiling():
+                router_logits._smoe_softmax_colsum_partials = (colsum, router_logits._version)
         else:
             router_logits = F.linear(x, router_w)
             _softmax_topk_fwd(router_logits, scores, indices, E, K)
@@ -437,7 +447,7 @@ class _TCLayerFunction(torch.autograd.Function):
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K, False, activation_type,
                                 stream_id, inference, order)
         ctx.order = order
-        ctx.fp8_backward = _fp8_backward_requested(b1, b2)
+        ctx.fp8_backward = _fp8_backward_requested(b1, b2, w1, w2)
         if not inference:
             ctx.save_for_backward(x, router_w, w1, w2, b2, z, scores, indices, off, gidx, sidx, ridx, tok_off)
         ctx.cfg = (K, activation_type, stream_id, inference, router_logits.dtype, b1 is not None)

@@ -99,3 +99,26 @@ def test_layer_with_fused_router(dev):
     out3, aux3 = moe(x)
     g_aux0 = torch.autograd.grad(aux3, [moe.router.weight])[0]
     assert rel_l2(g_aux, g_aux0) < 2e-2
+
+
+@pytest.mark.gpu
+def test_fused_router_hands_its_column_sums_to_the_loss(dev, monkeypatch):
+    """Inside `with fused_router(): moe(x)` the auxiliary loss is formed from the column sums the router kernel wrote
+    (one pass over x), not from a second pass over the logits; outside it the stand-alone pass runs."""
+    import sonicmoe.functional as SF
+    from sonicmoe import MoE
+    from sonicmoe.enums import ActivationType
+
+    calls = {"partials": 0, "full": 0}
+    real_p, real_f = SF._switch_loss_from_partials, SF._switch_loss_fwd
+    monkeypatch.setattr(SF, "_switch_loss_from_partials", lambda *a: (calls.__setitem__("partials", calls["partials"] + 1), real_p(*a))[1])
+    monkeypatch.setattr(SF, "_switch_loss_fwd", lambda *a: (calls.__setitem__("full", calls["full"] + 1), real_f(*a))[1])
+    torch.manual_seed(3)
+    moe = MoE(32, 4, 1024, 256, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+    x = torch.randn(1024, 1024, device=dev).to(torch.bfloat16)
+    with SF.fused_router():
+        _, aux = moe(x)
+    assert calls == {"partials": 1, "full": 0}
+    _, aux0 = moe(x)
+    assert calls == {"partials": 1, "full": 1}
+    assert abs(float(aux) - float(aux0)) < 1e-3 * abs(float(aux0))
