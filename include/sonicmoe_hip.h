@@ -314,6 +314,14 @@ int smoe_down_projection_forward_fp8(const void* y1q, const void* y1_scales, con
 int smoe_mx_quantize_transposed(const void* src, int64_t src_stride_e, int64_t src_stride_r, int E, int R, int C,
                                 void* q, void* scales, void* stream);
 
+/* Both quantised copies of E weight matrices from ONE pass over them (no counterpart in the reference, which has no
+ * fp8 path): q_rows (E * R, C) / scales_rows (C / 128, E * R) exactly as smoe_mx_quantize(src viewed as (E * R, C))
+ * writes them - the forward GEMMs' operand - and q_t / scales_t exactly as smoe_mx_quantize_transposed writes them -
+ * the activation-gradient GEMMs' operand.  R % 128 == 0, C % 128 == 0.  A training step that runs forward and backward
+ * on fp8 operands calls this once per weight in forward and keeps the transposed copy for its backward pass. */
+int smoe_mx_quantize_both(const void* src, int64_t src_stride_e, int64_t src_stride_r, int E, int R, int C,
+                          void* q_rows, void* scales_rows, void* q_t, void* scales_t, void* stream);
+
 /* The activation-gradient half of smoe_down_projection_backward with fp8 operands (no counterpart in the reference,
  * whose sonicmoe::_down_projection_backward, sonicmoe/functional/backward.py:286-461, is bf16):
  *   dy1 = doutq[x_gather_idx] w2tq[e]^T with the block scales applied (never stored), then as the bf16 operator:

@@ -704,10 +704,13 @@ static int launch_fp8_dz(int act, Fp8Params& p, const int32_t* off, void* ws, in
 // transposes, quantised along R (32 consecutive r share a scale); scales (R / 128, E * C) words as in mx_quantize.
 // One workgroup transposes a 128 (r) x 64 (c) tile through LDS: row-contiguous loads, column reads (one lane = one
 // column and one 32-row block), bytes parked transposed, row-contiguous stores of 128 bytes per output row.
+template <bool BOTH>
 __global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint16_t* __restrict__ src,
                                                                      int64_t src_stride_e, int64_t src_stride_r, int R,
                                                                      int C, int E, uint8_t* __restrict__ q,
-                                                                     uint32_t* __restrict__ scales) {
+                                                                     uint32_t* __restrict__ scales,
+                                                                     uint8_t* __restrict__ q_rows,
+                                                                     uint8_t* __restrict__ scales_rows) {
   constexpr int TR = 128, TC = 64, IN_PITCH = TC * 2 + 4, OUT_PITCH = TR + 8;
   __shared__ __attribute__((aligned(16))) char tile_in[TR * IN_PITCH];
   __shared__ __attribute__((aligned(16))) char tile_out[TC * OUT_PITCH];
@@ -727,6 +730,36 @@ __global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint1
     dst[3] = v[3];
   }
   __syncthreads();
+  if constexpr (BOTH) {
+    // the same tile once more along its rows (the forward GEMMs' operand): lane = (row, 32-column block), exactly
+    // what mx_quantize_kernel does with the matrix read from memory - the tile is read from HBM once for both copies
+    const int r = tid / 2, hb = tid % 2;
+    float w[32];
+    float am = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      const uint32_t two = *(const uint32_t*)(tile_in + r * IN_PITCH + hb * 64 + i * 4);
+      w[2 * i] = bf16_lo(two);
+      w[2 * i + 1] = bf16_hi(two);
+      am = fmaxf(am, fmaxf(fabsf(w[2 * i]), fabsf(w[2 * i + 1])));
+    }
+    const int exr = mx_scale_exponent(am);
+    const float invr = __uint_as_float((uint32_t)(254 - exr) << 23);
+    uint32_t o[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      int ww = 0;
+      ww = __builtin_amdgcn_cvt_pk_fp8_f32(w[4 * i] * invr, w[4 * i + 1] * invr, ww, false);
+      ww = __builtin_amdgcn_cvt_pk_fp8_f32(w[4 * i + 2] * invr, w[4 * i + 3] * invr, ww, true);
+      o[i] = (uint32_t)ww;
+    }
+    const int64_t grow = (int64_t)e * R + r0 + r;  // row of the (E * R, C) code matrix
+    u32x4* dst = (u32x4*)(q_rows + grow * C + c0 + hb * 32);
+    dst[0] = u32x4{o[0], o[1], o[2], o[3]};
+    dst[1] = u32x4{o[4], o[5], o[6], o[7]};
+    // scale table (C / 128, E * R) words, byte = 32-column block inside the 128
+    scales_rows[((int64_t)(c0 >> 7) * ((int64_t)E * R) + grow) * 4 + ((c0 & 127) >> 5) + hb] = (uint8_t)exr;
+  }
   const int c = tid % TC, rb = tid / TC;  // this lane's column and 32-row block
   float v[32];
   float amax = 0.f;
@@ -773,9 +806,26 @@ extern "C" int smoe_mx_quantize_transposed(const void* src, int64_t src_stride_e
   SMOE_REQUIRE(src && q && scales, SMOE_ERR_INVALID, "mx_quantize_transposed: null pointer");
   SMOE_REQUIRE_ALIGNED("mx_quantize_transposed", src, q, scales);
   SMOE_REQUIRE(E < 65536 && R / 128 < 65536, SMOE_ERR_UNSUPPORTED, "mx_quantize_transposed: tensor too large");
-  hipLaunchKernelGGL(mx_quantize_transposed_kernel, dim3((unsigned)(C / 64), (unsigned)(R / 128), (unsigned)E),
+  hipLaunchKernelGGL(mx_quantize_transposed_kernel<false>, dim3((unsigned)(C / 64), (unsigned)(R / 128), (unsigned)E),
                      dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, src_stride_e, src_stride_r, R, C, E,
-                     (uint8_t*)q, (uint32_t*)scales);
+                     (uint8_t*)q, (uint32_t*)scales, (uint8_t*)nullptr, (uint8_t*)nullptr);
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+extern "C" int smoe_mx_quantize_both(const void* src, int64_t src_stride_e, int64_t src_stride_r, int E, int R, int C,
+                                     void* q_rows, void* scales_rows, void* q_t, void* scales_t, void* stream) {
+  SMOE_REQUIRE(E >= 1 && R > 0 && C > 0, SMOE_ERR_INVALID, "mx_quantize_both: bad shape");
+  SMOE_REQUIRE(R % 128 == 0 && C % 128 == 0, SMOE_ERR_UNSUPPORTED,
+               "mx_quantize_both: (%d, %d) matrices: rows and columns must be multiples of 128", R, C);
+  SMOE_REQUIRE(src_stride_e % 8 == 0 && src_stride_r % 8 == 0, SMOE_ERR_UNSUPPORTED,
+               "mx_quantize_both: strides must be multiples of 8 elements");
+  SMOE_REQUIRE(src && q_rows && scales_rows && q_t && scales_t, SMOE_ERR_INVALID, "mx_quantize_both: null pointer");
+  SMOE_REQUIRE_ALIGNED("mx_quantize_both", src, q_rows, scales_rows, q_t, scales_t);
+  SMOE_REQUIRE(E < 65536 && R / 128 < 65536, SMOE_ERR_UNSUPPORTED, "mx_quantize_both: tensor too large");
+  hipLaunchKernelGGL(mx_quantize_transposed_kernel<true>, dim3((unsigned)(C / 64), (unsigned)(R / 128), (unsigned)E),
+                     dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, src_stride_e, src_stride_r, R, C, E,
+                     (uint8_t*)q_t, (uint32_t*)scales_t, (uint8_t*)q_rows, (uint8_t*)scales_rows);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }

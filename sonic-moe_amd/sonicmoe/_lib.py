@@ -62,6 +62,7 @@ _SIGNATURES = {
     "smoe_tr_compact": (c_int, [_P, _P, _I, _P, _L, _I, _P, _P, _P, _P]),
     "smoe_mx_quantize": (c_int, [_P, _L, _L, _I, _P, _P, _P]),
     "smoe_mx_quantize_transposed": (c_int, [_P, _L, _L, _I, _I, _I, _P, _P, _P]),
+    "smoe_mx_quantize_both": (c_int, [_P, _L, _L, _I, _I, _I, _P, _P, _P, _P, _P]),
     "smoe_down_projection_backward_fp8": (
         c_int,
         [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],

@@ -50,6 +50,7 @@ from .fp8 import (
     is_using_fp8_forward,
     mx_quantize,
     quantize_expert_weight,
+    quantize_expert_weight_both,
     quantize_expert_weight_transposed,
 )
 from .utils import enable_quack_gemm, is_using_quack_gemm
@@ -265,8 +266,11 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
     y1 = None if is_using_fp8_forward() else torch.empty(TK, I, dtype=x.dtype, device=x.device)
     y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
     if is_using_fp8_forward():
+        # a step whose backward pass runs on fp8 operands too reads each weight once for both quantised copies
+        both = is_using_fp8_backward() and not inference and b1 is None and b2 is None
+        quantize_weight = quantize_expert_weight_both if both else quantize_expert_weight
         xq, xs = mx_quantize(x)
-        w1q, w1s = quantize_expert_weight(w1)
+        w1q, w1s = quantize_weight(w1)
         # y1 leaves the up-projection already quantised (from the fp32 accumulator); its bf16 form is not stored
         y1q = torch.empty(TK, I, dtype=torch.uint8, device=x.device)
         y1s = torch.empty(I // 128, TK, dtype=torch.int32, device=x.device)
@@ -274,7 +278,7 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
             xq, xs, w1q, w1s, z, None, b1, off, gidx, E, stream_id, activation_type.value, glu, y1q, y1s
         )
         del xq, xs, w1q, w1s
-        w2q, w2s = quantize_expert_weight(w2)
+        w2q, w2s = quantize_weight(w2)
         _down_projection_forward_fp8(y1q, y1s, w2q, w2s, y2, b2, off, E, stream_id)
         del y1q, y1s, w2q, w2s
     else:

@@ -232,13 +232,81 @@ def _mx_quantize_transposed(src: torch.Tensor, q: torch.Tensor, scales: torch.Te
     _lib.check(rc, "_mx_quantize_transposed")
 
 
+@torch.library.custom_op(
+    f"{LIBRARY_NAME}::_mx_quantize_both", mutates_args={"q_rows", "scales_rows", "q_t", "scales_t"}
+)
+def _mx_quantize_both(src: torch.Tensor, q_rows: torch.Tensor, scales_rows: torch.Tensor, q_t: torch.Tensor,
+                      scales_t: torch.Tensor) -> None:
+    """src (E, R, C) bf16 -> both quantised copies from one pass over src: q_rows (E*R, C) / scales_rows (C/128, E*R) as
+    `_mx_quantize` of the (E*R, C) matrix, q_t (E, C, R) / scales_t (R/128, E*C) as `_mx_quantize_transposed`."""
+    _lib.require_device(src, q_rows, scales_rows, q_t, scales_t)
+    _check_bf16(("src", src))
+    E, R, C = src.shape
+    assert src.stride(2) == 1 and all(t.is_contiguous() for t in (q_rows, scales_rows, q_t, scales_t))
+    assert q_rows.dtype == torch.uint8 and q_rows.shape == (E * R, C) and q_t.dtype == torch.uint8 and q_t.shape == (E, C, R)
+    assert scales_rows.dtype == torch.int32 and scales_rows.shape == (C // 128, E * R)
+    assert scales_t.dtype == torch.int32 and scales_t.shape == (R // 128, E * C)
+    rc = _lib.lib().smoe_mx_quantize_both(
+        _lib.ptr(src), src.stride(0), src.stride(1), E, R, C, _lib.ptr(q_rows), _lib.ptr(scales_rows), _lib.ptr(q_t),
+        _lib.ptr(scales_t), _lib.current_stream_handle()
+    )
+    _lib.check(rc, "_mx_quantize_both")
+
+
+# Transposed quantised weights a forward pass made together with the row-quantised ones (one read of the weight for
+# both), waiting for the backward pass of the same step: key -> (weak owner, version, codes, scales).  An entry is used
+# once, and only while the weight is unchanged.
+_TRANSPOSED_STASH: dict = {}
+_TRANSPOSED_STASH_MAX = 16
+
+
+def _weight_key(w_view: torch.Tensor, w: torch.Tensor):
+    owner = w_view._base if w_view._base is not None else w_view  # the tensor whose version counter sees every write
+    return owner, (id(owner), w.data_ptr(), tuple(w.shape), w.device.index)
+
+
+def quantize_expert_weight_both(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """`quantize_expert_weight` for a step whose backward pass will ask for `quantize_expert_weight_transposed` of the
+    same weight: one kernel reads the weight once and writes both copies; the transposed one is kept for that call."""
+    w = w_view.permute(2, 0, 1)
+    E, N, K = w.shape
+    if not w.is_contiguous() or N % 128 or K % 128 or torch.compiler.is_compiling():
+        return quantize_expert_weight(w_view)
+    owner, key = _weight_key(w_view, w)
+    if _CACHE_WEIGHTS:
+        hit = _WEIGHT_CACHE.get(key)
+        if hit is not None and hit[0]() is owner and hit[1] == owner._version:
+            return hit[2], hit[3]  # unchanged since an earlier forward pass: only the transposed copy is missing
+    q = torch.empty(E * N, K, dtype=torch.uint8, device=w.device)
+    scales = torch.empty(K // 128, E * N, dtype=torch.int32, device=w.device)
+    qt = torch.empty(E, K, N, dtype=torch.uint8, device=w.device)
+    scales_t = torch.empty(N // 128, E * K, dtype=torch.int32, device=w.device)
+    _mx_quantize_both(w.detach(), q, scales, qt, scales_t)
+    if _CACHE_WEIGHTS:
+        if len(_WEIGHT_CACHE) >= _WEIGHT_CACHE_MAX:
+            _WEIGHT_CACHE.pop(next(iter(_WEIGHT_CACHE)))
+        _WEIGHT_CACHE[key] = (weakref.ref(owner, lambda _ref, k=key: _WEIGHT_CACHE.pop(k, None)), owner._version, q, scales)
+    if len(_TRANSPOSED_STASH) >= _TRANSPOSED_STASH_MAX:
+        _TRANSPOSED_STASH.pop(next(iter(_TRANSPOSED_STASH)))
+    _TRANSPOSED_STASH[key] = (weakref.ref(owner, lambda _ref, k=key: _TRANSPOSED_STASH.pop(k, None)), owner._version,
+                              qt.view(E * K, N), scales_t)
+    return q, scales
+
+
 def quantize_expert_weight_transposed(w_view: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     """w_view is the (out, in, E) permuted view of an (E, out, in) parameter; returns the (E * in, out) codes of the
     transposed matrices, quantised along `out`, and their scale table: the weight operand of the activation-gradient
-    GEMMs, which contract over `out`.  Not cached: a training step writes the weights between two backward passes."""
+    GEMMs, which contract over `out`.  Taken from the forward pass of the same step when that made it
+    (`quantize_expert_weight_both`); otherwise quantised here.  Not cached beyond that: a training step writes the
+    weights between two backward passes."""
     w = w_view.permute(2, 0, 1)
     if w.stride(2) != 1:
         w = w.contiguous()
+    elif not torch.compiler.is_compiling():
+        owner, key = _weight_key(w_view, w)
+        hit = _TRANSPOSED_STASH.pop(key, None)
+        if hit is not None and hit[0]() is owner and hit[1] == owner._version:
+            return hit[2], hit[3]
     E, N, K = w.shape
     if N % 128 or K % 64:
         raise NotImplementedError(f"quantize_expert_weight_transposed: ({N}, {K}) matrices need out % 128 == 0 and "

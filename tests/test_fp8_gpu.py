@@ -356,3 +356,58 @@ def test_weights_in_another_physical_layout_are_requantised_every_call(dev):
     q_ref, s_ref = fp8.mx_quantize(w_phys.permute(2, 0, 1).contiguous().reshape(E * N, K))
     assert torch.equal(q1, q_ref) and torch.equal(s1, s_ref)
     assert not (torch.equal(q0, q1) and torch.equal(s0, s1))
+
+
+@pytest.mark.parametrize("E,R,C", [(3, 256, 384), (2, 128, 128), (4, 512, 256)])
+def test_both_weight_copies_from_one_pass(dev, E, R, C):
+    """smoe_mx_quantize_both writes the row-quantised and the transposed-quantised copy of a weight exactly as the two
+    separate quantisers do (bit for bit, codes and scale words), also from a permuted parameter view."""
+    from sonicmoe.functional import fp8
+
+    g = torch.Generator().manual_seed(E * 1000 + R + C)
+    w = (torch.randn(E, R, C, generator=g) * 0.02).to(torch.bfloat16).to(dev)
+    w[0, :32, :32] = 0  # an all-zero block in either direction
+    q0, s0 = fp8.mx_quantize(w.reshape(E * R, C))
+    qt0 = torch.empty(E, C, R, dtype=torch.uint8, device=dev)
+    st0 = torch.empty(R // 128, E * C, dtype=torch.int32, device=dev)
+    fp8._mx_quantize_transposed(w, qt0, st0)
+    q1 = torch.empty(E * R, C, dtype=torch.uint8, device=dev)
+    s1 = torch.empty(C // 128, E * R, dtype=torch.int32, device=dev)
+    qt1 = torch.empty_like(qt0)
+    st1 = torch.empty_like(st0)
+    fp8._mx_quantize_both(w, q1, s1, qt1, st1)
+    assert torch.equal(q0, q1) and torch.equal(s0, s1)
+    assert torch.equal(qt0, qt1) and torch.equal(st0, st1)
+
+
+def test_fp8_step_reads_each_weight_once(dev, monkeypatch):
+    """With fp8 forward and backward enabled a training step quantises each expert weight with ONE kernel (both copies):
+    the backward pass finds the transposed copies its forward pass left, and the results equal those of the separate
+    quantisers bit for bit."""
+    import sonicmoe.functional as SF
+    from sonicmoe import MoE, enable_fp8_backward, enable_fp8_forward
+    from sonicmoe.enums import ActivationType
+    from sonicmoe.functional import fp8
+
+    calls = {"both": 0, "rows": 0, "transposed": 0}
+    real = {n: getattr(fp8, n) for n in ("_mx_quantize_both", "_mx_quantize_transposed")}
+    monkeypatch.setattr(fp8, "_mx_quantize_both", lambda *a: (calls.__setitem__("both", calls["both"] + 1), real["_mx_quantize_both"](*a))[1])
+    monkeypatch.setattr(fp8, "_mx_quantize_transposed", lambda *a: (calls.__setitem__("transposed", calls["transposed"] + 1), real["_mx_quantize_transposed"](*a))[1])
+    torch.manual_seed(5)
+    moe = MoE(8, 2, 512, 256, ActivationType.SWIGLU, False, 0.02).to(device=dev, dtype=torch.bfloat16)
+    x = torch.randn(1024, 512, device=dev).to(torch.bfloat16).requires_grad_()
+    dy = torch.randn(1024, 512, device=dev).to(torch.bfloat16)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_proj.weight]
+    with enable_fp8_forward(), enable_fp8_backward(), fp8.cache_quantized_weights(False):
+        out, _ = moe(x)
+        grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+    assert calls == {"both": 2, "rows": 0, "transposed": 0}, calls
+    # the same step with the one-pass quantiser switched off
+    monkeypatch.setattr(SF, "quantize_expert_weight_both", SF.quantize_expert_weight)
+    with enable_fp8_forward(), enable_fp8_backward(), fp8.cache_quantized_weights(False):
+        out0, _ = moe(x)
+        grads0 = torch.autograd.grad(out0, [x] + params, grad_outputs=dy)
+    assert calls["transposed"] == 2
+    assert torch.equal(out, out0)
+    for a, b in zip(grads, grads0):
+        assert torch.equal(a, b)
