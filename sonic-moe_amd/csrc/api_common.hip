@@ -21,7 +21,7 @@ void set_error(const char* fmt, ...) {
 
 namespace {
 std::once_flag g_tuning_once;
-Tuning g_tuning = {1, 0, 2, 1, 1};
+Tuning g_tuning = {1, 0, 2, 1, 1, 8, 1};
 
 struct Knob {
   const char* name;
@@ -35,6 +35,8 @@ const Knob g_knobs[] = {
     {"varlen_k_tile_order", "SMOE_VARLEN_K_TILE_ORDER", &Tuning::varlen_k_tile_order, 0, 2, 2},
     {"dz_stream", "SMOE_DZ_STREAM", &Tuning::dz_stream, 0, 1, 1},
     {"gemm_asm", "SMOE_GEMM_ASM", &Tuning::gemm_asm, 0, 1, 1},
+    {"gemm_group_tiles", "SMOE_GEMM_GROUP_TILES", &Tuning::gemm_group_tiles, 1, TILE_GROUP_MAX, 8},
+    {"gemm_group_snake", "SMOE_GEMM_GROUP_SNAKE", &Tuning::gemm_group_snake, 0, 1, 1},
 };
 
 void read_tuning_env() {
@@ -72,7 +74,7 @@ int device_compute_units(int* out) {
 // order == nullptr: experts are listed 0, 1, ...; otherwise position i of the list holds expert order[i]
 __global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __restrict__ off,
                                                               const int32_t* __restrict__ order, int E, int BM,
-                                                              TileMap tm) {
+                                                              int gmax, int snake, TileMap tm) {
   __shared__ int32_t wave_tot[16];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   int32_t base = 0;
@@ -99,9 +101,25 @@ __global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __r
       tot += wave_tot[w];
     }
     const int32_t start = base + wbase + v - tiles;
+    // groups of nearly equal height: the first `taller` of them have one token tile more
+    const int32_t ngroups = (tiles + gmax - 1) / gmax;
+    const int32_t hbase = ngroups ? tiles / ngroups : 0, taller = ngroups ? tiles % ngroups : 0;
+    const int32_t split = taller * (hbase + 1);
     for (int32_t i = 0; i < tiles; i++) {
       tm.expert[start + i] = e;
       tm.row0[start + i] = lo + i * BM;
+      int32_t g, first, h;
+      if (i < split) {
+        h = hbase + 1;
+        g = i / h;
+        first = g * h;
+      } else {
+        h = hbase;
+        g = (i - split) / h;
+        first = split + g * h;
+        g += taller;
+      }
+      tm.group[start + i] = (int32_t)((uint32_t)(start + first) | (uint32_t)h << 24 | (uint32_t)(snake & g & 1) << 31);
     }
     base += tot;
   }
@@ -109,7 +127,9 @@ __global__ __launch_bounds__(1024) void build_tile_map_kernel(const int32_t* __r
 }
 
 int launch_build_tile_map(const int32_t* off, const int32_t* order, int E, int BM, TileMap tm, hipStream_t st) {
-  hipLaunchKernelGGL(build_tile_map_kernel, dim3(1), dim3(1024), 0, st, off, order, E, BM, tm);
+  const Tuning& tune = tuning();
+  hipLaunchKernelGGL(build_tile_map_kernel, dim3(1), dim3(1024), 0, st, off, order, E, BM, tune.gemm_group_tiles,
+                     tune.gemm_group_snake, tm);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }

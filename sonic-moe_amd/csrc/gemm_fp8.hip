@@ -645,7 +645,7 @@ static int launch_fp8(Fp8Params& p, const int32_t* off, void* workspace, int64_t
                SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: operand too large for 32-bit offsets");
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
-  SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: too many tiles");
+  SMOE_REQUIRE(grid < (1ll << 31) && tile_map_fits(TK, E, C::BM), SMOE_ERR_UNSUPPORTED, "fp8 grouped gemm: too many tiles");
   const Tuning& tune = tuning();
   const int64_t lim24 = 1ll << 24;  // the tile-stream kernel forms its offsets with 24-bit multiplies
   const bool fits24 = data_rows < lim24 && p.p_rows < lim24 && p.p_stride < lim24 && p.N < lim24 && p.q_stride_row < lim24;

@@ -278,39 +278,9 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % C::WM, wn = wave / C::WM;
 
-  // tile bookkeeping is read through the constant address space: uniform addresses then become scalar loads, which do
-  // not touch the vector-memory counter the ring is timed with
-  typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
-  const const_i32_ptr tm_header = (const_i32_ptr)p.tm.header, tm_expert = (const_i32_ptr)p.tm.expert,
-                      tm_row0 = (const_i32_ptr)p.tm.row0, off = (const_i32_ptr)p.off;
-  const int num_m_tiles = tm_header[0];
-  const int64_t total = (int64_t)num_m_tiles * p.n_tiles;
-  const int64_t per_xcd = (total + 7) >> 3;
-  struct Tile {
-    int e, row0, row_end, n0;
-    bool valid;
-  };
-  // tile of virtual workgroup vb (the XCD-aware order of the one-tile-per-workgroup kernel)
-  auto tile_at = [&](int64_t vb) {
-    Tile t = {0, 0, 1, 0, false};
-    const int64_t slot = vb >> 3;
-    const int64_t lin = (vb & 7) * per_xcd + slot;
-    if (slot < per_xcd && lin < total) {
-      constexpr int GM = 8;
-      const int64_t per_group = (int64_t)GM * p.n_tiles;
-      const int group = (int)(lin / per_group);
-      const int first_m = group * GM;
-      const int gm = num_m_tiles - first_m < GM ? num_m_tiles - first_m : GM;
-      const int within = (int)(lin - (int64_t)group * per_group);
-      const int mt = first_m + within % gm;
-      t.e = tm_expert[mt];
-      t.row0 = tm_row0[mt];
-      t.row_end = off[t.e + 1];
-      t.n0 = (within / gm) * BN;
-      t.valid = true;
-    }
-    return t;
-  };
+  const StreamTiles tiles(p.tm, p.off, p.n_tiles, BN);
+  using Tile = StreamTile;
+  auto tile_at = [&](int64_t vb) { return tiles.at(vb); };
   int64_t vb = blockIdx.x;
   Tile cur = tile_at(vb);
   if (!cur.valid) return;
@@ -729,7 +699,7 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
   if (ROLE == ROLE_DZ) p.ds_cols = p.n_tiles * C::WN;
   const int64_t max_tiles = max_token_tiles(TK, E, C::BM) * p.n_tiles;
   const int64_t grid = ((max_tiles + 7) / 8) * 8;
-  SMOE_REQUIRE(grid < (1ll << 31), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
+  SMOE_REQUIRE(grid < (1ll << 31) && tile_map_fits(TK, E, C::BM), SMOE_ERR_UNSUPPORTED, "grouped gemm: too many tiles");
   {
     const Tuning& tune = tuning();
     if (tune.gemm_stream && (ROLE != ROLE_DZ || tune.dz_stream) && p.Kdim >= 3 * C::BK && offsets_fit32(p, C::QMN, false)) {
