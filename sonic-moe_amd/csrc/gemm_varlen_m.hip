@@ -494,24 +494,32 @@ __global__ __launch_bounds__(C::NT) void varlen_m_asm_kernel(const VarlenMParams
     asm volatile("" : "+v"(l));
     return l;
   };
-  // source rows of a tile's token operand: token indices (gathered) or the grouped rows themselves
+  const uint32_t p_row_bytes = (uint32_t)p.p_stride * 2u, q_row_bytes = (uint32_t)p.q_stride_row * 2u;
+  // extents: what the streams may touch (anything beyond is dropped by the range check instead of faulting)
+  const uint32_t p_bytes = (uint32_t)(p.p_rows * p.p_stride * 2);
+  // Rows of a ragged last tile behind the expert's end are not fetched at all when the tensor's end plus the longest
+  // stage offset still fits 32 bits: their loads get the tensor's end as offset, the range check drops them and the LDS
+  // receives zeros.  Otherwise they re-read the expert's last row.
+  const bool drop_rows = (uint64_t)p_bytes + (uint64_t)p.Kdim * 2u + 16u <= 0xffffffffull;
+  // source rows of a tile's token operand: token indices (gathered) or the grouped rows themselves; -1 = dropped
   auto token_rows = [&](const StreamTile& t, int(&rows)[C::P_INSTR]) {
     const int ln = opaque_lane();
 #pragma unroll
     for (int i = 0; i < C::P_INSTR; i++) {
-      int m = t.row0 + (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
-      m = m < t.row_end ? m : t.row_end - 1;
-      rows[i] = p.gidx ? p.gidx[m] : m;
+      const int m0 = t.row0 + (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
+      const int m = m0 < t.row_end ? m0 : t.row_end - 1;
+      const int row = p.gidx ? p.gidx[m] : m;
+      rows[i] = drop_rows && m0 >= t.row_end ? -1 : row;
     }
   };
-  const uint32_t p_row_bytes = (uint32_t)p.p_stride * 2u, q_row_bytes = (uint32_t)p.q_stride_row * 2u;
   auto point_p = [&](const int(&rows)[C::P_INSTR]) {
     const int ln = opaque_lane();
     i32x8 v;
 #pragma unroll
     for (int i = 0; i < C::P_INSTR; i++) {
       const int r = (wave * C::P_INSTR + i) * C::KRPI + ln / C::KPR;
-      v[i] = (int32_t)((uint32_t)rows[i] * p_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK, C::FR>(r)) << 4));
+      const uint32_t off = (uint32_t)rows[i] * p_row_bytes + ((((uint32_t)ln % C::KPR) ^ kswz<BK, C::FR>(r)) << 4);
+      v[i] = (int32_t)(rows[i] < 0 ? p_bytes : off);
     }
     return v;
   };
@@ -544,8 +552,6 @@ __global__ __launch_bounds__(C::NT) void varlen_m_asm_kernel(const VarlenMParams
     r[1] = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32) & 0xffffu);
     return r;
   };
-  // extents: what the streams may touch (anything beyond is dropped by the range check instead of faulting)
-  const uint32_t p_bytes = (uint32_t)(p.p_rows * p.p_stride * 2);
   const uint32_t q_bytes = C::QMN ? (uint32_t)(p.Kdim - 1) * q_row_bytes + (uint32_t)p.N * 2u
                                   : (uint32_t)(p.N - 1) * q_row_bytes + (uint32_t)p.Kdim * 2u;
   const i32x4 p_rsrc = make_buffer_resource(p.P, p_bytes);

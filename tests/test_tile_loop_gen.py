@@ -56,6 +56,18 @@ def test_replay_single_tile_and_ragged_columns(qmn):
     sim.simulate(_problem(qmn, 6, 320, [(0, 0, 256, 0), (0, 0, 256, 256)], False, seed=2, p_pad=8))
 
 
+@pytest.mark.parametrize("qmn", [False, True])
+def test_replay_rereads_the_last_row_next_to_the_32_bit_limit(qmn):
+    # Rows behind an expert's end are normally not fetched (offset = the tensor's end, dropped by the range check).
+    # With a token tensor that ends within one stage offset of 4 GiB that offset could wrap around into the tensor, so
+    # the kernel re-reads the expert's last row instead: both conventions have to replay clean.
+    small = _problem(qmn, 4, 512, TILES, True)
+    assert sim.drop_rows(small)
+    big = _problem(qmn, 4, 512, TILES, True, ntok=(0xffffffff - 64) // (4 * G.BK * 2))
+    assert not sim.drop_rows(big) and sim.p_extent(big) <= 0xffffffff
+    sim.simulate(big)
+
+
 def test_replay_nonzero_lds_base():
     sim.simulate(_problem(False, 4, 256, TILES[:3], True), lds_base=0)
 

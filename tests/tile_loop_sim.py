@@ -98,6 +98,7 @@ class Wave:
         self.ldsp_reg = G.S_LDSP  # register that holds the LDS address of the token operand's ring
         self.rsrc_regs = (G.S_PRSRC, G.S_QRSRC)  # first registers of the two streams' buffer resources
         self.oob_zero = False  # loads beyond the extent write zeros (the weight-gradient loop relies on it)
+        self.oob_zero_p = False  # the same for the token stream only: dropped rows of a ragged tile
         self.smem_out = set()  # scalar registers a scalar load in flight will write
         self.expect = None  # callable(wave, fn, fm, stage, ks) -> (want_q, want_p); default: the varlen-M operands
 
@@ -115,7 +116,7 @@ class Wave:
         soff = self.s[soff_reg] if soff_reg is not None else 0
         off = (self.v[voff_reg] + soff) & 0xffffffff
         oob = off + 16 > extent
-        if oob.any() and not self.oob_zero:
+        if oob.any() and not (self.oob_zero or (self.oob_zero_p and stream == P_STREAM)):
             raise SimError(f"wave {self.w}: load offset {int(off.max())} + 16 beyond extent {extent} (stream {stream})")
         if (off % 16).any():
             raise SimError("unaligned global piece")
@@ -218,9 +219,12 @@ class Wave:
             nc = start + n % 8
             want_q = e * prob.q_stride_e + k * prob.q_stride_row + nc[:, None]
         want_q = want_q | (Q_STREAM << 60)
-        m = np.minimum(row0 + wm * G.TM + fm * G.FR + lane % 16, row_end - 1)
+        m0 = row0 + wm * G.TM + fm * G.FR + lane % 16
+        m = np.minimum(m0, row_end - 1)
         row = prob.gidx[m] if prob.gidx is not None else m
         want_p = (row[:, None] * prob.p_stride + k) | (P_STREAM << 60)
+        if drop_rows(prob):
+            want_p = np.where((m0 >= row_end)[:, None], ZERO, want_p)
         self._compare(qreg, preg, want_q, want_p, stage, ks, fn, fm)
 
     def _compare(self, qreg, preg, want_q, want_p, stage, ks, fn, fm):
@@ -381,13 +385,25 @@ def run_wave(w: Wave, lines: list[str]):
 
 
 # ---- the C++ side, restated ------------------------------------------------------------------------------------------
+def p_extent(prob: Problem) -> int:
+    return prob.p_rows * prob.p_stride * 2
+
+
+def drop_rows(prob: Problem) -> bool:
+    """rows behind an expert's end are not fetched (offset = the tensor's end: dropped by the range check) when that
+    offset plus the longest stage offset cannot wrap around 32 bits; otherwise they re-read the expert's last row"""
+    return p_extent(prob) + prob.K * 2 + 16 <= 0xffffffff
+
+
 def token_rows(prob: Problem, wave: int, tile):
     e, row0, row_end, n0 = tile
     lane = np.arange(64)
     rows = []
     for i in range(G.P_INSTR):
-        m = np.minimum(row0 + (wave * G.P_INSTR + i) * 8 + lane // 8, row_end - 1)
-        rows.append(prob.gidx[m] if prob.gidx is not None else m)
+        m0 = row0 + (wave * G.P_INSTR + i) * 8 + lane // 8
+        m = np.minimum(m0, row_end - 1)
+        row = prob.gidx[m] if prob.gidx is not None else m
+        rows.append(np.where(m0 >= row_end, -1, row) if drop_rows(prob) else row)
     return rows
 
 
@@ -396,7 +412,8 @@ def point_p(prob: Problem, wave: int, rows):
     out = []
     for i in range(G.P_INSTR):
         r = (wave * G.P_INSTR + i) * 8 + lane // 8
-        out.append(rows[i] * (prob.p_stride * 2) + (((lane % 8) ^ kswz(r)) << 4))
+        off = rows[i] * (prob.p_stride * 2) + (((lane % 8) ^ kswz(r)) << 4)
+        out.append(np.where(rows[i] < 0, p_extent(prob), off))
     return out
 
 
@@ -450,6 +467,8 @@ def simulate(prob: Problem, lds_base: int = 0) -> dict:
     lines = asm_lines(prob.qmn)
     lds = Lds()
     waves = [Wave(w, lds, prob) for w in range(G.NW)]
+    for w in waves:
+        w.oob_zero_p = drop_rows(prob)
     tiles = prob.tiles
     q_step = G.BK * prob.q_stride_row * 2 if prob.qmn else G.BK * 2
     q_ring = G.P_SLOTS * G.P_STAGE
