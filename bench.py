@@ -173,6 +173,9 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
                 ("fp8:down_projection_backward(dz, +quantised dz)", lambda: fp8._down_projection_backward_fp8(doq, dos, w2tq, w2ts, z, dz, dzq, dzs, y1sc, ds, sflat, off, gidx, sidx, E, stream, "swiglu", True), gemm, None),
                 ("fp8:quantize_transposed(W1)", lambda: fp8._mx_quantize_transposed(w1.detach(), w1t3, w1ts), None, E * 2 * I * H * 3 + E * 2 * I * H // 32),
                 ("fp8:up_projection_backward(dx)", lambda: fp8._down_projection_forward_fp8(dzq, dzs, w1tq, w1ts, dxe, None, off, E, stream), 2 * gemm, None),
+                # what a training step runs instead of the four weight quantisers above: both copies from one read
+                ("fp8:quantize_both(W1)", lambda: fp8._mx_quantize_both(w1.detach(), w1q, w1s, w1t3, w1ts), None, E * 2 * I * H * 4 + E * 2 * I * H // 16),
+                ("fp8:quantize_both(W2)", lambda: fp8._mx_quantize_both(w2.detach(), w2q, w2s, w2t3, w2ts), None, E * H * I * 4 + E * H * I // 16),
             ]
         rows = []
         for name, fn, flops, nbytes in ops:

@@ -702,26 +702,29 @@ static int launch_fp8_dz(int act, Fp8Params& p, const int32_t* off, void* ws, in
 // ---- transposing quantiser -----------------------------------------------------------------------------------------
 // src: E matrices (R, C) bf16, row stride src_stride_r, matrix stride src_stride_e.  q: E matrices (C, R) e4m3, the
 // transposes, quantised along R (32 consecutive r share a scale); scales (R / 128, E * C) words as in mx_quantize.
-// One workgroup transposes a 128 (r) x 64 (c) tile through LDS: row-contiguous loads, column reads (one lane = one
+// One workgroup transposes a 128 (r) x TC (c) tile through LDS: row-contiguous loads, column reads (one lane = one
 // column and one 32-row block), bytes parked transposed, row-contiguous stores of 128 bytes per output row.
+// BOTH: the same tile is also quantised along its rows (the forward GEMMs' operand, exactly what mx_quantize_kernel
+// computes from the matrix in memory), so a weight is read from HBM once for both copies; the tile is 128 columns wide
+// then, so that the row-quantised copy is written in whole 128-byte lines and whole scale words as well.
 template <bool BOTH>
 __global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint16_t* __restrict__ src,
                                                                      int64_t src_stride_e, int64_t src_stride_r, int R,
                                                                      int C, int E, uint8_t* __restrict__ q,
                                                                      uint32_t* __restrict__ scales,
                                                                      uint8_t* __restrict__ q_rows,
-                                                                     uint8_t* __restrict__ scales_rows) {
-  constexpr int TR = 128, TC = 64, IN_PITCH = TC * 2 + 4, OUT_PITCH = TR + 8;
+                                                                     uint32_t* __restrict__ scales_rows) {
+  constexpr int TR = 128, TC = BOTH ? 128 : 64, IN_PITCH = TC * 2 + 4, OUT_PITCH = TR + 8;
+  constexpr int LPR = TC / 8, RPP = 256 / LPR;  // lanes per input row (16 bytes each), input rows per pass
   __shared__ __attribute__((aligned(16))) char tile_in[TR * IN_PITCH];
   __shared__ __attribute__((aligned(16))) char tile_out[TC * OUT_PITCH];
   __shared__ uint8_t exps[TC][4];
   const int tid = threadIdx.x;
   const int c0 = blockIdx.x * TC, r0 = blockIdx.y * TR, e = blockIdx.z;
   const uint16_t* base = src + (int64_t)e * src_stride_e + (int64_t)r0 * src_stride_r + c0;
-  // 8 lanes x 16 bytes per input row, 32 rows per pass
 #pragma unroll
-  for (int pass = 0; pass < TR / 32; pass++) {
-    const int r = pass * 32 + tid / 8, piece = tid % 8;
+  for (int pass = 0; pass < TR / RPP; pass++) {
+    const int r = pass * RPP + tid / LPR, piece = tid % LPR;
     const u32x4 v = *(const u32x4*)(base + (int64_t)r * src_stride_r + piece * 8);
     uint32_t* dst = (uint32_t*)(tile_in + r * IN_PITCH + piece * 16);
     dst[0] = v[0];
@@ -731,55 +734,64 @@ __global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint1
   }
   __syncthreads();
   if constexpr (BOTH) {
-    // the same tile once more along its rows (the forward GEMMs' operand): lane = (row, 32-column block), exactly
-    // what mx_quantize_kernel does with the matrix read from memory - the tile is read from HBM once for both copies
+    // lane = (row, half of its 128 columns): two 32-column blocks, 64 contiguous output bytes
     const int r = tid / 2, hb = tid % 2;
-    float w[32];
-    float am = 0.f;
+    u32x4 o[4];
+    uint32_t ex2 = 0;
 #pragma unroll
-    for (int i = 0; i < 16; i++) {
-      const uint32_t two = *(const uint32_t*)(tile_in + r * IN_PITCH + hb * 64 + i * 4);
-      w[2 * i] = bf16_lo(two);
-      w[2 * i + 1] = bf16_hi(two);
-      am = fmaxf(am, fmaxf(fabsf(w[2 * i]), fabsf(w[2 * i + 1])));
-    }
-    const int exr = mx_scale_exponent(am);
-    const float invr = __uint_as_float((uint32_t)(254 - exr) << 23);
-    uint32_t o[8];
+    for (int blk = 0; blk < 2; blk++) {
+      float w[32];
+      float am = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      int ww = 0;
-      ww = __builtin_amdgcn_cvt_pk_fp8_f32(w[4 * i] * invr, w[4 * i + 1] * invr, ww, false);
-      ww = __builtin_amdgcn_cvt_pk_fp8_f32(w[4 * i + 2] * invr, w[4 * i + 3] * invr, ww, true);
-      o[i] = (uint32_t)ww;
+      for (int i = 0; i < 16; i++) {
+        const uint32_t two = *(const uint32_t*)(tile_in + r * IN_PITCH + hb * 128 + blk * 64 + i * 4);
+        w[2 * i] = bf16_lo(two);
+        w[2 * i + 1] = bf16_hi(two);
+        am = fmaxf(am, fmaxf(fabsf(w[2 * i]), fabsf(w[2 * i + 1])));
+      }
+      const int exr = mx_scale_exponent(am);
+      const float invr = __uint_as_float((uint32_t)(254 - exr) << 23);
+      ex2 |= (uint32_t)exr << (8 * blk);
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        int ww = 0;
+        ww = __builtin_amdgcn_cvt_pk_fp8_f32(w[4 * i] * invr, w[4 * i + 1] * invr, ww, false);
+        ww = __builtin_amdgcn_cvt_pk_fp8_f32(w[4 * i + 2] * invr, w[4 * i + 3] * invr, ww, true);
+        o[2 * blk + i / 4][i % 4] = (uint32_t)ww;
+      }
     }
     const int64_t grow = (int64_t)e * R + r0 + r;  // row of the (E * R, C) code matrix
-    u32x4* dst = (u32x4*)(q_rows + grow * C + c0 + hb * 32);
-    dst[0] = u32x4{o[0], o[1], o[2], o[3]};
-    dst[1] = u32x4{o[4], o[5], o[6], o[7]};
-    // scale table (C / 128, E * R) words, byte = 32-column block inside the 128
-    scales_rows[((int64_t)(c0 >> 7) * ((int64_t)E * R) + grow) * 4 + ((c0 & 127) >> 5) + hb] = (uint8_t)exr;
-  }
-  const int c = tid % TC, rb = tid / TC;  // this lane's column and 32-row block
-  float v[32];
-  float amax = 0.f;
+    u32x4* dst = (u32x4*)(q_rows + grow * C + c0 + hb * 64);
 #pragma unroll
-  for (int i = 0; i < 32; i++) {
-    const uint16_t h = *(const uint16_t*)(tile_in + (rb * 32 + i) * IN_PITCH + c * 2);
-    v[i] = __uint_as_float((uint32_t)h << 16);
-    amax = fmaxf(amax, fabsf(v[i]));
+    for (int i = 0; i < 4; i++) dst[i] = o[i];
+    // scale table (C / 128, E * R) words: the row's four blocks of this 128-column tile are one word
+    const uint32_t other = __shfl_xor(ex2, 1, 64);
+    if (hb == 0) scales_rows[(int64_t)(c0 >> 7) * ((int64_t)E * R) + grow] = ex2 | (other << 16);
   }
-  const int ex = mx_scale_exponent(amax);
-  const float inv = __uint_as_float((uint32_t)(254 - ex) << 23);
+  // lane = (column, 32-row block)
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i] * inv, v[8 * i + 1] * inv, 0, false);
-    w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 2] * inv, v[8 * i + 3] * inv, w0, true);
-    int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 4] * inv, v[8 * i + 5] * inv, 0, false);
-    w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 6] * inv, v[8 * i + 7] * inv, w1, true);
-    *(u32x2*)(tile_out + c * OUT_PITCH + rb * 32 + i * 8) = u32x2{(uint32_t)w0, (uint32_t)w1};
+  for (int rb = tid / TC; rb < TR / 32; rb += 256 / TC) {
+    const int c = tid % TC;
+    float v[32];
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+      const uint16_t h = *(const uint16_t*)(tile_in + (rb * 32 + i) * IN_PITCH + c * 2);
+      v[i] = __uint_as_float((uint32_t)h << 16);
+      amax = fmaxf(amax, fabsf(v[i]));
+    }
+    const int ex = mx_scale_exponent(amax);
+    const float inv = __uint_as_float((uint32_t)(254 - ex) << 23);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      int w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i] * inv, v[8 * i + 1] * inv, 0, false);
+      w0 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 2] * inv, v[8 * i + 3] * inv, w0, true);
+      int w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 4] * inv, v[8 * i + 5] * inv, 0, false);
+      w1 = __builtin_amdgcn_cvt_pk_fp8_f32(v[8 * i + 6] * inv, v[8 * i + 7] * inv, w1, true);
+      *(u32x2*)(tile_out + c * OUT_PITCH + rb * 32 + i * 8) = u32x2{(uint32_t)w0, (uint32_t)w1};
+    }
+    exps[c][rb] = (uint8_t)ex;
   }
-  exps[c][rb] = (uint8_t)ex;
   __syncthreads();
   // 16 lanes x 8 bytes per output row, 16 rows per pass
   uint8_t* qbase = q + ((int64_t)e * C + c0) * R + r0;
@@ -808,7 +820,7 @@ extern "C" int smoe_mx_quantize_transposed(const void* src, int64_t src_stride_e
   SMOE_REQUIRE(E < 65536 && R / 128 < 65536, SMOE_ERR_UNSUPPORTED, "mx_quantize_transposed: tensor too large");
   hipLaunchKernelGGL(mx_quantize_transposed_kernel<false>, dim3((unsigned)(C / 64), (unsigned)(R / 128), (unsigned)E),
                      dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, src_stride_e, src_stride_r, R, C, E,
-                     (uint8_t*)q, (uint32_t*)scales, (uint8_t*)nullptr, (uint8_t*)nullptr);
+                     (uint8_t*)q, (uint32_t*)scales, (uint8_t*)nullptr, (uint32_t*)nullptr);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }
@@ -823,9 +835,9 @@ extern "C" int smoe_mx_quantize_both(const void* src, int64_t src_stride_e, int6
   SMOE_REQUIRE(src && q_rows && scales_rows && q_t && scales_t, SMOE_ERR_INVALID, "mx_quantize_both: null pointer");
   SMOE_REQUIRE_ALIGNED("mx_quantize_both", src, q_rows, scales_rows, q_t, scales_t);
   SMOE_REQUIRE(E < 65536 && R / 128 < 65536, SMOE_ERR_UNSUPPORTED, "mx_quantize_both: tensor too large");
-  hipLaunchKernelGGL(mx_quantize_transposed_kernel<true>, dim3((unsigned)(C / 64), (unsigned)(R / 128), (unsigned)E),
+  hipLaunchKernelGGL(mx_quantize_transposed_kernel<true>, dim3((unsigned)(C / 128), (unsigned)(R / 128), (unsigned)E),
                      dim3(256), 0, (hipStream_t)stream, (const uint16_t*)src, src_stride_e, src_stride_r, R, C, E,
-                     (uint8_t*)q_t, (uint32_t*)scales_t, (uint8_t*)q_rows, (uint8_t*)scales_rows);
+                     (uint8_t*)q_t, (uint32_t*)scales_t, (uint8_t*)q_rows, (uint32_t*)scales_rows);
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }

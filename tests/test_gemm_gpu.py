@@ -190,7 +190,9 @@ def test_tile_streams(dev, tuning, grid, T, H, I, E, K, skew, empty):
 
 
 @pytest.mark.parametrize("knob,value", [("gemm_stream", 0), ("gemm_asm", 0), ("dz_stream", 0),
-                                        ("varlen_k_tile_order", 0), ("varlen_k_tile_order", 1)])
+                                        ("varlen_k_tile_order", 0), ("varlen_k_tile_order", 1),
+                                        ("gemm_group_tiles", 1), ("gemm_group_tiles", 3), ("gemm_group_tiles", 127),
+                                        ("gemm_group_snake", 0)])
 def test_kernel_selection_knobs(dev, tuning, knob, value):
     """The alternative kernels / tile orders a tuning knob selects give the same results as the defaults
     (bit-identical: the arithmetic of a tile does not depend on who computes it or when; the score gradient is a sum of
