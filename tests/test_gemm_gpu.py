@@ -74,6 +74,35 @@ def test_forward_ops(dev, T, H, I, E, K, skew, empty):
     assert torch.equal(o, o2)
 
 
+@pytest.mark.parametrize("rows_short_of_4gib", [2, 1])
+def test_token_tensor_ending_next_to_4gib(dev, rows_short_of_4gib):
+    """The tile streams address the gathered token operand with 32-bit byte offsets from the tensor's start, and drop the
+    loads of rows behind an expert's end by giving them the tensor's end as offset - unless that end plus a stage offset
+    could wrap around 32 bits, in which case they re-read the expert's last row.  A token tensor of 4 GiB less two rows
+    takes the first form, less one row the second; gathered rows include the tensor's first and last ones, experts end in
+    ragged tiles."""
+    fwd, _ = _ops()
+    H, I, E = 2048, 128, 3
+    T = 2**32 // (H * 2) - rows_short_of_4gib
+    _, w1, _ = make_weights(E, H, I, dev, seed=77)
+    g = torch.Generator(device=dev).manual_seed(78)
+    x = torch.randn(T, H, generator=g, device=dev, dtype=torch.bfloat16)
+    counts = [300, 0, 291]
+    TK = sum(counts)
+    sel = torch.randperm(T, generator=torch.Generator().manual_seed(79))[:TK - 4]
+    gidx = torch.cat([torch.tensor([T - 1, 0, T - 2, 1]), sel]).to(torch.int32).to(dev)
+    off = torch.tensor([0, 300, 300, 591], dtype=torch.int32, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+    z = torch.empty(TK, 2 * I, dtype=torch.bfloat16, device=dev)
+    y1 = torch.empty(TK, I, dtype=torch.bfloat16, device=dev)
+    fwd._up_projection_forward(x, w1.permute(1, 2, 0), z, y1, None, off, None, gidx, stream, "swiglu", True, False)
+    # the oracle on the gathered rows only
+    xg = x[gidx.long()].cpu()
+    z_ref, y1_ref = M.up_projection_forward(xg, w1.cpu(), off.cpu(), torch.arange(TK))
+    assert rel_l2(z.cpu(), z_ref) < TOL
+    assert rel_l2(y1.cpu(), y1_ref) < TOL
+
+
 @pytest.mark.parametrize("T,H,I,E,K,skew,empty", SHAPES)
 def test_backward_ops(dev, T, H, I, E, K, skew, empty):
     fwd, bwd = _ops()
