@@ -103,6 +103,33 @@ def test_token_tensor_ending_next_to_4gib(dev, rows_short_of_4gib):
     assert rel_l2(y1.cpu(), y1_ref) < TOL
 
 
+@pytest.mark.parametrize("pad_short", [0, 64])
+def test_weight_view_with_rows_4gib_apart(dev, pad_short):
+    """The C ABI takes any weight row stride; the tile streams form weight addresses as 32-bit byte offsets from the
+    expert's matrix.  A (N1, E, padded H) storage whose (N1, H, E) view spans exactly 4 GiB per expert must be sent to the
+    kernels with 64-bit pointers; 64 columns less, the offsets just fit and the tile stream takes it."""
+    fwd, _ = _ops()
+    T, H, I, E, K = 600, 256, 128, 2, 1
+    N1 = 2 * I
+    hpad = 2**31 // (N1 * E) - pad_short
+    assert (N1 * E * hpad * 2 >= 2**32) == (pad_short == 0)
+    store = torch.empty(N1, E, hpad, dtype=torch.bfloat16, device=dev)
+    g = torch.Generator(device=dev).manual_seed(91)
+    store[:, :, :H] = (torch.randn(N1, E, H, generator=g, device=dev) * 0.05).to(torch.bfloat16)
+    w1_view = store[:, :, :H].permute(0, 2, 1)  # (N1, H, E), rows E * hpad elements apart
+    w1_dense = store[:, :, :H].permute(1, 0, 2).contiguous()  # (E, N1, H)
+    idx, scores, meta, md = make_tc_routing(T, E, K, dev, seed=92, skew=0.0, empty=())
+    x = torch.randn(T, H, generator=g, device=dev, dtype=torch.bfloat16)
+    off, gidx = md["expert_frequency_offset"], md["x_gather_idx"]
+    stream = torch.cuda.current_stream().cuda_stream
+    z = torch.empty(T * K, N1, dtype=torch.bfloat16, device=dev)
+    y1 = torch.empty(T * K, I, dtype=torch.bfloat16, device=dev)
+    fwd._up_projection_forward(x, w1_view, z, y1, None, off, None, gidx, stream, "swiglu", True, False)
+    z_ref, y1_ref = M.up_projection_forward(x.cpu(), w1_dense.cpu(), off.cpu(), gidx.cpu())
+    assert rel_l2(z, z_ref) < TOL
+    assert rel_l2(y1, y1_ref) < TOL
+
+
 @pytest.mark.parametrize("T,H,I,E,K,skew,empty", SHAPES)
 def test_backward_ops(dev, T, H, I, E, K, skew, empty):
     fwd, bwd = _ops()
