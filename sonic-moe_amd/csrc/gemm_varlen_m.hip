@@ -643,9 +643,11 @@ __global__ __launch_bounds__(C::NT) void varlen_m_asm_kernel(const VarlenMParams
       da.row_end = cur.row_end;
       da.n_base = cur.n0 + wn * C::TN;
       da.N = p.N;
-      dz_epilogue_at<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) ? 2 : 1, false, 16>(
+      // z and dz do not pass through LDS here (dz_epilogue_direct); only y1s is parked, in the first 4 KiB of the region
+      // (two fragment rows of z in flight for the gated activations; one for GEGLU, whose erf needs the registers)
+      dz_epilogue_direct<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) && act_pointwise(ACT) != PW_GELU ? 2 : 1>(
           [&](auto fn_c, auto fm_c) { return agpr_read4<SMOE_TL_ACC(decltype(fn_c)::value, decltype(fm_c)::value)>(); },
-          region, opaque_lane(), da, [] {});
+          region, opaque_lane(), da);
     } else {
       FwdEpilogueArgs ea;
       ea.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
