@@ -53,14 +53,22 @@ int smoe_version(void);
 const char* smoe_last_error(void);
 
 /* Kernel-selection knobs.  Each is read from the environment once, at the first launch that needs it; this call
- * overrides one afterwards (value < 0 restores the default).  Results do not depend on any of them; they exist for
- * tuning and so that tests can walk through every kernel.  No counterpart in the reference.
+ * overrides one afterwards (value < 0 restores the default).  Results do not depend on any of them (the two kernel
+ * families "gemm_asm" selects between group the score gradient's partial sums differently: ds agrees to 1e-5); they
+ * exist for tuning and so that tests can walk through every kernel.  No counterpart in the reference.
+ *   "gemm_asm"             SMOE_GEMM_ASM             1 (default): the bf16 grouped GEMMs run on the hand-scheduled
+ *                                                    four-wavefront loop where their shape allows; 0: on the
+ *                                                    compiler-scheduled eight-wavefront kernels
  *   "gemm_stream"          SMOE_GEMM_STREAM          1: token-grouped GEMMs run as tile streams (default); 0: one tile
  *                                                    per workgroup
  *   "gemm_stream_grid"     SMOE_GEMM_STREAM_GRID     workgroups of a tile-stream launch; 0 = one per compute unit
  *   "dz_stream"            SMOE_DZ_STREAM            1 (default) the bf16 dz kernel is a tile stream too; 0 one tile per
  *                                                    workgroup for dz alone
- *   "varlen_k_tile_order"  SMOE_VARLEN_K_TILE_ORDER  2 blocked (default), 0 round-robin, 1 whole experts per XCD */
+ *   "gemm_group_tiles"     SMOE_GEMM_GROUP_TILES     tile order of the token-grouped streams: most token tiles of one
+ *                                                    expert that sweep the feature tiles together (default 8, 1..127)
+ *   "gemm_group_snake"     SMOE_GEMM_GROUP_SNAKE     1 (default): consecutive groups sweep in opposite directions
+ *   "varlen_k_tile_order"  SMOE_VARLEN_K_TILE_ORDER  eight-wavefront weight-gradient kernel: 2 blocked (default),
+ *                                                    0 round-robin, 1 whole experts per XCD */
 int smoe_set_tuning(const char* name, int value);
 
 /* ---------------------------------------------------------------------------------------------------------
