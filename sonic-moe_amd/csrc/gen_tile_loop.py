@@ -93,8 +93,21 @@ class Emitter:
         return f"L{stem}{self.nlabel}_%="
 
 
+def fragment_order(idx: int) -> tuple[int, int]:
+    """The idx-th matrix instruction of a k-slice works on fragment (fn, fm).  Two weight fragments at a time, zigzag over
+    the token fragments, every other pair backwards: consecutive instructions always share one operand fragment.
+    Measured against weight-fragment-major order: 1.3 % of the kernels (2 x 2 blocks 0.9 %, a Hilbert curve 1.2 %, 4 x 4
+    blocks slower); the instruction reads its operands from the register file either way, so this is power, not issue."""
+    pair, w = idx // (2 * FM), idx % (2 * FM)
+    fm = w // 2
+    fn = 2 * pair + ((w % 2) ^ (fm & 1))
+    if pair & 1:
+        fm = FM - 1 - fm
+    return fn, fm
+
+
 def mfma(setno: int, idx: int, fresh: bool) -> str:
-    fn, fm = idx // FM, idx % FM
+    fn, fm = fragment_order(idx)
     a = acc_reg(fn, fm)
     q, p = qfrag(setno, fn), pfrag(setno, fm)
     c = "0" if fresh else f"a[{a}:{a + 3}]"
