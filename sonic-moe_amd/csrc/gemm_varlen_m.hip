@@ -258,7 +258,8 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     da.n_base = n_base;
     da.N = p.N;
     static_assert(C::NW * DzStaging<C::TN, ACT>::BYTES <= C::RING, "dz staging must fit into the idle ring");
-    dz_epilogue<Mma, C::TM, C::TN, ACT>(acc, smem + wave * DzStaging<C::TN, ACT>::BYTES, lane, da, [&]() {
+    // (GEGLU: one batch of z in flight instead of two, its erf needs the registers)
+    dz_epilogue<Mma, C::TM, C::TN, ACT, act_pointwise(ACT) == PW_GELU ? 1 : 2>(acc, smem + wave * DzStaging<C::TN, ACT>::BYTES, lane, da, [&]() {
       wait_lds_all();
       lds_barrier();  // every wave has finished reading the ring
     });
@@ -433,7 +434,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
       da.n_base = cur.n0 + wn * C::TN;
       da.N = p.N;
       // every wave has issued its reads of the last stage ahead of the barrier in front of the last step
-      dz_epilogue<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) ? 2 : 1, false, 16>(acc, region, opaque_lane(), da, [] {});
+      dz_epilogue<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) && act_pointwise(ACT) != PW_GELU ? 2 : 1, false, 16>(acc, region, opaque_lane(), da, [] {});
       return advance_tile();
     }
     FwdEpilogueArgs ea;
