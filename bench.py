@@ -141,8 +141,17 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
             ops.append(("router_forward_fused(gemm+topk+colsum)",
                         lambda: forward._router_forward_fused(xd, wr.detach(), rf_logits, scores, idx, rf_part),
                         2.0 * T * H * E, T * H * 2 + T * E * 2 + T * K * 8))
+        # the down projection fused with the combine (opt-in, sonicmoe.functional.fused_combine): zero-fill of the output
+        # + one kernel with atomic adds, against down_projection_forward + router_forward(combine) above
+        o_fused = torch.empty(T, H, dtype=bf, device=dev)
+
+        def down_combine_fused():
+            o_fused.zero_()
+            forward._down_projection_forward_combine(w2v, y1, o_fused, None, sflat, off, None, gidx, sidx, stream)
+
+        ops.append(("down_projection_forward_fused_combine(atomics)", down_combine_fused, gemm, None))
         if gemms_only:
-            ops = [o for o in ops if o[2] and "router_gemm" not in o[0]]
+            ops = [o for o in ops if o[2] and "router_gemm" not in o[0] and "fused_combine" not in o[0]]
         if H % 128 == 0 and I % 128 == 0 and (only is None or only.startswith("fp8:")) and not gemms_only:
             # fp8 forward (config 5 = this shape with block-scaled e4m3 operands): quantisers and the two fp8 GEMMs
             from sonicmoe.functional import fp8

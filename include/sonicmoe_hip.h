@@ -162,6 +162,21 @@ int smoe_down_projection_forward(const void* y1, const void* w2, int64_t w2_stri
                                  int64_t TK, int H, int I, int E, void* workspace, size_t workspace_bytes,
                                  void* stream);
 
+/* The down projection FUSED with the score-weighted combine: o[x_gather_idx[m]] += scores[s_scatter_idx[m]] *
+ * (y1[m] W2[e]^T (+ b2[e])), y2 is never stored.  No counterpart in the reference, which stores y2
+ * (sonicmoe/functional/forward.py:132-178) and reduces it with a second kernel (forward.py:181-236,
+ * reduction_over_k_gather.py:441-517); what it replaces is that pair.
+ *   o (T, H) bf16, MUST BE ZERO on entry; scores fp32 flat slots; the other arguments as above and as in
+ *   smoe_down_projection_backward
+ * A token's rows come from different experts' tiles, so the additions are packed-bf16 atomics: every addition rounds
+ * to bf16 and their order is not fixed, i.e. the result is within bf16 accumulation error of the two-kernel path and
+ * not bit-reproducible from run to run.  Slower than the two kernels on MI355X (measured); kept as an option. */
+int smoe_down_projection_forward_combine(const void* y1, const void* w2, int64_t w2_stride_e, int64_t w2_stride_row,
+                                         const void* b2, void* o, const float* scores, const int32_t* off,
+                                         const int32_t* expert_schedule_order, const int32_t* x_gather_idx,
+                                         const int32_t* s_scatter_idx, int64_t T, int64_t TK, int H, int I, int E,
+                                         void* workspace, size_t workspace_bytes, void* stream);
+
 /* out[t] = sum_{j in [tok_off[t], tok_off[t+1])} w[j] * src[ridx[j]]  (w == NULL: unweighted), fp32 accumulate.
  * Replaces sonicmoe::_router_forward and sonicmoe::_token_broadcast_backward
  * (sonicmoe/functional/forward.py:181-202, backward.py:464-484; kernel reduction_over_k_gather.py:441-517).

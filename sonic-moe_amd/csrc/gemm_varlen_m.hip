@@ -10,7 +10,9 @@
 
 namespace smoe {
 
-enum Role { ROLE_UP_FWD = 0, ROLE_PLAIN = 1, ROLE_DZ = 2 };
+// ROLE_COMBINE: the down-projection forward that adds its score-weighted rows onto the tokens' output rows instead of
+// storing y2 (opt-in, atomic: combine_epilogue_batch)
+enum Role { ROLE_UP_FWD = 0, ROLE_PLAIN = 1, ROLE_DZ = 2, ROLE_COMBINE = 3 };
 
 struct VarlenMParams {
   const uint16_t* P;
@@ -34,6 +36,7 @@ struct VarlenMParams {
   const int32_t* sidx;
   float* ds_partial;
   int ds_cols;
+  const int32_t* out_rows;  // ROLE_COMBINE: grouped row -> row of out0 (the token)
 };
 
 template <int BM_, int BN_, int WM_, int WN_, bool QMN_, int BK_, int NSTAGE_>
@@ -239,6 +242,21 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     wait_vmem_all();
     lds_barrier();  // all waves are done reading the last stage
     forward_epilogue<Mma, C::TM, C::TN, ROLE == ROLE_UP_FWD, ACT>(acc, smem, wave, lane, ea);
+  } else if constexpr (ROLE == ROLE_COMBINE) {
+    CombineEpilogueArgs ca;
+    ca.bias = p.bias ? p.bias + (int64_t)e * p.N : nullptr;
+    ca.o = p.out0;
+    ca.o_stride = p.out0_stride;
+    ca.out_rows = p.out_rows;
+    ca.scores = p.scores;
+    ca.sidx = p.sidx;
+    ca.m_base = m_base;
+    ca.row_end = row_end;
+    ca.n_base = n_base;
+    ca.N = p.N;
+    wait_vmem_all();
+    lds_barrier();  // all waves are done reading the last stage
+    combine_epilogue_rows<Mma, C::TM, C::TN>(acc, smem + wave * (32 * EpiLayout<C::TN>::ROW_BYTES), lane, ca);
   } else {
     // ---- dz epilogue (dz_epilogue in gemm_common.h) ----
     DzEpilogueArgs da = {};
@@ -649,6 +667,19 @@ __global__ __launch_bounds__(C::NT) void varlen_m_asm_kernel(const VarlenMParams
       dz_epilogue_direct<Mma, C::TM, C::TN, ACT, act_is_glu(ACT) && act_pointwise(ACT) != PW_GELU ? 2 : 1>(
           [&](auto fn_c, auto fm_c) { return agpr_read4<SMOE_TL_ACC(decltype(fn_c)::value, decltype(fm_c)::value)>(); },
           region, opaque_lane(), da);
+    } else if constexpr (ROLE == ROLE_COMBINE) {
+      CombineEpilogueArgs ca;
+      ca.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
+      ca.o = p.out0;
+      ca.o_stride = p.out0_stride;
+      ca.out_rows = p.out_rows;
+      ca.scores = p.scores;
+      ca.sidx = p.sidx;
+      ca.m_base = cur.row0 + wm * C::TM;
+      ca.row_end = cur.row_end;
+      ca.n_base = cur.n0 + wn * C::TN;
+      ca.N = p.N;
+      combine_epilogue_rows_agpr<Mma, C::TM, C::TN>(region, opaque_lane(), ca);
     } else {
       FwdEpilogueArgs ea;
       ea.bias = p.bias ? p.bias + (int64_t)cur.e * p.N : nullptr;
@@ -731,13 +762,15 @@ static int launch_varlen_m(VarlenMParams& p, const int32_t* off, void* workspace
         SMOE_LAUNCH_CHECK();
         return SMOE_OK;
       }
-      static LdsLimitOnce lds_limit_stream;
-      auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
-      const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
-      if (rc_s) return rc_s;
-      hipLaunchKernelGGL(skern, dim3((unsigned)sgrid), dim3(C::NT), C::SMEM, st, p);
-      SMOE_LAUNCH_CHECK();
-      return SMOE_OK;
+      if constexpr (ROLE != ROLE_COMBINE) {  // (the combining epilogue exists in the two other kernels only)
+        static LdsLimitOnce lds_limit_stream;
+        auto skern = varlen_m_stream_kernel<C, ROLE, ACT>;
+        const int rc_s = lds_limit_stream.ensure((const void*)skern, C::SMEM);
+        if (rc_s) return rc_s;
+        hipLaunchKernelGGL(skern, dim3((unsigned)sgrid), dim3(C::NT), C::SMEM, st, p);
+        SMOE_LAUNCH_CHECK();
+        return SMOE_OK;
+      }
     }
   }
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(C::NT), C::SMEM, st, p);
@@ -853,6 +886,41 @@ extern "C" int smoe_down_projection_forward(const void* y1, const void* w2, int6
   p.out0 = (uint16_t*)y2;
   p.out0_stride = H;
   return launch_varlen_m<TileCfg<false>, ROLE_PLAIN, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
+}
+
+extern "C" int smoe_down_projection_forward_combine(const void* y1, const void* w2, int64_t w2_stride_e,
+                                                    int64_t w2_stride_row, const void* b2, void* o,
+                                                    const float* scores, const int32_t* off,
+                                                    const int32_t* expert_schedule_order,
+                                                    const int32_t* x_gather_idx, const int32_t* s_scatter_idx,
+                                                    int64_t T, int64_t TK, int H, int I, int E, void* workspace,
+                                                    size_t workspace_bytes, void* stream) {
+  int rc = check_common(TK, H, I, E, workspace, workspace_bytes, "down_projection_forward_combine");
+  if (rc) return rc;
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(y1 && w2 && o && scores && off && x_gather_idx && s_scatter_idx && T > 0, SMOE_ERR_INVALID,
+               "down_projection_forward_combine: null pointer");
+  SMOE_REQUIRE_ALIGNED("down_projection_forward_combine", y1, w2, b2, o);
+  SMOE_REQUIRE(stride8(w2_stride_e) && stride8(w2_stride_row), SMOE_ERR_UNSUPPORTED,
+               "down_projection_forward_combine: weight strides must be multiples of 8 elements");
+  hipStream_t st = (hipStream_t)stream;
+  VarlenMParams p = {};
+  p.P = (const uint16_t*)y1;
+  p.p_stride = I;
+  p.Q = (const uint16_t*)w2;
+  p.q_stride_e = w2_stride_e;
+  p.q_stride_row = w2_stride_row;
+  p.off = off;
+  p.order = expert_schedule_order;
+  p.N = H;
+  p.Kdim = I;
+  p.bias = (const uint16_t*)b2;
+  p.out0 = (uint16_t*)o;
+  p.out0_stride = H;
+  p.out_rows = x_gather_idx;
+  p.scores = scores;
+  p.sidx = s_scatter_idx;
+  return launch_varlen_m<TileCfg<false>, ROLE_COMBINE, SMOE_ACT_SWIGLU>(p, off, workspace, TK, E, st);
 }
 
 // activation-gradient halves of the two backward operators; the weight-gradient halves live in gemm_varlen_k.hip

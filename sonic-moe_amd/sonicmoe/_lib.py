@@ -37,6 +37,7 @@ _SIGNATURES = {
         [_P, _P, _L, _L, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
     "smoe_down_projection_forward": (c_int, [_P, _P, _L, _L, _P, _P, _P, _P, _L, _I, _I, _I, _P, _Z, _P]),
+    "smoe_down_projection_forward_combine": (c_int, [_P, _P, _L, _L, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _P, _Z, _P]),
     "smoe_gather_sum": (c_int, [_P, _P, _P, _P, _P, _L, _I, _I, _P]),
     "smoe_dz_partial_cols": (c_int, [_I]),
     "smoe_down_projection_backward": (

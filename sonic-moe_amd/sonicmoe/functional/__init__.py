@@ -31,6 +31,7 @@ from .backward import (
 )
 from .forward import (
     _down_projection_forward,
+    _down_projection_forward_combine,
     _router_forward,
     _router_forward_fused,
     _softmax_topk_fwd,
@@ -206,6 +207,25 @@ def fused_router(enable: bool = True):
         _FUSED_ROUTER = previous
 
 
+_FUSED_COMBINE = os.environ.get("SMOE_FUSED_COMBINE", "0") == "1"
+
+
+@contextmanager
+def fused_combine(enable: bool = True):
+    """Inside the block the bf16 forward pass runs the down projection and the score-weighted combine as ONE kernel
+    (`_down_projection_forward_combine`): every output tile is scaled by its rows' routing scores and added onto the
+    tokens' output rows with packed-bf16 atomics, `y2` (TK, H) is never stored.  Off by default: on MI355X the atomic
+    traffic costs more than the stores of `y2` plus the separate gather-sum, the result carries bf16 accumulation error
+    (K roundings instead of one) and is not bit-reproducible from run to run.  The backward pass is unchanged (it never
+    reads `y2`)."""
+    global _FUSED_COMBINE
+    previous, _FUSED_COMBINE = _FUSED_COMBINE, enable
+    try:
+        yield
+    finally:
+        _FUSED_COMBINE = previous
+
+
 _SCHEDULE_POLICY = "expert_index"
 
 
@@ -254,7 +274,7 @@ def _schedule_order(off):
 
 
 def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K, activation_type,
-                     stream_id, inference, order=None):
+                     stream_id, inference, order=None, sidx=None):
     """o = combine(down(act(up(gather(x))))); returns (o, z) with z = None in inference mode."""
     T, H = x.shape
     N1, _, E = w1.shape
@@ -264,6 +284,12 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
 
     z = None if inference else torch.empty(TK, N1, dtype=x.dtype, device=x.device)
     y1 = None if is_using_fp8_forward() else torch.empty(TK, I, dtype=x.dtype, device=x.device)
+    if _FUSED_COMBINE and sidx is not None and not is_using_fp8_forward():
+        # down projection + combine in one kernel (atomic adds onto a zeroed output); y2 does not exist
+        _up_projection_forward(x, w1, z, y1, b1, off, order, gidx, stream_id, activation_type.value, glu, inference)
+        o = torch.zeros(T, H, dtype=x.dtype, device=x.device)
+        _down_projection_forward_combine(w2, y1, o, b2, scores_flat, off, order, gidx, sidx, stream_id)
+        return o, z
     y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
     if is_using_fp8_forward():
         # a step whose backward pass runs on fp8 operands too reads each weight once for both quantised copies
@@ -386,7 +412,7 @@ class _ExpertsFunction(torch.autograd.Function):
         scores_flat = scores_flat.contiguous()
         order = _schedule_order(off)
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K_or_maxK, is_varlen_K,
-                                activation_type, stream_id, inference, order)
+                                activation_type, stream_id, inference, order, sidx)
         ctx.order = order
         ctx.fp8_backward = _fp8_backward_requested(b1, b2, w1, w2)
         if not inference:
@@ -449,7 +475,7 @@ class _TCLayerFunction(torch.autograd.Function):
         scores_flat = scores.view(-1)
         order = _schedule_order(off)
         o, z = _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K, False, activation_type,
-                                stream_id, inference, order)
+                                stream_id, inference, order, sidx)
         ctx.order = order
         ctx.fp8_backward = _fp8_backward_requested(b1, b2, w1, w2)
         if not inference:
@@ -612,6 +638,7 @@ __all__ = [
     "enable_fp8_backward",
     "is_using_fp8_backward",
     "expert_schedule",
+    "fused_combine",
     "fused_router",
     "largest_first_schedule_order",
     "moe_TC_softmax_topk_layer",

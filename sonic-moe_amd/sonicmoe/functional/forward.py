@@ -173,6 +173,61 @@ def _down_projection_forward(
     _lib.check(rc, "_down_projection_forward")
 
 
+@torch.library.custom_op(f"{LIBRARY_NAME}::_down_projection_forward_combine", mutates_args={"o"})
+def _down_projection_forward_combine(
+    w2: torch.Tensor,
+    y1: torch.Tensor,
+    o: torch.Tensor,
+    b2: torch.Tensor | None,
+    topk_scores: torch.Tensor,
+    expert_frequency_offset: torch.Tensor,
+    expert_schedule_order: torch.Tensor | None,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    stream_id: int,
+) -> None:
+    """o[x_gather_idx[m]] += topk_scores[s_scatter_idx[m]] * (y1[m] W2[e]^T (+ b2[e])): the down projection and the
+    score-weighted combine (`_down_projection_forward` + `_router_forward`, sonicmoe/functional/forward.py:132-236) as
+    ONE kernel that never stores y2.  `o` (T, H) must be zero on entry.  The additions are packed-bf16 atomics: within
+    bf16 accumulation error of the two-kernel path, not bit-reproducible from run to run, and slower on MI355X; an
+    option (`sonicmoe.functional.fused_combine()`), not the default."""
+    _lib.require_device(w2, y1, o, b2, topk_scores, expert_frequency_offset, expert_schedule_order, x_gather_idx,
+                        s_scatter_idx)
+    _check_schedule_order(expert_schedule_order, w2.size(2))
+    _check_bf16(("w2", w2), ("y1", y1), ("o", o), ("b2", b2))
+    H, I, E = w2.shape
+    T, TK = o.size(0), y1.size(0)
+    assert y1.is_contiguous() and o.is_contiguous() and o.size(1) == H
+    assert topk_scores.dtype == torch.float32 and topk_scores.is_contiguous()
+    assert x_gather_idx.dtype == torch.int32 and s_scatter_idx.dtype == torch.int32
+    assert x_gather_idx.numel() == TK and s_scatter_idx.numel() == TK
+    assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous())
+    s_e, s_row = expert_major_strides(w2, "w2")
+    ws = _gemm_workspace(TK, E, y1.device, stream_id)
+    rc = _lib.lib().smoe_down_projection_forward_combine(
+        _lib.ptr(y1),
+        _lib.ptr(w2),
+        s_e,
+        s_row,
+        _lib.ptr(b2),
+        _lib.ptr(o),
+        _lib.ptr(topk_scores),
+        _lib.ptr(expert_frequency_offset),
+        _lib.ptr(expert_schedule_order),
+        _lib.ptr(x_gather_idx),
+        _lib.ptr(s_scatter_idx),
+        T,
+        TK,
+        H,
+        I,
+        E,
+        _lib.ptr(ws),
+        ws.numel(),
+        stream_id,
+    )
+    _lib.check(rc, "_down_projection_forward_combine")
+
+
 def _gather_sum(src, out, weights, ridx, tok_off, K, H, is_varlen_K, what):
     _lib.require_device(src, out, weights, ridx, tok_off)
     _check_bf16((what + ".src", src), (what + ".out", out))

@@ -99,6 +99,47 @@ def test_fused_layer_node_matches_three_nodes(dev, monkeypatch):
     assert torch.equal(g1[2], g0[2]) and torch.equal(g1[3], g0[3])
 
 
+def test_layer_with_fused_combine(dev):
+    """`with fused_combine():` - the down projection adds its score-weighted rows onto the output itself (atomics, no
+    y2): the output stays within the layer's tolerance of the two-kernel path, every gradient is bit-identical (the
+    backward pass never reads y2 or o), and the general-routing entry takes the same path."""
+    from sonicmoe.functional import fused_combine, moe_TC_softmax_topk_layer, moe_general_routing_inputs
+    from helpers import make_weights
+
+    T, H, I, E, K = 2048, 768, 256, 32, 4
+    wr, w1, w2 = make_weights(E, H, I, dev, seed=17)
+    g = torch.Generator().manual_seed(18)
+    x0 = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+
+    def run(fused):
+        x = x0.clone().requires_grad_()
+        ps = [p.detach().clone().requires_grad_() for p in (wr, w1, w2)]
+        with fused_combine(fused):
+            o, logits, freq = moe_TC_softmax_topk_layer(x, ps[0], ps[1].permute(1, 2, 0), None, ps[2].permute(1, 2, 0),
+                                                        None, K, 0)
+        return o, torch.autograd.grad((o.float() * dy.float()).sum(), [x] + ps)
+
+    o1, g1 = run(True)
+    o0, g0 = run(False)
+    assert rel_l2(o1, o0) < 1e-2
+    for a, b in zip(g1, g0):
+        assert torch.equal(a, b)
+
+    # general routing: explicit (token, expert, score) triples
+    scores = torch.softmax(torch.randn(T, K, generator=g), dim=-1).to(dev)
+    experts = torch.stack([torch.randperm(E, generator=g)[:K] for _ in range(T)]).to(torch.int32).to(dev)
+    tokens = torch.arange(T, dtype=torch.int32, device=dev).repeat_interleave(K)
+
+    def run_general(fused):
+        with fused_combine(fused), torch.no_grad():
+            out, _ = moe_general_routing_inputs(x0, scores.view(-1), tokens, experts.view(-1), w1.permute(1, 2, 0), None,
+                                                w2.permute(1, 2, 0), None, E, 0, "swiglu")
+        return out
+
+    assert rel_l2(run_general(True), run_general(False)) < 1e-2
+
+
 def test_module_aux_loss_value_and_gradient(dev):
     """MoE.forward's auxiliary loss on the HIP path (fused switch-loss kernels) against the oracle's formula on the
     same router logits and expert counts, differentiated by autograd: the value, and the gradients a loss of
