@@ -353,13 +353,21 @@ int smoe_mx_quantize_both(const void* src, int64_t src_stride_e, int64_t src_str
  *   doutq (T, H) bytes + dout_scales (H/128, T); w2tq (E, I, H) bytes + w2t_scales (H/128, E*I)
  *   (smoe_mx_quantize_transposed of W2); z (TK, N1) bf16; ds_partial: TK * smoe_dz_partial_cols(I) floats.
  * The weight and bias gradients are left to smoe_down_projection_backward with dz == NULL, which reads y1s.
- * Limits: H % 128 == 0, I % 64 == 0, N1 % 128 == 0; no b2 term in ds. */
+ * Limits: H % 128 == 0, I % 64 == 0, N1 % 128 == 0; no b2 term in ds (smoe_score_grad_bias_term adds it). */
 int smoe_down_projection_backward_fp8(const void* doutq, const void* dout_scales, const void* w2tq,
                                       const void* w2t_scales, const void* z, void* dz, void* dzq, void* dzq_scales,
                                       void* y1s, float* ds, float* ds_partial, const float* scores,
                                       const int32_t* off, const int32_t* x_gather_idx, const int32_t* s_scatter_idx,
                                       int64_t T, int64_t TK, int H, int I, int E, int activation, void* workspace,
                                       size_t workspace_bytes, void* stream);
+
+/* ds[s_scatter_idx[m]] += <dout[x_gather_idx[m]], b2[e(m)]> for the TK grouped rows m (e(m) from off): what the
+ * down-projection bias adds to the score gradient, the "dot(dout, b2)" of the reference's db2_and_ds_kernel
+ * (sonicmoe/functional/backward.py:36-107, called at :410-436).  smoe_down_projection_backward does this itself when it
+ * is given b2; this entry point is for a backward pass whose dz came from smoe_down_projection_backward_fp8.
+ * dout (T, H) bf16, b2 (E, H) bf16 contiguous, ds (TK) fp32 already holding the GEMM's part; H % 8 == 0. */
+int smoe_score_grad_bias_term(const void* dout, const void* b2, const int32_t* off, const int32_t* x_gather_idx,
+                              const int32_t* s_scatter_idx, float* ds, int64_t TK, int H, int E, void* stream);
 
 #ifdef __cplusplus
 }

@@ -196,3 +196,17 @@ extern "C" int smoe_gather_sum(const void* src, void* out, const float* w, const
   SMOE_LAUNCH_CHECK();
   return SMOE_OK;
 }
+
+extern "C" int smoe_score_grad_bias_term(const void* dout, const void* b2, const int32_t* off,
+                                         const int32_t* x_gather_idx, const int32_t* s_scatter_idx, float* ds,
+                                         int64_t TK, int H, int E, void* stream) {
+  SMOE_REQUIRE(TK >= 0 && E >= 1, SMOE_ERR_INVALID, "score_grad_bias_term: TK=%lld, E=%d", (long long)TK, E);
+  if (TK == 0) return SMOE_OK;
+  SMOE_REQUIRE(dout && b2 && off && x_gather_idx && s_scatter_idx && ds, SMOE_ERR_INVALID,
+               "score_grad_bias_term: null pointer");
+  SMOE_REQUIRE(H > 0 && H % 8 == 0, SMOE_ERR_UNSUPPORTED, "score_grad_bias_term: H=%d must be a positive multiple of 8",
+               H);
+  SMOE_REQUIRE_ALIGNED("score_grad_bias_term", dout, b2);
+  return launch_ds_bias_term((const uint16_t*)dout, (const uint16_t*)b2, x_gather_idx, s_scatter_idx, off, E, H, ds, TK,
+                             (hipStream_t)stream);
+}

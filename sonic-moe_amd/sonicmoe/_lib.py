@@ -73,6 +73,7 @@ _SIGNATURES = {
         [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _L, _L, _I, _I, _I, _I, _P, _Z, _P],
     ),
     "smoe_down_projection_forward_fp8": (c_int, [_P, _P, _P, _P, _P, _P, _P, _L, _I, _I, _I, _P, _Z, _P]),
+    "smoe_score_grad_bias_term": (c_int, [_P, _P, _P, _P, _P, _P, _L, _I, _I, _P]),
 }
 
 

@@ -44,6 +44,7 @@ from .forward import (
 from .fp8 import (
     _down_projection_backward_fp8,
     _down_projection_forward_fp8,
+    _score_grad_bias_term,
     _up_projection_forward_fp8,
     enable_fp8_backward,
     enable_fp8_forward,
@@ -254,13 +255,11 @@ def largest_first_schedule_order(expert_frequency_offset: torch.Tensor) -> torch
 
 def _fp8_backward_requested(b1, b2, w1=None, w2=None) -> bool:
     """The fp8-backward switch as it stands while the forward pass runs (the backward pass may run outside the block).
-    What the fp8 backward cannot do is refused here, in forward, not in the middle of a backward pass: biases, and
-    weight shapes whose transposed quantised copies do not split into 128-element blocks.  (The fp8 kernels take the
-    experts in index order: an expert_schedule policy only reorders the bf16 weight-gradient GEMMs of such a step.)"""
+    What the fp8 backward cannot do is refused here, in forward, not in the middle of a backward pass: weight shapes
+    whose transposed quantised copies do not split into 128-element blocks.  (The fp8 kernels take the experts in index
+    order: an expert_schedule policy only reorders the bf16 weight-gradient GEMMs of such a step.)"""
     if not is_using_fp8_backward():
         return False
-    if b1 is not None or b2 is not None:
-        raise NotImplementedError("enable_fp8_backward: layers with biases are not supported")
     if w1 is not None and (w1.size(0) % 128 != 0 or w1.size(1) % 128 != 0):
         # the activation gradients contract over the up-projection's output columns (dx) and over H (dz): both are
         # quantised in blocks along those indices
@@ -293,7 +292,7 @@ def _experts_forward(x, w1, b1, w2, b2, scores_flat, off, gidx, ridx, tok_off, K
     y2 = torch.empty(TK, H, dtype=x.dtype, device=x.device)
     if is_using_fp8_forward():
         # a step whose backward pass runs on fp8 operands too reads each weight once for both quantised copies
-        both = is_using_fp8_backward() and not inference and b1 is None and b2 is None
+        both = is_using_fp8_backward() and not inference
         quantize_weight = quantize_expert_weight_both if both else quantize_expert_weight
         xq, xs = mx_quantize(x)
         w1q, w1s = quantize_weight(w1)
@@ -326,8 +325,8 @@ def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx
     dout = dout.contiguous()
 
     if fp8:
-        return _experts_backward_fp8(dout, x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK,
-                                     is_varlen_K, activation_type, stream_id, order)
+        return _experts_backward_fp8(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK,
+                                     is_varlen_K, activation_type, stream_id, has_b1, order)
 
     dw2 = torch.empty_like(w2)  # keeps the (E, H, I)-contiguous layout of the parameter view
     db2 = None if b2 is None else torch.empty_like(b2)
@@ -346,11 +345,11 @@ def _experts_backward(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx
     return dx, dw1, db1, dw2, db2, ds
 
 
-def _experts_backward_fp8(dout, x, w1, w2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
-                          activation_type, stream_id, order):
-    """_experts_backward with the two activation-gradient GEMMs on fp8 operands (no biases): dout and W2^T are
-    quantised for dz, the dz kernel leaves dz in bf16 (for dW1) and quantised (for dx), W1^T is quantised for dx; dW2
-    and dW1 are the bf16 weight-gradient GEMMs."""
+def _experts_backward_fp8(dout, x, w1, w2, b2, z, scores_flat, off, gidx, sidx, ridx, tok_off, K_or_maxK, is_varlen_K,
+                          activation_type, stream_id, has_b1, order):
+    """_experts_backward with the two activation-gradient GEMMs on fp8 operands: dout and W2^T are quantised for dz,
+    the dz kernel leaves dz in bf16 (for dW1 and db1) and quantised (for dx), W1^T is quantised for dx; dW2 and dW1
+    are the bf16 weight-gradient GEMMs, and the bias gradients and the bias term of ds are the bf16 step's kernels."""
     T, H = x.shape
     TK = gidx.numel()
     N1, _, E = w1.shape
@@ -366,19 +365,23 @@ def _experts_backward_fp8(dout, x, w1, w2, z, scores_flat, off, gidx, sidx, ridx
     _down_projection_backward_fp8(doutq, dout_scales, w2tq, w2t_scales, z, dz, dzq, dzq_scales, y1s, ds, scores_flat,
                                   off, gidx, sidx, E, stream_id, activation_type.value, glu)
     del doutq, dout_scales, w2tq, w2t_scales
+    if b2 is not None:  # y2 = y1 W2^T + b2 puts <dout, b2> into the score gradient
+        _score_grad_bias_term(dout, b2, ds, off, gidx, sidx, stream_id)
     dw2 = torch.empty_like(w2)
-    _down_projection_weight_grad(dout, y1s, dw2, None, scores_flat, off, order, gidx, sidx, stream_id)
+    db2 = None if b2 is None else torch.empty_like(b2)
+    _down_projection_weight_grad(dout, y1s, dw2, db2, scores_flat, off, order, gidx, sidx, stream_id)
     del y1s
     w1tq, w1t_scales = quantize_expert_weight_transposed(w1)
     dx_expanded = torch.empty(TK, H, dtype=x.dtype, device=x.device)
     _down_projection_forward_fp8(dzq, dzq_scales, w1tq, w1t_scales, dx_expanded, None, off, E, stream_id)
     del dzq, dzq_scales, w1tq, w1t_scales
     dw1 = torch.empty_like(w1)
-    _up_projection_backward(x, w1, None, dw1, dz, None, off, order, gidx, sidx, glu, stream_id)
+    db1 = torch.empty(w1.size(2), w1.size(0), dtype=x.dtype, device=x.device) if has_b1 else None
+    _up_projection_backward(x, w1, None, dw1, dz, db1, off, order, gidx, sidx, glu, stream_id)
     del dz
     dx = torch.empty(T, H, dtype=x.dtype, device=x.device)
     _token_broadcast_backward(dx, dx_expanded, ridx, tok_off, K_or_maxK, H, is_varlen_K)
-    return dx, dw1, None, dw2, None, ds
+    return dx, dw1, db1, dw2, db2, ds
 
 
 class _ExpertsFunction(torch.autograd.Function):

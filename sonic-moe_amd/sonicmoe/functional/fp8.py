@@ -384,3 +384,30 @@ def _down_projection_backward_fp8(
         stream_id,
     )
     _lib.check(rc, "_down_projection_backward_fp8")
+
+
+@torch.library.custom_op(f"{LIBRARY_NAME}::_score_grad_bias_term", mutates_args={"ds"})
+def _score_grad_bias_term(
+    dout: torch.Tensor,
+    b2: torch.Tensor,
+    ds: torch.Tensor,
+    expert_frequency_offset: torch.Tensor,
+    x_gather_idx: torch.Tensor,
+    s_scatter_idx: torch.Tensor,
+    stream_id: int,
+) -> None:
+    """ds[s_scatter_idx[m]] += <dout[x_gather_idx[m]], b2[expert of m]>: the part of the score gradient that the
+    down-projection bias causes (the reference folds it into db2_and_ds_kernel, sonicmoe/functional/backward.py:36-107).
+    `_down_projection_backward` adds it itself; `_down_projection_backward_fp8` does not know b2."""
+    _lib.require_device(dout, b2, ds, expert_frequency_offset, x_gather_idx, s_scatter_idx)
+    _check_bf16(("dout", dout), ("b2", b2))
+    T, H = dout.shape
+    E = expert_frequency_offset.numel() - 1
+    TK = x_gather_idx.numel()
+    assert dout.is_contiguous() and b2.shape == (E, H) and b2.is_contiguous()
+    assert ds.dtype == torch.float32 and ds.numel() == TK and ds.is_contiguous() and s_scatter_idx.numel() == TK
+    rc = _lib.lib().smoe_score_grad_bias_term(
+        _lib.ptr(dout), _lib.ptr(b2), _lib.ptr(expert_frequency_offset), _lib.ptr(x_gather_idx), _lib.ptr(s_scatter_idx),
+        _lib.ptr(ds), TK, H, E, stream_id,
+    )
+    _lib.check(rc, "_score_grad_bias_term")

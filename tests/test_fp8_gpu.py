@@ -241,9 +241,41 @@ def test_layer_with_fp8_forward_and_backward(dev):
     # fp8 forward and backward in series (three quantised GEMMs on the way to dx): measured 5.4e-2 .. 6.7e-2, outside
     # the 5e-2 stated for fp8 -- recorded bound, like the forward-only layer test below
     assert all(e < 9e-2 for e in errs8), errs8
-    moe_b = MoE(E, K, H, I, ActivationType.SWIGLU, True, 0.02).to(device=dev, dtype=torch.bfloat16)
-    with enable_fp8_backward(), pytest.raises(NotImplementedError, match="biases"):
-        moe_b(x)
+
+
+@pytest.mark.parametrize("fp8_forward", [False, True])
+def test_layer_with_biases_and_fp8_backward(dev, fp8_forward):
+    """A layer with biases through the fp8 backward: db1 (column sums of the bf16 dz the fp8 kernel stores), db2 and the
+    <dout, b2> term of the score gradient come from the bf16 step's kernels, against the bf16 path of the same module."""
+    from contextlib import nullcontext
+
+    from sonicmoe import MoE, enable_fp8_backward, enable_fp8_forward
+    from sonicmoe.enums import ActivationType
+
+    T, H, I, E, K = 1536, 512, 256, 8, 2
+    torch.manual_seed(11)
+    moe = MoE(E, K, H, I, ActivationType.SWIGLU, True, 0.02).to(device=dev, dtype=torch.bfloat16)
+    with torch.no_grad():   # biases so large that <dout, b2> dominates the score gradient: dWr fails without the term
+        moe.c_fc.bias.copy_(torch.randn_like(moe.c_fc.bias) * 0.5)
+        moe.c_proj.bias.copy_(torch.randn_like(moe.c_proj.bias) * 0.5)
+    x = torch.randn(T, H, device=dev).to(torch.bfloat16).requires_grad_()
+    dy = torch.randn(T, H, device=dev).to(torch.bfloat16)
+    params = [moe.router.weight, moe.c_fc.weight, moe.c_fc.bias, moe.c_proj.weight, moe.c_proj.bias]
+    out, _ = moe(x)
+    grads = torch.autograd.grad(out, [x] + params, grad_outputs=dy)
+    with (enable_fp8_forward() if fp8_forward else nullcontext()), enable_fp8_backward():
+        out8, _ = moe(x)
+        grads8 = torch.autograd.grad(out8, [x] + params, grad_outputs=dy)
+    if not fp8_forward:
+        assert torch.equal(out8, out)
+    errs = dict(zip(["dx", "dWr", "dW1", "db1", "dW2", "db2"], [rel_l2(a, b) for a, b in zip(grads8, grads)]))
+    print("fp8 backward with biases, fp8 forward =", fp8_forward, errs)
+    if not fp8_forward:
+        assert errs["db2"] < 1e-6 and errs["dW2"] < 1e-2, errs   # no quantised GEMM on their way
+        assert errs["dWr"] < 5e-2 and errs["dW1"] < 5e-2 and errs["db1"] < 5e-2, errs   # one quantised GEMM
+        assert errs["dx"] < 7e-2, errs                            # two in series: the bound of the test above
+    else:
+        assert all(e < 9e-2 for e in errs.values()), errs
 
 
 def test_layer_with_fp8_forward(dev):
