@@ -1,8 +1,10 @@
-"""Build libsonicmoe_hip.so (gfx950) from csrc/*.hip with hipcc.  No torch headers, no pybind: plain C ABI.
+"""Build libsonicmoe_hip.so and libsonicmoe_hip_f16.so (gfx950) from csrc/*.hip with hipcc.  No torch headers, no
+pybind: plain C ABI.  The two libraries come from the same sources and export the same entry points; the first takes
+bf16 for the 16-bit tensors of the GEMM-side operators, the second (compiled with -DSMOE_ELEM_F16) fp16.
 
     python sonic-moe_amd/build.py [--verbose] [--resource-usage]
 
-The library lands in sonic-moe_amd/sonicmoe/lib/ so that it travels with the source tree.
+The libraries land in sonic-moe_amd/sonicmoe/lib/ so that they travel with the source tree.
 """
 
 from __future__ import annotations
@@ -19,6 +21,8 @@ CSRC = ROOT / "csrc"
 OUT_DIR = ROOT / "sonicmoe" / "lib"
 OBJ_DIR = ROOT / "build"
 LIB_NAME = "libsonicmoe_hip.so"
+# (library, extra compiler flags, suffix of the object files)
+VARIANTS = [(LIB_NAME, [], ""), ("libsonicmoe_hip_f16.so", ["-DSMOE_ELEM_F16"], "_f16")]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -57,21 +61,26 @@ def build(verbose: bool = False, resource_usage: bool = False, jobs: int | None 
     OUT_DIR.mkdir(parents=True, exist_ok=True)
     extra = ["-Rpass-analysis=kernel-resource-usage"] if resource_usage else []
 
-    def compile_one(src: Path) -> Path:
-        obj = OBJ_DIR / (src.stem + ".o")
-        out = _run([HIPCC, *FLAGS, *extra, "-c", str(src), "-o", str(obj)], verbose)
+    def compile_one(job: tuple[Path, list[str], str]) -> Path:
+        src, defines, suffix = job
+        obj = OBJ_DIR / (src.stem + suffix + ".o")
+        out = _run([HIPCC, *FLAGS, *defines, *extra, "-c", str(src), "-o", str(obj)], verbose)
         if out.strip() and (verbose or resource_usage):
             print(out, flush=True)
         return obj
 
-    jobs = jobs or min(len(sources), os.cpu_count() or 1, 8)
+    # the longest compilations first: the wall time is the largest source's either way
+    sources.sort(key=lambda p: -p.stat().st_size)
+    work = [(src, defines, suffix) for src in sources for _, defines, suffix in VARIANTS]
+    jobs = jobs or min(len(work), os.cpu_count() or 1, 8)
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(compile_one, sources))
-    lib = OUT_DIR / LIB_NAME
-    tmp = OUT_DIR / (LIB_NAME + ".tmp")
-    _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)], verbose)
-    os.replace(tmp, lib)
-    return lib
+        objs = list(ex.map(compile_one, work))
+    for name, _, suffix in VARIANTS:
+        mine = [o for o, (_, _, sfx) in zip(objs, work) if sfx == suffix]
+        tmp = OUT_DIR / (name + ".tmp")
+        _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, mine)], verbose)
+        os.replace(tmp, OUT_DIR / name)
+    return OUT_DIR / LIB_NAME
 
 
 if __name__ == "__main__":

@@ -42,14 +42,14 @@ __global__ __launch_bounds__(512) void gather_sum_kernel(const uint16_t* __restr
       for (int u = 0; u < UNROLL; u++) {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-          acc[2 * q] += ws[u] * bf16_lo(v[u][q]);
-          acc[2 * q + 1] += ws[u] * bf16_hi(v[u][q]);
+          acc[2 * q] += ws[u] * elem_lo(v[u][q]);
+          acc[2 * q + 1] += ws[u] * elem_hi(v[u][q]);
         }
       }
     }
     u32x4 o;
 #pragma unroll
-    for (int q = 0; q < 4; q++) o[q] = pack_bf16x2(acc[2 * q], acc[2 * q + 1]);
+    for (int q = 0; q < 4; q++) o[q] = pack_elem2(acc[2 * q], acc[2 * q + 1]);
     __builtin_nontemporal_store(o, (u32x4*)(out + t * H + (int64_t)c * 8));
   }
 }
@@ -109,8 +109,8 @@ __global__ __launch_bounds__(256) void expert_colsum_kernel(const uint16_t* __re
     for (int u = 0; u < UNROLL; u++)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
-        acc[2 * q] += w[u] * bf16_lo(v[u][q]);
-        acc[2 * q + 1] += w[u] * bf16_hi(v[u][q]);
+        acc[2 * q] += w[u] * elem_lo(v[u][q]);
+        acc[2 * q + 1] += w[u] * elem_hi(v[u][q]);
       }
   }
 #pragma unroll
@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void expert_colsum_kernel(const uint16_t* __re
       const float a = part[0][lane][2 * q] + part[1][lane][2 * q] + part[2][lane][2 * q] + part[3][lane][2 * q];
       const float b = part[0][lane][2 * q + 1] + part[1][lane][2 * q + 1] + part[2][lane][2 * q + 1] +
                       part[3][lane][2 * q + 1];
-      o[q] = pack_bf16x2(a, b);
+      o[q] = pack_elem2(a, b);
     }
     *(u32x4*)(out + (int64_t)e * ncols + col) = o;
   }
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(256) void ds_bias_term_kernel(const uint16_t* __res
   for (int c = lane * 8; c < H; c += 512) {
     const u32x4 a = *(const u32x4*)(row + c), b = *(const u32x4*)(bias + c);
 #pragma unroll
-    for (int q = 0; q < 4; q++) s += bf16_lo(a[q]) * bf16_lo(b[q]) + bf16_hi(a[q]) * bf16_hi(b[q]);
+    for (int q = 0; q < 4; q++) s += elem_lo(a[q]) * elem_lo(b[q]) + elem_hi(a[q]) * elem_hi(b[q]);
   }
 #pragma unroll
   for (int d = 32; d >= 1; d >>= 1) s += __shfl_xor(s, d, 64);

@@ -43,8 +43,8 @@ __global__ __launch_bounds__(256) void mx_quantize_kernel(const uint16_t* __rest
       const u32x4 w = p[i];
 #pragma unroll
       for (int j = 0; j < 4; j++) {
-        v[i * 8 + 2 * j] = bf16_lo(w[j]);
-        v[i * 8 + 2 * j + 1] = bf16_hi(w[j]);
+        v[i * 8 + 2 * j] = elem_lo(w[j]);
+        v[i * 8 + 2 * j + 1] = elem_hi(w[j]);
       }
     }
 #pragma unroll
@@ -153,7 +153,7 @@ struct Fp8Mma {
   typedef Fp8Frag Frag;
   typedef f32x16 Acc;
   // a step is ONE of the wave's four token fragments on one k-slice of 64 contraction bytes; the feature fragments
-  // are read on the first of a slice's four steps (see Bf16Mma16).  Two sets of 1 + 2 fragments are live.
+  // are read on the first of a slice's four steps (see ElemMma16).  Two sets of 1 + 2 fragments are live.
   static constexpr int FR = 32, KSTEP = 64, PH = 4, ACC_REGS = 16, FRAG_REGS = 9;
   static constexpr int qset(int step) { return (step >> 2) & 1; }
   static constexpr int phalf(int step) { return step & 3; }
@@ -745,8 +745,8 @@ __global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint1
 #pragma unroll
       for (int i = 0; i < 16; i++) {
         const uint32_t two = *(const uint32_t*)(tile_in + r * IN_PITCH + hb * 128 + blk * 64 + i * 4);
-        w[2 * i] = bf16_lo(two);
-        w[2 * i + 1] = bf16_hi(two);
+        w[2 * i] = elem_lo(two);
+        w[2 * i + 1] = elem_hi(two);
         am = fmaxf(am, fmaxf(fabsf(w[2 * i]), fabsf(w[2 * i + 1])));
       }
       const int exr = mx_scale_exponent(am);
@@ -777,7 +777,7 @@ __global__ __launch_bounds__(256) void mx_quantize_transposed_kernel(const uint1
 #pragma unroll
     for (int i = 0; i < 32; i++) {
       const uint16_t h = *(const uint16_t*)(tile_in + (rb * 32 + i) * IN_PITCH + c * 2);
-      v[i] = __uint_as_float((uint32_t)h << 16);
+      v[i] = elem_bits_to_f32(h);
       amax = fmaxf(amax, fabsf(v[i]));
     }
     const int ex = mx_scale_exponent(amax);

@@ -35,7 +35,7 @@ struct KCfg {
   static constexpr int BA = BA_, BB = BB_, WA = WA_, WB = WB_, BK = BK_, NSTAGE = NSTAGE_;
   static constexpr bool R_GATHER = R_GATHER_, S_GATHER = S_GATHER_;
   static constexpr int NW = WA * WB, NT = NW * 64;
-  typedef Bf16Mma Mma;
+  typedef ElemMma Mma;
   static constexpr int TA = BA / WA, TB = BB / WB;
   static constexpr int FR = Mma::FR;                   // rows / columns of a matrix-instruction fragment
   static constexpr int FA = TA / FR, FB = TB / FR;     // fragments of the wave tile
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
       for (int j = 0; j < RPW; j++) tok[j] = tok_next[j];
     }
   };
-  auto load = [&](int buf, int /*s*/, auto step_c, bf16x8(&sf)[FB], bf16x8(&rf)[C::NP]) {
+  auto load = [&](int buf, int /*s*/, auto step_c, elemx8(&sf)[FB], elemx8(&rf)[C::NP]) {
     constexpr int step = decltype(step_c)::value;
     constexpr int kofs = Mma::kslice(step) * Mma::KSTEP, ph = Mma::phalf(step);
     const char* st = smem + buf * C::STAGE;
@@ -287,8 +287,8 @@ __global__ __launch_bounds__(C::NT) void varlen_k_kernel(const VarlenKParams p) 
     constexpr int fa = decltype(fa_c)::value;
     static_for<FB * QPF>([&](auto q_c) {
       constexpr int fb = decltype(q_c)::value / QPF, rg = decltype(q_c)::value % QPF;
-      u32x2 v = {pack_bf16x2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
-                 pack_bf16x2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
+      u32x2 v = {pack_elem2(acc[fb][fa][4 * rg + 0], acc[fb][fa][4 * rg + 1]),
+                 pack_elem2(acc[fb][fa][4 * rg + 2], acc[fb][fa][4 * rg + 3])};
       *(u32x2*)(region + (fa * FR + AL::row(lane)) * L::ROW_BYTES + (fb * FR + AL::col(rg, lane)) * 2) = v;
     });
   });
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(256) void varlen_k_stream_kernel(const VarlenKParam
                                                               const int32_t* table, int max_rounds) {
   static_assert(RG != SG, "exactly one operand is gathered");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  typedef Bf16Mma Mma;
+  typedef ElemMma Mma;
   constexpr int BA = 256, BB = 256, TA = 128, TB = 128, BK = 64, ROWB = 512, NINSTR = SMOE_TL_P_INSTR;
   static_assert(TA / 16 == SMOE_TL_FM && TB / 16 == SMOE_TL_FN && Mma::FR == 16, "the generated loop is written for this tile shape");
   const uint32_t smem_base = lds_address(smem);

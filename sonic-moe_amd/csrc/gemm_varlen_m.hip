@@ -44,7 +44,7 @@ struct Cfg {
   static constexpr int BM = BM_, BN = BN_, WM = WM_, WN = WN_, BK = BK_, NSTAGE = NSTAGE_;
   static constexpr bool QMN = QMN_;
   static constexpr int NW = WM * WN, NT = NW * 64;
-  typedef Bf16Mma Mma;
+  typedef ElemMma Mma;
   static constexpr int TM = BM / WM, TN = BN / WN;
   static constexpr int FR = Mma::FR;                       // rows / columns of a matrix-instruction fragment
   static constexpr int FM = TM / FR, FN = TN / FR;         // fragments of the wave tile
@@ -113,7 +113,7 @@ SMOE_DEV void fragment_offsets(int wm, int wn, int lane, int (&p_off)[C::KSL], i
 // k-slice
 template <class C, int STEP>
 SMOE_DEV void read_fragments(const char* sp, const char* sq, const int (&p_off)[C::KSL],
-                             const int (&q_off)[C::QMN ? 2 * C::FN : C::KSL], bf16x8 (&qf)[C::FN], bf16x8 (&pf)[C::NP]) {
+                             const int (&q_off)[C::QMN ? 2 * C::FN : C::KSL], elemx8 (&qf)[C::FN], elemx8 (&pf)[C::NP]) {
   using Mma = typename C::Mma;
   constexpr int ksl = Mma::kslice(STEP), ph = Mma::phalf(STEP);
 #pragma unroll
@@ -219,7 +219,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_kernel(const VarlenMParams p) 
     load16_to_lds(q_src[j], smem_base + Q_RING + slot * C::Q_STAGE + (wave * C::Q_INSTR + j) * 1024);
     q_src[j] += q_step;
   };
-  auto load = [&](int p_slot, int q_slot, auto step_c, bf16x8(&qf)[FN], bf16x8(&pf)[C::NP]) {
+  auto load = [&](int p_slot, int q_slot, auto step_c, elemx8(&qf)[FN], elemx8(&pf)[C::NP]) {
     read_fragments<C, decltype(step_c)::value>(smem + p_slot * C::P_STAGE, smem + Q_RING + q_slot * C::Q_STAGE, p_off,
                                                q_off, qf, pf);
   };
@@ -406,7 +406,7 @@ __global__ __launch_bounds__(C::NT) void varlen_m_stream_kernel(const VarlenMPar
       point_q(nxt);
     }
   };
-  auto load = [&](int p_slot, int q_slot, auto step_c, bf16x8(&qf)[FN], bf16x8(&pf)[C::NP]) {
+  auto load = [&](int p_slot, int q_slot, auto step_c, elemx8(&qf)[FN], elemx8(&pf)[C::NP]) {
     read_fragments<C, decltype(step_c)::value>(smem + p_slot * C::P_STAGE, smem + Q_RING + q_slot * C::Q_STAGE, p_off,
                                                q_off, qf, pf);
   };

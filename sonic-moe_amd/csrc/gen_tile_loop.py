@@ -640,6 +640,12 @@ def mm_operands():
     return outs, ins
 
 
+def asm_text(line: str) -> str:
+    """An instruction as it stands inside the asm statement's string literals: the matrix instructions take the suffix
+    of the library's 16-bit element type (bf16 or f16) from the macro SMOE_ELEM_ASM."""
+    return line.replace("v_mfma_f32_16x16x32_bf16", 'v_mfma_f32_16x16x32_" SMOE_ELEM_ASM "')
+
+
 def mm_statement(name: str, lines: list[str], with_matrix: bool) -> str:
     outs, ins = mm_operands()
     clob = [f"v{i}" for i in range(MV_T, MV_T + 2)]
@@ -650,7 +656,7 @@ def mm_statement(name: str, lines: list[str], with_matrix: bool) -> str:
     params = ", ".join(n for _, n in outs + ins)
     body = [f"#define {name}({params}) \\", "  asm volatile( \\"]
     for ln in lines:
-        body.append(f'    "{ln}\\n\\t" \\')
+        body.append(f'    "{asm_text(ln)}\\n\\t" \\')
     body.append("    : " + ", ".join(f'"+{{{r}}}"({n})' for r, n in outs) + " \\")
     body.append("    : " + ", ".join(f'"{{{r}}}"({n})' for r, n in ins) + " \\")
     cl = [", ".join(f'"{c}"' for c in clob[i:i + 16]) for i in range(0, len(clob), 16)]
@@ -693,7 +699,7 @@ def statement(name: str, qmn: bool) -> str:
     params = ", ".join(n for _, n in outs + ins)
     body = [f"#define {name}({params}) \\", "  asm volatile( \\"]
     for ln in lines:
-        body.append(f'    "{ln}\\n\\t" \\')
+        body.append(f'    "{asm_text(ln)}\\n\\t" \\')
     body.append("    : " + ", ".join(f'"+{{{r}}}"({n})' for r, n in outs) + " \\")
     body.append("    : " + ", ".join(f'"{{{r}}}"({n})' for r, n in ins) + " \\")
     # clobber list, a few per line

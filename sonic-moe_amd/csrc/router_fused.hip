@@ -21,6 +21,15 @@
 
 namespace smoe {
 
+// This kernel is bf16 whatever the library's element type: the winner search orders the logits by the 16 bits of their
+// bf16 form.  The fp16 build of the library refuses the entry point and callers take the unfused chain.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+SMOE_DEV uint32_t pack_bf16x2(float lo, float hi) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
+}
+
 SMOE_DEV uint32_t rf_orderable(uint32_t bits) { return bits ^ ((bits >> 31) ? 0xffffffffu : 0x80000000u); }
 SMOE_DEV uint32_t rf_unorderable(uint32_t o) { return o ^ ((o >> 31) ? 0x80000000u : 0xffffffffu); }
 SMOE_DEV uint64_t rf_shfl_xor_u64(uint64_t v, int mask) {
@@ -240,6 +249,9 @@ extern "C" int smoe_router_forward_fused(const void* x, const void* wr, int64_t 
   SMOE_REQUIRE(H >= 32 * RF_XB && H % (32 * RF_XB) == 0, SMOE_ERR_UNSUPPORTED,
                "router_forward_fused: H=%d must be a multiple of %d", H, 32 * RF_XB);
   SMOE_REQUIRE(K >= 1 && K <= E, SMOE_ERR_INVALID, "router_forward_fused: K=%d out of range [1, E]", K);
+#ifdef SMOE_ELEM_F16
+  SMOE_REQUIRE(false, SMOE_ERR_UNSUPPORTED, "router_forward_fused: bf16 only (this is the fp16 build of the library)");
+#endif
   if (T == 0) return SMOE_OK;
   SMOE_REQUIRE(x && wr && logits && scores && indices, SMOE_ERR_INVALID, "router_forward_fused: null pointer");
   SMOE_REQUIRE_ALIGNED("router_forward_fused", x, wr, logits);

@@ -1,7 +1,8 @@
-"""ctypes binding of libsonicmoe_hip.so (declared in include/sonicmoe_hip.h).
+"""ctypes binding of libsonicmoe_hip.so and libsonicmoe_hip_f16.so (declared in include/sonicmoe_hip.h).
 
-The library is the only compute path of the `sonicmoe` backend: if it is missing or fails to load, every operator
-raises.  There is no eager / CPU fallback.
+The two libraries are builds of the same sources with the same entry points: the first takes bfloat16 for the 16-bit
+tensors of the GEMM-side operators, the second float16.  They are the only compute path of the `sonicmoe` backend: if
+the one an operator needs is missing or fails to load, the operator raises.  There is no eager / CPU fallback.
 """
 
 from __future__ import annotations
@@ -13,7 +14,9 @@ from pathlib import Path
 
 import torch
 
-_LIB: ctypes.CDLL | None = None
+_LIBS: dict[torch.dtype, ctypes.CDLL] = {}
+_LAST: ctypes.CDLL | None = None   # the library of the latest lib() call: check() asks it for the error text
+_TUNING: dict[str, int] = {}       # overrides made so far, for a library that is loaded later
 
 DT_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
@@ -77,15 +80,24 @@ _SIGNATURES = {
 }
 
 
-def library_path() -> Path:
-    env = os.environ.get("SONICMOE_HIP_LIB")
-    return Path(env) if env else Path(__file__).resolve().parent / "lib" / "libsonicmoe_hip.so"
+_LIB_FILES = {torch.bfloat16: ("libsonicmoe_hip.so", "SONICMOE_HIP_LIB"),
+              torch.float16: ("libsonicmoe_hip_f16.so", "SONICMOE_HIP_LIB_F16")}
 
 
-def lib() -> ctypes.CDLL:
-    global _LIB
-    if _LIB is None:
-        path = library_path()
+def library_path(dtype: torch.dtype = torch.bfloat16) -> Path:
+    name, var = _LIB_FILES[dtype]
+    env = os.environ.get(var)
+    return Path(env) if env else Path(__file__).resolve().parent / "lib" / name
+
+
+def lib(dtype: torch.dtype = torch.bfloat16) -> ctypes.CDLL:
+    """The library whose 16-bit element type is `dtype` (operators without such tensors use the default)."""
+    global _LAST
+    handle = _LIBS.get(dtype)
+    if handle is None:
+        if dtype not in _LIB_FILES:
+            raise NotImplementedError(f"no build of the HIP library for {dtype} tensors (bfloat16 and float16 exist)")
+        path = library_path(dtype)
         if not path.exists():
             raise RuntimeError(
                 f"{path} not found: the HIP library is not built (run `python sonic-moe_amd/build.py`); "
@@ -96,8 +108,11 @@ def lib() -> ctypes.CDLL:
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        _LIB = handle
-    return _LIB
+        for name, value in _TUNING.items():
+            handle.smoe_set_tuning(name.encode(), value)
+        _LIBS[dtype] = handle
+    _LAST = handle
+    return handle
 
 
 def exported_symbols() -> list[str]:
@@ -106,13 +121,19 @@ def exported_symbols() -> list[str]:
 
 def check(rc: int, what: str) -> None:
     if rc != 0:
-        msg = lib().smoe_last_error().decode(errors="replace")
+        msg = (_LAST or lib()).smoe_last_error().decode(errors="replace")
         raise RuntimeError(f"{what} failed (status {rc}): {msg}")
 
 
 def set_tuning(name: str, value: int) -> None:
-    """Override a kernel-selection knob of the library (value < 0 restores the default)."""
-    check(lib().smoe_set_tuning(name.encode(), int(value)), f"smoe_set_tuning({name}, {value})")
+    """Override a kernel-selection knob (value < 0 restores the default) in every build of the library, those loaded
+    later included."""
+    for handle in list(_LIBS.values()) or [lib()]:
+        rc = handle.smoe_set_tuning(name.encode(), int(value))
+        if rc != 0:
+            raise RuntimeError(f"smoe_set_tuning({name}, {value}) failed (status {rc}): "
+                               f"{handle.smoe_last_error().decode(errors='replace')}")
+    _TUNING[name] = int(value)
 
 
 def ptr(t: torch.Tensor | None):

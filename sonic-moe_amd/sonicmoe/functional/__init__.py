@@ -441,7 +441,8 @@ def _router_wgrad(dlogits: torch.Tensor, x: torch.Tensor, like: torch.Tensor) ->
     contraction elements, which a library GEMM without a split runs on an eighth of the chip), torch otherwise."""
     T, E = dlogits.shape
     H = x.size(1)
-    fast = x.is_cuda and x.dtype == torch.bfloat16 and dlogits.dtype == torch.bfloat16 and E % 8 == 0 and H % 8 == 0
+    fast = (x.is_cuda and x.dtype in (torch.bfloat16, torch.float16) and dlogits.dtype == x.dtype and E % 8 == 0
+            and H % 8 == 0)
     if fast and T >= 256 and os.environ.get("SMOE_ROUTER_WGRAD", "1") != "0":
         partial = torch.empty(router_weight_grad_chunks(T, E, H), E, H, dtype=x.dtype, device=x.device)
         _router_weight_grad(dlogits.contiguous(), x.contiguous(), partial)

@@ -9,7 +9,7 @@ import torch
 from .. import _lib
 from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
 from ..utils import expert_major_strides
-from .forward import _check_bf16, _check_schedule_order, _gather_sum, _gemm_workspace
+from .forward import _check_schedule_order, _elem_dtype, _gather_sum, _gemm_workspace
 
 
 @torch.library.custom_op(f"{LIBRARY_NAME}::_up_projection_backward", mutates_args={"dw1", "dx_expanded", "db1"})
@@ -31,7 +31,7 @@ def _up_projection_backward(
     output may be None to skip it."""
     _lib.require_device(x, w1, dx_expanded, dw1, db1, dz, expert_frequency_offset, expert_schedule_order, x_gather_idx)
     _check_schedule_order(expert_schedule_order, w1.size(2))
-    _check_bf16(("x", x), ("w1", w1), ("dx_expanded", dx_expanded), ("dw1", dw1), ("db1", db1), ("dz", dz))
+    dt = _elem_dtype(("x", x), ("w1", w1), ("dx_expanded", dx_expanded), ("dw1", dw1), ("db1", db1), ("dz", dz))
     N1, H, E = w1.shape
     I = N1 // 2 if is_glu_activation else N1
     T, TK = x.size(0), dz.size(0)
@@ -40,7 +40,7 @@ def _up_projection_backward(
     w_se, w_sr = expert_major_strides(w1, "w1")
     d_se, d_sr = expert_major_strides(dw1, "dw1") if dw1 is not None else (0, 0)
     ws = _gemm_workspace(TK, E, x.device, stream_id)
-    rc = _lib.lib().smoe_up_projection_backward(
+    rc = _lib.lib(dt).smoe_up_projection_backward(
         _lib.ptr(x),
         _lib.ptr(w1),
         w_se,
@@ -92,7 +92,7 @@ def _down_projection_backward(
     _lib.require_device(dout, z, w2, dw2, dz, ds, b2, db2, topk_scores, expert_frequency_offset, expert_schedule_order,
                         x_gather_idx, s_scatter_idx)
     _check_schedule_order(expert_schedule_order, w2.size(2))
-    _check_bf16(("dout", dout), ("z", z), ("w2", w2), ("dw2", dw2), ("dz", dz), ("b2", b2), ("db2", db2))
+    dt = _elem_dtype(("dout", dout), ("z", z), ("w2", w2), ("dw2", dw2), ("dz", dz), ("b2", b2), ("db2", db2))
     H, I, E = w2.shape
     assert (b2 is None) == (db2 is None), "b2 and db2 have to be given together"
     assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous() and db2.shape == (E, H) and db2.is_contiguous())
@@ -104,10 +104,10 @@ def _down_projection_backward(
     w_se, w_sr = expert_major_strides(w2, "w2")
     d_se, d_sr = expert_major_strides(dw2, "dw2") if dw2 is not None else (0, 0)
     y1s = torch.empty(TK, I, dtype=z.dtype, device=z.device)
-    ncols = _lib.lib().smoe_dz_partial_cols(I)
+    ncols = _lib.lib(dt).smoe_dz_partial_cols(I)
     ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
     ws = _gemm_workspace(TK, E, z.device, stream_id)
-    rc = _lib.lib().smoe_down_projection_backward(
+    rc = _lib.lib(dt).smoe_down_projection_backward(
         _lib.ptr(dout),
         _lib.ptr(z),
         _lib.ptr(w2),
@@ -157,7 +157,7 @@ def _down_projection_weight_grad(
     db2[e] = sum_m s dout[t_m], from the y1s = s * act(z) an earlier call (the fp8 activation-gradient operator) left."""
     _lib.require_device(dout, y1s, dw2, db2, topk_scores, expert_frequency_offset, expert_schedule_order, x_gather_idx,
                         s_scatter_idx)
-    _check_bf16(("dout", dout), ("y1s", y1s), ("dw2", dw2), ("db2", db2))
+    dt = _elem_dtype(("dout", dout), ("y1s", y1s), ("dw2", dw2), ("db2", db2))
     T, H = dout.shape
     TK, I = y1s.shape
     E = expert_frequency_offset.numel() - 1
@@ -168,7 +168,7 @@ def _down_projection_weight_grad(
     assert db2 is None or (db2.shape == (E, H) and db2.is_contiguous())
     d_se, d_sr = expert_major_strides(dw2, "dw2") if dw2 is not None else (0, 0)
     ws = _gemm_workspace(TK, E, dout.device, stream_id)
-    rc = _lib.lib().smoe_down_projection_backward(
+    rc = _lib.lib(dt).smoe_down_projection_backward(
         _lib.ptr(dout), None, None, 0, 0, None, _lib.ptr(dw2), d_se, d_sr, _lib.ptr(db2), None, _lib.ptr(y1s), None,
         None, _lib.ptr(topk_scores), _lib.ptr(expert_frequency_offset), _lib.ptr(expert_schedule_order),
         _lib.ptr(x_gather_idx), _lib.ptr(s_scatter_idx), T, TK, H, I, E, 0, _lib.ptr(ws), ws.numel(), stream_id,
@@ -236,13 +236,12 @@ def _router_weight_grad(dlogits: torch.Tensor, x: torch.Tensor, partial: torch.T
     """partial[c] (E, H) = dlogits[rows of chunk c]^T x[rows of chunk c]; the chunks are partial.size(0) equal token
     ranges.  Their sum is the weight gradient of router_logits = F.linear(x, router_w)."""
     _lib.require_device(dlogits, x, partial)
-    if dlogits.dtype != torch.bfloat16 or x.dtype != torch.bfloat16 or partial.dtype != torch.bfloat16:
-        raise NotImplementedError("_router_weight_grad: bf16 only")
+    dt = _elem_dtype(("dlogits", dlogits), ("x", x), ("partial", partial))
     T, E = dlogits.shape
     H = x.size(1)
     assert dlogits.is_contiguous() and x.is_contiguous() and partial.is_contiguous()
     assert x.size(0) == T and partial.shape[1:] == (E, H)
-    rc = _lib.lib().smoe_router_weight_grad(
+    rc = _lib.lib(dt).smoe_router_weight_grad(
         _lib.ptr(dlogits), _lib.ptr(x), _lib.ptr(partial), T, E, H, partial.size(0), _lib.current_stream_handle()
     )
     _lib.check(rc, "_router_weight_grad")

@@ -35,7 +35,24 @@ def _gemm_workspace(TK: int, E: int, device, stream_id: int, fp8_gathered_k: int
 def _check_bf16(*named):
     for name, t in named:
         if t is not None and t.dtype != torch.bfloat16:
-            raise NotImplementedError(f"{name}: the HIP grouped GEMMs take bfloat16 tensors, got {t.dtype}")
+            raise NotImplementedError(f"{name}: this operator takes bfloat16 tensors, got {t.dtype}")
+
+
+def _elem_dtype(*named) -> torch.dtype:
+    """The 16-bit element type of an operator call (it selects the library build, `_lib.lib(dtype)`): every tensor
+    given has the same one, bfloat16 or float16 -- the types the reference's grouped GEMMs take
+    (sonicmoe/functional/grouped_gemm.py:3033-3044)."""
+    dt = None
+    for name, t in named:
+        if t is None:
+            continue
+        if t.dtype not in (torch.bfloat16, torch.float16):
+            raise NotImplementedError(f"{name}: the HIP grouped GEMMs take bfloat16 or float16 tensors, got {t.dtype}")
+        if dt is None:
+            dt = t.dtype
+        elif t.dtype != dt:
+            raise NotImplementedError(f"{name} is {t.dtype} next to {dt} tensors: one operator call, one element type")
+    return dt or torch.bfloat16
 
 
 def _check_schedule_order(order: torch.Tensor | None, E: int) -> None:
@@ -100,7 +117,7 @@ def _up_projection_forward(
     gated activations and I otherwise; b1 is (E, N1)."""
     _lib.require_device(x, w1, y1, b1, expert_frequency_offset, expert_schedule_order, x_gather_idx)
     _check_schedule_order(expert_schedule_order, w1.size(2))
-    _check_bf16(("x", x), ("w1", w1), ("z", z), ("y1", y1), ("b1", b1))
+    dt = _elem_dtype(("x", x), ("w1", w1), ("z", z), ("y1", y1), ("b1", b1))
     N1, H, E = w1.shape
     I = N1 // 2 if is_glu_activation else N1
     T, TK = x.size(0), y1.size(0)
@@ -108,7 +125,7 @@ def _up_projection_forward(
     assert b1 is None or (b1.shape == (E, N1) and b1.is_contiguous())
     s_e, s_row = expert_major_strides(w1, "w1")
     ws = _gemm_workspace(TK, E, x.device, stream_id)
-    rc = _lib.lib().smoe_up_projection_forward(
+    rc = _lib.lib(dt).smoe_up_projection_forward(
         _lib.ptr(x),
         _lib.ptr(w1),
         s_e,
@@ -146,14 +163,14 @@ def _down_projection_forward(
     """y2 = y1 W2^T (+ b2) per expert; w2 is the (H, I, E) view of the (E, H, I) parameter, b2 is (E, H)."""
     _lib.require_device(w2, y1, y2, b2, expert_frequency_offset, expert_schedule_order)
     _check_schedule_order(expert_schedule_order, w2.size(2))
-    _check_bf16(("w2", w2), ("y1", y1), ("y2", y2), ("b2", b2))
+    dt = _elem_dtype(("w2", w2), ("y1", y1), ("y2", y2), ("b2", b2))
     H, I, E = w2.shape
     TK = y1.size(0)
     assert y1.is_contiguous() and y2.is_contiguous()
     assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous())
     s_e, s_row = expert_major_strides(w2, "w2")
     ws = _gemm_workspace(TK, E, y1.device, stream_id)
-    rc = _lib.lib().smoe_down_projection_forward(
+    rc = _lib.lib(dt).smoe_down_projection_forward(
         _lib.ptr(y1),
         _lib.ptr(w2),
         s_e,
@@ -194,7 +211,7 @@ def _down_projection_forward_combine(
     _lib.require_device(w2, y1, o, b2, topk_scores, expert_frequency_offset, expert_schedule_order, x_gather_idx,
                         s_scatter_idx)
     _check_schedule_order(expert_schedule_order, w2.size(2))
-    _check_bf16(("w2", w2), ("y1", y1), ("o", o), ("b2", b2))
+    dt = _elem_dtype(("w2", w2), ("y1", y1), ("o", o), ("b2", b2))
     H, I, E = w2.shape
     T, TK = o.size(0), y1.size(0)
     assert y1.is_contiguous() and o.is_contiguous() and o.size(1) == H
@@ -204,7 +221,7 @@ def _down_projection_forward_combine(
     assert b2 is None or (b2.shape == (E, H) and b2.is_contiguous())
     s_e, s_row = expert_major_strides(w2, "w2")
     ws = _gemm_workspace(TK, E, y1.device, stream_id)
-    rc = _lib.lib().smoe_down_projection_forward_combine(
+    rc = _lib.lib(dt).smoe_down_projection_forward_combine(
         _lib.ptr(y1),
         _lib.ptr(w2),
         s_e,
@@ -230,14 +247,14 @@ def _down_projection_forward_combine(
 
 def _gather_sum(src, out, weights, ridx, tok_off, K, H, is_varlen_K, what):
     _lib.require_device(src, out, weights, ridx, tok_off)
-    _check_bf16((what + ".src", src), (what + ".out", out))
+    dt = _elem_dtype((what + ".src", src), (what + ".out", out))
     assert src.is_contiguous() and out.is_contiguous() and ridx.dtype == torch.int32
     if weights is not None:
         assert weights.dtype == torch.float32 and weights.is_contiguous()
     if src.size(0) == 0:  # no routed row at all: every token's sum is empty
         out.zero_()
         return
-    rc = _lib.lib().smoe_gather_sum(
+    rc = _lib.lib(dt).smoe_gather_sum(
         _lib.ptr(src),
         _lib.ptr(out),
         _lib.ptr(weights),

@@ -17,7 +17,7 @@ import torch
 
 from .. import _lib
 from ..enums import ACTIVATION_CODE, LIBRARY_NAME, ActivationType
-from .forward import _check_bf16, _gemm_workspace
+from .forward import _elem_dtype, _gemm_workspace
 
 _FP8_FORWARD = False
 
@@ -58,11 +58,11 @@ def is_using_fp8_backward() -> bool:
 def _mx_quantize(src: torch.Tensor, q: torch.Tensor, scales: torch.Tensor) -> None:
     """src (R, C) bf16 -> q (R, C) uint8 e4m3 codes, scales (C/128, R) int32 (four exponent bytes per word)."""
     _lib.require_device(src, q, scales)
-    _check_bf16(("src", src))
+    dt = _elem_dtype(("src", src))
     R, C = src.shape
     assert src.stride(1) == 1 and q.is_contiguous() and scales.is_contiguous()
     assert q.dtype == torch.uint8 and q.shape == (R, C) and scales.dtype == torch.int32 and scales.shape == (C // 128, R)
-    rc = _lib.lib().smoe_mx_quantize(
+    rc = _lib.lib(dt).smoe_mx_quantize(
         _lib.ptr(src), src.stride(0), R, C, _lib.ptr(q), _lib.ptr(scales), _lib.current_stream_handle()
     )
     _lib.check(rc, "_mx_quantize")
@@ -144,7 +144,7 @@ def _up_projection_forward_fp8(
     """z = gather(xq) w1q^T (+ b1) with the block scales applied, y1 = act(z); xq (T, H), w1q (E*N1, H).  y1 comes back
     in bf16 (`y1`) and / or quantised in the epilogue (`y1q` (TK, I) uint8 with `y1q_scales` (I/128, TK) int32)."""
     _lib.require_device(xq, x_scales, w1q, w1_scales, y1, y1q, y1q_scales, b1, expert_frequency_offset, x_gather_idx)
-    _check_bf16(("z", z), ("y1", y1), ("b1", b1))
+    dt = _elem_dtype(("z", z), ("y1", y1), ("b1", b1))
     T, H = xq.shape
     TK, I = (y1 if y1 is not None else y1q).shape
     assert y1q is None or (y1q.dtype == torch.uint8 and y1q.is_contiguous() and y1q_scales.shape == (I // 128, TK))
@@ -152,7 +152,7 @@ def _up_projection_forward_fp8(
     assert w1q.shape == (E * N1, H) and x_scales.shape == (H // 128, T) and w1_scales.shape == (H // 128, E * N1)
     assert z is None or (z.shape == (TK, N1) and z.is_contiguous())
     ws = _gemm_workspace(TK, E, xq.device, stream_id, fp8_gathered_k=H)
-    rc = _lib.lib().smoe_up_projection_forward_fp8(
+    rc = _lib.lib(dt).smoe_up_projection_forward_fp8(
         _lib.ptr(xq),
         _lib.ptr(x_scales),
         _lib.ptr(w1q),
@@ -191,12 +191,12 @@ def _down_projection_forward_fp8(
 ) -> None:
     """y2 = y1q w2q^T (+ b2) with the block scales applied; y1q (TK, I), w2q (E*H, I)."""
     _lib.require_device(y1q, y1_scales, w2q, w2_scales, y2, b2, expert_frequency_offset)
-    _check_bf16(("y2", y2), ("b2", b2))
+    dt = _elem_dtype(("y2", y2), ("b2", b2))
     TK, I = y1q.shape
     H = y2.size(1)
     assert w2q.shape == (E * H, I) and y1_scales.shape == (I // 128, TK) and w2_scales.shape == (I // 128, E * H)
     ws = _gemm_workspace(TK, E, y1q.device, stream_id)
-    rc = _lib.lib().smoe_down_projection_forward_fp8(
+    rc = _lib.lib(dt).smoe_down_projection_forward_fp8(
         _lib.ptr(y1q),
         _lib.ptr(y1_scales),
         _lib.ptr(w2q),
@@ -220,12 +220,12 @@ def _mx_quantize_transposed(src: torch.Tensor, q: torch.Tensor, scales: torch.Te
     """src (E, R, C) bf16 (last dimension contiguous) -> q (E, C, R) uint8, the transposed matrices quantised along R,
     scales (R/128, E*C) int32."""
     _lib.require_device(src, q, scales)
-    _check_bf16(("src", src))
+    dt = _elem_dtype(("src", src))
     E, R, C = src.shape
     assert src.stride(2) == 1 and q.is_contiguous() and scales.is_contiguous()
     assert q.dtype == torch.uint8 and q.shape == (E, C, R)
     assert scales.dtype == torch.int32 and scales.shape == (R // 128, E * C)
-    rc = _lib.lib().smoe_mx_quantize_transposed(
+    rc = _lib.lib(dt).smoe_mx_quantize_transposed(
         _lib.ptr(src), src.stride(0), src.stride(1), E, R, C, _lib.ptr(q), _lib.ptr(scales),
         _lib.current_stream_handle()
     )
@@ -240,13 +240,13 @@ def _mx_quantize_both(src: torch.Tensor, q_rows: torch.Tensor, scales_rows: torc
     """src (E, R, C) bf16 -> both quantised copies from one pass over src: q_rows (E*R, C) / scales_rows (C/128, E*R) as
     `_mx_quantize` of the (E*R, C) matrix, q_t (E, C, R) / scales_t (R/128, E*C) as `_mx_quantize_transposed`."""
     _lib.require_device(src, q_rows, scales_rows, q_t, scales_t)
-    _check_bf16(("src", src))
+    dt = _elem_dtype(("src", src))
     E, R, C = src.shape
     assert src.stride(2) == 1 and all(t.is_contiguous() for t in (q_rows, scales_rows, q_t, scales_t))
     assert q_rows.dtype == torch.uint8 and q_rows.shape == (E * R, C) and q_t.dtype == torch.uint8 and q_t.shape == (E, C, R)
     assert scales_rows.dtype == torch.int32 and scales_rows.shape == (C // 128, E * R)
     assert scales_t.dtype == torch.int32 and scales_t.shape == (R // 128, E * C)
-    rc = _lib.lib().smoe_mx_quantize_both(
+    rc = _lib.lib(dt).smoe_mx_quantize_both(
         _lib.ptr(src), src.stride(0), src.stride(1), E, R, C, _lib.ptr(q_rows), _lib.ptr(scales_rows), _lib.ptr(q_t),
         _lib.ptr(scales_t), _lib.current_stream_handle()
     )
@@ -345,7 +345,7 @@ def _down_projection_backward_fp8(
     y1s = s * act(z) and ds exactly as the bf16 operator forms them.  doutq (T, H), w2tq (E*I, H)."""
     _lib.require_device(doutq, dout_scales, w2tq, w2t_scales, z, dz, dzq, dzq_scales, y1s, ds, topk_scores,
                         expert_frequency_offset, x_gather_idx, s_scatter_idx)
-    _check_bf16(("z", z), ("dz", dz), ("y1s", y1s))
+    dt = _elem_dtype(("z", z), ("dz", dz), ("y1s", y1s))
     T, H = doutq.shape
     TK, N1 = z.shape
     I = N1 // 2 if is_glu_activation else N1
@@ -354,10 +354,10 @@ def _down_projection_backward_fp8(
     assert dzq.dtype == torch.uint8 and dzq.shape == (TK, N1) and dzq.is_contiguous()
     assert dzq_scales.dtype == torch.int32 and dzq_scales.shape == (N1 // 128, TK) and dzq_scales.is_contiguous()
     assert ds.dtype == torch.float32 and ds.numel() == TK and topk_scores.dtype == torch.float32
-    ncols = _lib.lib().smoe_dz_partial_cols(I)
+    ncols = _lib.lib(dt).smoe_dz_partial_cols(I)
     ds_partial = torch.empty(max(TK, 1), ncols, dtype=torch.float32, device=z.device)
     ws = _gemm_workspace(TK, E, z.device, stream_id, fp8_gathered_k=H)
-    rc = _lib.lib().smoe_down_projection_backward_fp8(
+    rc = _lib.lib(dt).smoe_down_projection_backward_fp8(
         _lib.ptr(doutq),
         _lib.ptr(dout_scales),
         _lib.ptr(w2tq),
@@ -400,13 +400,13 @@ def _score_grad_bias_term(
     down-projection bias causes (the reference folds it into db2_and_ds_kernel, sonicmoe/functional/backward.py:36-107).
     `_down_projection_backward` adds it itself; `_down_projection_backward_fp8` does not know b2."""
     _lib.require_device(dout, b2, ds, expert_frequency_offset, x_gather_idx, s_scatter_idx)
-    _check_bf16(("dout", dout), ("b2", b2))
+    dt = _elem_dtype(("dout", dout), ("b2", b2))
     T, H = dout.shape
     E = expert_frequency_offset.numel() - 1
     TK = x_gather_idx.numel()
     assert dout.is_contiguous() and b2.shape == (E, H) and b2.is_contiguous()
     assert ds.dtype == torch.float32 and ds.numel() == TK and ds.is_contiguous() and s_scatter_idx.numel() == TK
-    rc = _lib.lib().smoe_score_grad_bias_term(
+    rc = _lib.lib(dt).smoe_score_grad_bias_term(
         _lib.ptr(dout), _lib.ptr(b2), _lib.ptr(expert_frequency_offset), _lib.ptr(x_gather_idx), _lib.ptr(s_scatter_idx),
         _lib.ptr(ds), TK, H, E, stream_id,
     )

@@ -104,7 +104,38 @@ def test_tuning_knobs(lib):
 def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     from sonicmoe import _lib
 
+    import torch
+
     monkeypatch.setenv("SONICMOE_HIP_LIB", str(tmp_path / "nope.so"))
-    monkeypatch.setattr(_lib, "_LIB", None)
+    monkeypatch.setenv("SONICMOE_HIP_LIB_F16", str(tmp_path / "nope_f16.so"))
+    monkeypatch.setattr(_lib, "_LIBS", {})
     with pytest.raises(RuntimeError, match="not found"):
         _lib.lib()
+    with pytest.raises(RuntimeError, match="not found"):
+        _lib.lib(torch.float16)
+    with pytest.raises(NotImplementedError, match="no build"):
+        _lib.lib(torch.float32)
+
+
+def test_the_fp16_build_exports_the_same_entry_points(lib):
+    """libsonicmoe_hip_f16.so is the same sources with fp16 as the 16-bit element type: same symbols, same argument
+    checks; the fused router (bf16 bit tricks) refuses."""
+    import torch
+
+    from sonicmoe import _lib
+
+    lib16 = _lib.lib(torch.float16)
+    assert lib16 is not lib and lib16._name.endswith("libsonicmoe_hip_f16.so")
+    for n in declared_functions():
+        assert getattr(lib16, n) is not None
+    assert lib16.smoe_version() == lib.smoe_version()
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    assert lib16.smoe_up_projection_forward(p, p, 0, 0, None, p, p, p, None, p, 4, 8, 96, 64, 2, 0, p, 1 << 20,
+                                            None) == 2
+    assert b"multiple of 64" in lib16.smoe_last_error()
+    assert lib16.smoe_router_forward_fused(p, p, 16, 512, 16, 2, p, p, p, None, None) == 2
+    assert b"bf16 only" in lib16.smoe_last_error()
+    # a knob set through the binding reaches both builds
+    _lib.set_tuning("gemm_stream", 0)
+    _lib.set_tuning("gemm_stream", -1)
