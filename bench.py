@@ -45,10 +45,10 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_inputs(cfg, dev, seed=0):
+def make_inputs(cfg, dev, seed=0, dtype=torch.bfloat16):
     g = torch.Generator(device=dev).manual_seed(seed)
     T, H, I, E = cfg["T"], cfg["H"], cfg["I"], cfg["E"]
-    bf = torch.bfloat16
+    bf = dtype
     x = torch.randn(T, H, generator=g, device=dev, dtype=torch.float32).to(bf).requires_grad_()
     wr = (0.02 * torch.randn(E, H, generator=g, device=dev)).to(bf).requires_grad_()
     w1 = (0.02 * torch.randn(E, 2 * I, H, generator=g, device=dev)).to(bf).requires_grad_()
@@ -365,7 +365,7 @@ def cpu_baseline(cfg, budget_s=20.0):
     )
 
 
-def measure_layer(cfg, name, dev, steps, warmup):
+def measure_layer(cfg, name, dev, steps, warmup, dtype=torch.bfloat16):
     """Forward and forward+backward of the whole layer at one configuration.  Returns (record, tensors) where tensors are
     the inputs, kept for the per-kernel breakdown of the headline configuration."""
     from sonicmoe.enums import ActivationType
@@ -378,10 +378,10 @@ def measure_layer(cfg, name, dev, steps, warmup):
     )
 
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
-    x, wr, w1, w2, dout = make_inputs(cfg, dev)
+    x, wr, w1, w2, dout = make_inputs(cfg, dev, dtype=dtype)
     stream = torch.cuda.current_stream().cuda_stream
     w1v, w2v = w1.permute(1, 2, 0), w2.permute(1, 2, 0)
-    bias = zipf_bias(E, dev).to(torch.bfloat16) if cfg["zipf"] else None
+    bias = zipf_bias(E, dev).to(dtype) if cfg["zipf"] else None
 
     rounding = cfg.get("rounding")
     if rounding:
@@ -595,6 +595,11 @@ def main():
             del tt
             torch.cuda.empty_cache()
         out["other_configs"] = others
+        # the headline configuration on fp16 tensors (the second build of the library; same kernels, f16 MFMA)
+        r16, tt = measure_layer(CONFIGS["C2"], "C2 on fp16 tensors", dev, max(5, a.steps // 2), 2, dtype=torch.float16)
+        out["fp16_fwd_bwd"] = {k: r16[k] for k in ("ms_per_step", "tflops", "frac_of_peak", "fwd_ms", "fwd_tflops")}
+        del tt
+        torch.cuda.empty_cache()
         shapes = {}
         for name in ("I512", "I256"):
             c = CONFIGS[name]

@@ -1,11 +1,22 @@
-/* C ABI of libsonicmoe_hip.so: the gfx950 (MI355X) kernels behind the `sonicmoe::*` operators of the MoE layer.
+/* C ABI of libsonicmoe_hip.so and libsonicmoe_hip_f16.so: the gfx950 (MI355X) kernels behind the `sonicmoe::*`
+ * operators of the MoE layer.
+ *
+ * Two libraries, one interface.  Both are built from the same sources and export every entry point declared here with
+ * the same arguments.  They differ in the 16-bit ELEMENT TYPE of the tensors that the grouped GEMMs, the gather-sums,
+ * the bias / score-gradient kernels, the router weight gradient and the fp8 quantisers read and write: bf16 in
+ * libsonicmoe_hip.so, fp16 in libsonicmoe_hip_f16.so - the two types the reference's grouped GEMMs take
+ * (sonicmoe/functional/grouped_gemm.py:3033-3044).  "bf16" in the comments below means that element type.  A caller
+ * links or dlopen()s the one that matches its tensors (both may be loaded into one process: load them without
+ * RTLD_GLOBAL, the symbol names are the same).  Entry points that take an smoe_dtype code (top-k, switch loss, token
+ * rounding) behave identically in both; smoe_router_forward_fused exists for bf16 only and returns
+ * SMOE_ERR_UNSUPPORTED in the fp16 library.  Tuning knobs and the last-error text are per library.
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; the library never allocates device memory
  *   - `stream` is a hipStream_t passed as void* (NULL = default stream); all work is asynchronous on it
  *   - return value: 0 = SMOE_OK, otherwise an smoe_status; smoe_last_error() gives the message of the last
  *     failing call on the calling thread
- *   - activations / weights are bf16 (raw uint16 bits), routing scores fp32, all indices int32
+ *   - activations / weights are the library's 16-bit element type (raw bits), routing scores fp32, all indices int32
  *   - weights are addressed in the PARAMETER layout of the reference module: W1 (E, 2I, H) and W2 (E, H, I),
  *     innermost dimension contiguous, with explicit expert and row strides in ELEMENTS (the reference hands its
  *     kernels permuted views of exactly these buffers: sonicmoe/moe.py:223-225)
