@@ -136,7 +136,7 @@ int launch_build_tile_map(const int32_t* off, const int32_t* order, int E, int B
 
 }  // namespace smoe
 
-extern "C" int smoe_version(void) { return 300; }
+extern "C" int smoe_version(void) { return 310; }
 extern "C" const char* smoe_last_error(void) { return smoe::g_error; }
 
 extern "C" int smoe_set_tuning(const char* name, int value) {
