@@ -139,3 +139,19 @@ def test_the_fp16_build_exports_the_same_entry_points(lib):
     # a knob set through the binding reaches both builds
     _lib.set_tuning("gemm_stream", 0)
     _lib.set_tuning("gemm_stream", -1)
+
+
+def test_element_type_of_an_operator_call():
+    """Host logic that picks the library build: one 16-bit element type per operator call, bf16 or fp16."""
+    import torch
+
+    from sonicmoe.functional.forward import _elem_dtype
+
+    b, h, f = (torch.empty(2, dtype=d) for d in (torch.bfloat16, torch.float16, torch.float32))
+    assert _elem_dtype(("x", b), ("bias", None), ("y", b)) == torch.bfloat16
+    assert _elem_dtype(("x", h), ("y", h)) == torch.float16
+    assert _elem_dtype(("bias", None)) == torch.bfloat16   # nothing to go by: the default build
+    with pytest.raises(NotImplementedError, match="one element type"):
+        _elem_dtype(("x", b), ("w", h))
+    with pytest.raises(NotImplementedError, match="bfloat16 or float16"):
+        _elem_dtype(("x", f))
