@@ -186,16 +186,18 @@ def test_torch_backend_of_module_matches_oracle(dev):
     assert rel_l2(out, out_ref) < 1e-5
 
 
-def test_general_routing_layer(dev):
-    """moe_general_routing_inputs against the per-expert masked loop of the reference's benchmark."""
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, TOL), (torch.float16, 3e-3)], ids=["bf16", "fp16"])
+def test_general_routing_layer(dev, dtype, tol):
+    """moe_general_routing_inputs against the per-expert masked loop of the reference's benchmark, on bf16 tensors and
+    on fp16 ones (the second build of the library)."""
     from sonicmoe.enums import ActivationType
     from sonicmoe.functional import moe_general_routing_inputs
     from helpers import make_weights
 
     T, H, I, E = 1024, 512, 256, 16
-    _, w1, w2 = make_weights(E, H, I, dev, seed=3)
+    _, w1, w2 = make_weights(E, H, I, dev, dtype=dtype, seed=3)
     g = torch.Generator().manual_seed(4)
-    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev).requires_grad_()
+    x = torch.randn(T, H, generator=g).to(dtype).to(dev).requires_grad_()
     # ragged: token t gets (t % 5) experts, so some tokens get none
     tok, exp = [], []
     for t in range(T):
@@ -209,7 +211,7 @@ def test_general_routing_layer(dev):
     w1p, w2p = w1.requires_grad_(), w2.requires_grad_()
     o, freq = moe_general_routing_inputs(x, scores, tok, exp, w1p.permute(1, 2, 0), None, w2p.permute(1, 2, 0), None, E,
                                          torch.cuda.current_stream().cuda_stream, ActivationType.SWIGLU, False)
-    dy = torch.randn(T, H, generator=g).to(torch.bfloat16).to(dev)
+    dy = torch.randn(T, H, generator=g).to(dtype).to(dev)
     grads = torch.autograd.grad(o, [x, scores, w1p, w2p], grad_outputs=dy)
 
     xr, sr = x.detach().clone().requires_grad_(), scores.detach().clone().requires_grad_()
@@ -217,9 +219,9 @@ def test_general_routing_layer(dev):
     o_ref = M.general_routing_reference(xr, sr, tok, exp, w1r, w2r, E)
     grads_ref = torch.autograd.grad(o_ref, [xr, sr, w1r, w2r], grad_outputs=dy.float())
     assert torch.equal(freq.cpu(), torch.bincount(exp.long().cpu(), minlength=E).int())
-    assert rel_l2(o, o_ref) < TOL
+    assert o.dtype == dtype and rel_l2(o, o_ref) < tol
     for n, a, b in zip(["dx", "dscores", "dw1", "dw2"], grads, grads_ref):
-        assert rel_l2(a, b) < TOL, n
+        assert rel_l2(a, b) < tol, n
     # tokens without any expert get exactly zero
     assert bool((o[::5] == 0).all())
 
