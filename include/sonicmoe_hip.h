@@ -109,6 +109,12 @@ int smoe_topk_softmax_fwd(const void* logits, int dtype, int64_t T, int E, int K
 int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const float* dscores, const float* scores,
                           const int32_t* indices, int64_t T, int K, void* stream);
 
+/* Backward of the top-K WITHOUT softmax (smoe_topk_softmax_fwd with softmax == 0): dlogits[t, indices[t, k]] =
+ * dvalues[t, k]; the caller zero-fills dlogits.  Replaces sonicmoe::_topk_bwd (sonicmoe/functional/backward.py:559-610;
+ * no caller inside the reference's layer entry points).  dvalues (T, K) fp32 contiguous, dlogits has `dtype`. */
+int smoe_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const float* dvalues, const int32_t* indices, int64_t T,
+                  int K, void* stream);
+
 /* Routing metadata by a stable counting sort over expert ids.  Replaces TC_topk_router_metadata and
  * general_routing_router_metadata incl. their count_cumsum / argsort / index kernels
  * (sonicmoe/functional/__init__.py:19-46, :49-82).

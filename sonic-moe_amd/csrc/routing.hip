@@ -163,6 +163,18 @@ __global__ __launch_bounds__(256) void softmax_topk_bwd_kernel(T* __restrict__ d
   for (int k = 0; k < K; k++) store_from_f32<T>(out + ix[k], s[k] * (g[k] - dot));
 }
 
+// Backward of the un-fused top-K (values without softmax): the gradient of a selected logit is the gradient of its
+// value.  One thread per token; the caller has zero-filled dlogits.
+template <typename T>
+__global__ __launch_bounds__(256) void topk_bwd_kernel(T* __restrict__ dlogits, int64_t row_stride,
+                                                       const float* __restrict__ dvalues,
+                                                       const int32_t* __restrict__ indices, int64_t Trows, int K) {
+  const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (row >= Trows) return;
+  T* out = dlogits + row * row_stride;
+  for (int k = 0; k < K; k++) store_from_f32<T>(out + indices[row * K + k], dvalues[row * K + k]);
+}
+
 // ============================================================================================================
 // count + inclusive cumsum (standalone operator)
 // ============================================================================================================
@@ -436,6 +448,33 @@ extern "C" int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_strid
       break;
     default:
       set_error("softmax_topk_bwd: unknown dtype %d", dtype);
+      return SMOE_ERR_INVALID;
+  }
+  SMOE_LAUNCH_CHECK();
+  return SMOE_OK;
+}
+
+extern "C" int smoe_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const float* dvalues, const int32_t* indices,
+                             int64_t T, int K, void* stream) {
+  SMOE_REQUIRE(T >= 0 && K >= 1, SMOE_ERR_INVALID, "topk_bwd: bad sizes");
+  if (T == 0) return SMOE_OK;
+  SMOE_REQUIRE(dlogits && dvalues && indices, SMOE_ERR_INVALID, "topk_bwd: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)ceil_div(T, 256)), block(256);
+  switch (dtype) {
+    case SMOE_DT_BF16:
+      hipLaunchKernelGGL(topk_bwd_kernel<uint16_t>, grid, block, 0, st, (uint16_t*)dlogits, row_stride, dvalues, indices,
+                         T, K);
+      break;
+    case SMOE_DT_F16:
+      hipLaunchKernelGGL(topk_bwd_kernel<__half>, grid, block, 0, st, (__half*)dlogits, row_stride, dvalues, indices, T,
+                         K);
+      break;
+    case SMOE_DT_F32:
+      hipLaunchKernelGGL(topk_bwd_kernel<float>, grid, block, 0, st, (float*)dlogits, row_stride, dvalues, indices, T, K);
+      break;
+    default:
+      set_error("topk_bwd: unknown dtype %d", dtype);
       return SMOE_ERR_INVALID;
   }
   SMOE_LAUNCH_CHECK();

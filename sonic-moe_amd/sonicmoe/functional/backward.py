@@ -231,6 +231,23 @@ def _softmax_topk_bwd(
     _lib.check(rc, "_softmax_topk_bwd")
 
 
+@torch.library.custom_op(f"{LIBRARY_NAME}::_topk_bwd", mutates_args={"dlogits_full"})
+def _topk_bwd(dlogits_full: torch.Tensor, dtopk_values: torch.Tensor, topk_indices: torch.Tensor, K: int) -> None:
+    """dlogits_full[t, idx[t,k]] = dtopk_values[t,k]: backward of `_topk_fwd` without the softmax fusion; the caller
+    zero-fills dlogits_full (sonicmoe/functional/backward.py:589-610 of the reference, which has no caller for it)."""
+    _lib.require_device(dlogits_full, dtopk_values, topk_indices)
+    if dlogits_full.dtype not in _lib.DT_CODE:
+        raise NotImplementedError(f"_topk_bwd: unsupported dtype {dlogits_full.dtype}")
+    dtopk_values = dtopk_values.contiguous().float()
+    assert topk_indices.is_contiguous() and topk_indices.dtype == torch.int32 and dlogits_full.stride(1) == 1
+    assert dtopk_values.shape == topk_indices.shape and dtopk_values.size(1) == K
+    rc = _lib.lib().smoe_topk_bwd(
+        _lib.ptr(dlogits_full), _lib.DT_CODE[dlogits_full.dtype], dlogits_full.stride(0), _lib.ptr(dtopk_values),
+        _lib.ptr(topk_indices), dtopk_values.size(0), K, _lib.current_stream_handle(),
+    )
+    _lib.check(rc, "_topk_bwd")
+
+
 @torch.library.custom_op(f"{LIBRARY_NAME}::_router_weight_grad", mutates_args={"partial"})
 def _router_weight_grad(dlogits: torch.Tensor, x: torch.Tensor, partial: torch.Tensor) -> None:
     """partial[c] (E, H) = dlogits[rows of chunk c]^T x[rows of chunk c]; the chunks are partial.size(0) equal token

@@ -149,6 +149,23 @@ def test_softmax_topk_bwd(dev, dtype):
         np.testing.assert_allclose(got, torch.from_numpy(ref).to(dtype).float().numpy(), rtol=1e-2, atol=1e-6)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_topk_bwd_is_the_gradient_of_topk(dev, dtype):
+    """`_topk_bwd` (the un-fused top-K's backward) against autograd through torch.topk on tie-free fp32 logits: the
+    gradient of a selected logit is the gradient of its value, every other entry stays zero; exact (a scatter)."""
+    _, _, fwd, bwd = _ops()
+    T, E, K = 513, 64, 6
+    g = torch.Generator().manual_seed(11)
+    logits = torch.randn(T, E, generator=g).requires_grad_()
+    vals, idx = torch.topk(logits, K, dim=-1)
+    dv = torch.randn(T, K, generator=g)
+    (ref,) = torch.autograd.grad(vals, logits, grad_outputs=dv)
+    dl = torch.zeros(T, E, dtype=dtype, device=dev)
+    bwd._topk_bwd(dl, dv.to(dev), idx.to(torch.int32).to(dev), K)
+    torch.cuda.synchronize()
+    assert torch.equal(dl.cpu(), ref.to(dtype))
+
+
 @pytest.mark.parametrize("mode", ["nr", "up", "down"])
 @pytest.mark.parametrize("T,E,K,tile,dtype", [
     (512, 16, 2, 32, torch.bfloat16),
