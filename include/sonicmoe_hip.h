@@ -104,10 +104,12 @@ int smoe_count_cumsum(const void* x, int x_is_int64, int64_t n, int E, int32_t* 
 int smoe_topk_softmax_fwd(const void* logits, int dtype, int64_t T, int E, int K, int64_t row_stride,
                           float* scores, int32_t* indices, int softmax, void* stream);
 
-/* dlogits[t, idx[t,k]] = s_k (ds_k - sum_j ds_j s_j); other entries are left untouched (caller zero-fills).
+/* dlogits[t, idx[t,k]] = s_k (ds_k - sum_j ds_j s_j) (+ dlogits_add[t, idx[t,k]] when dlogits_add is not NULL: the
+ * reference's optional `dlogits` argument, a gradient that reached the selected logits some other way; same dtype and
+ * row stride as dlogits, may be dlogits itself); other entries are left untouched (caller zero-fills).
  * Replaces sonicmoe::_softmax_topk_bwd (sonicmoe/functional/backward.py:487-556). dlogits has `dtype`. */
-int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const float* dscores, const float* scores,
-                          const int32_t* indices, int64_t T, int K, void* stream);
+int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const void* dlogits_add, const float* dscores,
+                          const float* scores, const int32_t* indices, int64_t T, int K, void* stream);
 
 /* Backward of the top-K WITHOUT softmax (smoe_topk_softmax_fwd with softmax == 0): dlogits[t, indices[t, k]] =
  * dvalues[t, k]; the caller zero-fills dlogits.  Replaces sonicmoe::_topk_bwd (sonicmoe/functional/backward.py:559-610;

@@ -148,7 +148,7 @@ __device__ __forceinline__ void store_from_f32<float>(float* p, float v) {
 
 template <typename T>
 __global__ __launch_bounds__(256) void softmax_topk_bwd_kernel(T* __restrict__ dlogits, int64_t row_stride,
-                                                               const float* __restrict__ dscores,
+                                                               const T* dlogits_add, const float* __restrict__ dscores,
                                                                const float* __restrict__ scores,
                                                                const int32_t* __restrict__ indices, int64_t Trows,
                                                                int K) {
@@ -160,7 +160,13 @@ __global__ __launch_bounds__(256) void softmax_topk_bwd_kernel(T* __restrict__ d
   float dot = 0.f;
   for (int k = 0; k < K; k++) dot += g[k] * s[k];
   T* out = dlogits + row * row_stride;
-  for (int k = 0; k < K; k++) store_from_f32<T>(out + ix[k], s[k] * (g[k] - dot));
+  // dlogits_add (may be dlogits itself): a gradient that reached the selected logits some other way is added in
+  const T* add = dlogits_add ? dlogits_add + row * row_stride : nullptr;
+  for (int k = 0; k < K; k++) {
+    float v = s[k] * (g[k] - dot);
+    if (add) v += __uint_as_float(load_as_f32_bits<T>(add + ix[k]));
+    store_from_f32<T>(out + ix[k], v);
+  }
 }
 
 // Backward of the un-fused top-K (values without softmax): the gradient of a selected logit is the gradient of its
@@ -426,8 +432,9 @@ extern "C" int smoe_topk_softmax_fwd(const void* logits, int dtype, int64_t T, i
   return SMOE_ERR_INVALID;
 }
 
-extern "C" int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const float* dscores,
-                                     const float* scores, const int32_t* indices, int64_t T, int K, void* stream) {
+extern "C" int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_stride, const void* dlogits_add,
+                                     const float* dscores, const float* scores, const int32_t* indices, int64_t T, int K,
+                                     void* stream) {
   SMOE_REQUIRE(T >= 0 && K >= 1, SMOE_ERR_INVALID, "softmax_topk_bwd: bad sizes");
   if (T == 0) return SMOE_OK;
   SMOE_REQUIRE(dlogits && dscores && scores && indices, SMOE_ERR_INVALID, "softmax_topk_bwd: null pointer");
@@ -436,15 +443,15 @@ extern "C" int smoe_softmax_topk_bwd(void* dlogits, int dtype, int64_t row_strid
   switch (dtype) {
     case SMOE_DT_BF16:
       hipLaunchKernelGGL(softmax_topk_bwd_kernel<uint16_t>, grid, block, 0, st, (uint16_t*)dlogits, row_stride,
-                         dscores, scores, indices, T, K);
+                         (const uint16_t*)dlogits_add, dscores, scores, indices, T, K);
       break;
     case SMOE_DT_F16:
-      hipLaunchKernelGGL(softmax_topk_bwd_kernel<__half>, grid, block, 0, st, (__half*)dlogits, row_stride, dscores,
-                         scores, indices, T, K);
+      hipLaunchKernelGGL(softmax_topk_bwd_kernel<__half>, grid, block, 0, st, (__half*)dlogits, row_stride,
+                         (const __half*)dlogits_add, dscores, scores, indices, T, K);
       break;
     case SMOE_DT_F32:
-      hipLaunchKernelGGL(softmax_topk_bwd_kernel<float>, grid, block, 0, st, (float*)dlogits, row_stride, dscores,
-                         scores, indices, T, K);
+      hipLaunchKernelGGL(softmax_topk_bwd_kernel<float>, grid, block, 0, st, (float*)dlogits, row_stride,
+                         (const float*)dlogits_add, dscores, scores, indices, T, K);
       break;
     default:
       set_error("softmax_topk_bwd: unknown dtype %d", dtype);

@@ -28,7 +28,7 @@ _SIGNATURES = {
     "smoe_set_tuning": (c_int, [c_char_p, _I]),
     "smoe_count_cumsum": (c_int, [_P, _I, _L, _I, _P, _P, _P]),
     "smoe_topk_softmax_fwd": (c_int, [_P, _I, _L, _I, _I, _L, _P, _P, _I, _P]),
-    "smoe_softmax_topk_bwd": (c_int, [_P, _I, _L, _P, _P, _P, _L, _I, _P]),
+    "smoe_softmax_topk_bwd": (c_int, [_P, _I, _L, _P, _P, _P, _P, _L, _I, _P]),
     "smoe_topk_bwd": (c_int, [_P, _I, _L, _P, _P, _L, _I, _P]),
     "smoe_routing_metadata_workspace_bytes": (c_size_t, [_L, _I]),
     "smoe_routing_metadata": (c_int, [_P, _P, _L, _L, _I, _I, _P, _P, _P, _P, _P, _P, _P, _Z, _P]),

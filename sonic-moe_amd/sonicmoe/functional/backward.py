@@ -209,18 +209,21 @@ def _softmax_topk_bwd(
     topk_router_indices: torch.Tensor,
     K: int,
 ) -> None:
-    """dlogits_full[t, idx[t,k]] = s_k (ds_k - sum_j ds_j s_j); the caller zero-fills dlogits_full."""
-    if dlogits is not None:
-        raise NotImplementedError("_softmax_topk_bwd: accumulating into an existing dlogits is not supported")
-    _lib.require_device(dlogits_full, dtopk_score, topk_router_score, topk_router_indices)
+    """dlogits_full[t, idx[t,k]] = s_k (ds_k - sum_j ds_j s_j) (+ dlogits[t, idx[t,k]] when `dlogits` is given, as in
+    the reference: a gradient that reached the selected logits some other way); the caller zero-fills dlogits_full."""
+    _lib.require_device(dlogits_full, dlogits, dtopk_score, topk_router_score, topk_router_indices)
     if dlogits_full.dtype not in _lib.DT_CODE:
         raise NotImplementedError(f"_softmax_topk_bwd: unsupported dtype {dlogits_full.dtype}")
+    if dlogits is not None and (dlogits.dtype != dlogits_full.dtype or dlogits.shape != dlogits_full.shape
+                                or dlogits.stride() != dlogits_full.stride()):
+        raise ValueError("_softmax_topk_bwd: dlogits must have the dtype, shape and strides of dlogits_full")
     dtopk_score = dtopk_score.contiguous().float()
     assert topk_router_score.is_contiguous() and topk_router_indices.is_contiguous() and dlogits_full.stride(1) == 1
     rc = _lib.lib().smoe_softmax_topk_bwd(
         _lib.ptr(dlogits_full),
         _lib.DT_CODE[dlogits_full.dtype],
         dlogits_full.stride(0),
+        _lib.ptr(dlogits),
         _lib.ptr(dtopk_score),
         _lib.ptr(topk_router_score),
         _lib.ptr(topk_router_indices),

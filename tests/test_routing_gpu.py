@@ -147,6 +147,15 @@ def test_softmax_topk_bwd(dev, dtype):
         np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-7)
     else:
         np.testing.assert_allclose(got, torch.from_numpy(ref).to(dtype).float().numpy(), rtol=1e-2, atol=1e-6)
+    # the optional `dlogits` argument: a gradient already sitting at the selected positions is added in (and only
+    # there: what the reference's kernel does, backward.py:520-525)
+    extra = torch.randn(T, E, generator=g).to(dtype)
+    dl2 = torch.zeros(T, E, dtype=dtype, device=dev)
+    bwd._softmax_topk_bwd(dl2, extra.to(dev), ds.to(dev), torch.from_numpy(s).to(dev), torch.from_numpy(i).to(dev), K)
+    sel = torch.zeros(T, E, dtype=torch.bool).scatter_(1, torch.from_numpy(i).long(), True)
+    want = torch.where(sel, torch.from_numpy(ref) + extra.float(), torch.zeros(()))
+    np.testing.assert_allclose(dl2.float().cpu().numpy(), want.to(dtype).float().numpy(),
+                               rtol=1e-5 if dtype == torch.float32 else 1e-2, atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
