@@ -6,8 +6,9 @@
  * the bias / score-gradient kernels, the router weight gradient and the fp8 quantisers read and write: bf16 in
  * libsonicmoe_hip.so, fp16 in libsonicmoe_hip_f16.so - the two types the reference's grouped GEMMs take
  * (sonicmoe/functional/grouped_gemm.py:3033-3044).  "bf16" in the comments below means that element type.  A caller
- * links or dlopen()s the one that matches its tensors (both may be loaded into one process: load them without
- * RTLD_GLOBAL, the symbol names are the same).  Entry points that take an smoe_dtype code (top-k, switch loss, token
+ * links or dlopen()s the one that matches its tensors.  Both may be loaded into one process with dlopen(): the symbol
+ * names are the same, so look the entry points up per handle (dlsym), and each library is linked -Bsymbolic so that it
+ * keeps calling its own kernels even next to an RTLD_GLOBAL copy of the other.  Entry points that take an smoe_dtype code (top-k, switch loss, token
  * rounding) behave identically in both; smoe_router_forward_fused exists for bf16 only and returns
  * SMOE_ERR_UNSUPPORTED in the fp16 library.  Tuning knobs and the last-error text are per library.
  *

@@ -78,7 +78,10 @@ def build(verbose: bool = False, resource_usage: bool = False, jobs: int | None 
     for name, _, suffix in VARIANTS:
         mine = [o for o, (_, _, sfx) in zip(objs, work) if sfx == suffix]
         tmp = OUT_DIR / (name + ".tmp")
-        _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, mine)], verbose)
+        # -Bsymbolic: the two libraries define the same symbols; each binds its internal references (kernel stubs
+        # included) to its own definitions even if a host program loads the other one with RTLD_GLOBAL first
+        _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", str(tmp), *map(str, mine)],
+             verbose)
         os.replace(tmp, OUT_DIR / name)
     return OUT_DIR / LIB_NAME
 

@@ -9,13 +9,15 @@ from __future__ import annotations
 
 import ctypes
 import os
+import threading
 from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 from pathlib import Path
 
 import torch
 
 _LIBS: dict[torch.dtype, ctypes.CDLL] = {}
-_LAST: ctypes.CDLL | None = None   # the library of the latest lib() call: check() asks it for the error text
+_TLS = threading.local()           # .last = the library of this thread's latest lib() call: check() asks it for the
+                                   # error text (the libraries keep their last error per thread as well)
 _TUNING: dict[str, int] = {}       # overrides made so far, for a library that is loaded later
 
 DT_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
@@ -93,7 +95,6 @@ def library_path(dtype: torch.dtype = torch.bfloat16) -> Path:
 
 def lib(dtype: torch.dtype = torch.bfloat16) -> ctypes.CDLL:
     """The library whose 16-bit element type is `dtype` (operators without such tensors use the default)."""
-    global _LAST
     handle = _LIBS.get(dtype)
     if handle is None:
         if dtype not in _LIB_FILES:
@@ -112,7 +113,7 @@ def lib(dtype: torch.dtype = torch.bfloat16) -> ctypes.CDLL:
         for name, value in _TUNING.items():
             handle.smoe_set_tuning(name.encode(), value)
         _LIBS[dtype] = handle
-    _LAST = handle
+    _TLS.last = handle
     return handle
 
 
@@ -122,7 +123,7 @@ def exported_symbols() -> list[str]:
 
 def check(rc: int, what: str) -> None:
     if rc != 0:
-        msg = (_LAST or lib()).smoe_last_error().decode(errors="replace")
+        msg = (getattr(_TLS, "last", None) or lib()).smoe_last_error().decode(errors="replace")
         raise RuntimeError(f"{what} failed (status {rc}): {msg}")
 
 

@@ -6,6 +6,8 @@ the bf16 tests' 1e-2: relative L2 <= 1.5e-3 per operator (measured ~3e-4, the ou
 through bf16 on its way would sit at 2e-3 .. 4e-3 and fail it.
 """
 
+from pathlib import Path
+
 import pytest
 import torch
 
@@ -14,6 +16,7 @@ from oracle import moe_math as M
 from oracle import routing as R
 
 pytestmark = pytest.mark.gpu
+ROOT = Path(__file__).resolve().parent.parent
 F16 = torch.float16
 TOL = 1.5e-3
 
@@ -182,3 +185,38 @@ def test_fp16_layer_with_fp8_gemms(dev):
     errs = [rel_l2(out8, out)] + [rel_l2(a, b) for a, b in zip(grads8, grads)]
     print("fp16 tensors, fp8 GEMMs: out, dx, dWr, dW1, dW2 rel-L2 vs the fp16 path:", errs)
     assert all(1e-2 < e < 9e-2 for e in errs), errs
+
+
+def test_libraries_do_not_interpose_each_other(dev):
+    """The two builds define the same symbols.  A host program that has loaded the bf16 library with RTLD_GLOBAL must
+    still get fp16 arithmetic from the fp16 library (each is linked to bind its own definitions): a child process does
+    exactly that and runs one fp16 up-projection against torch."""
+    import subprocess
+    import sys
+    import textwrap
+
+    code = textwrap.dedent("""
+        import ctypes, sys, torch
+        sys.path[:0] = [%r, %r]
+        from sonicmoe import _lib
+        ctypes.CDLL(str(_lib.library_path(torch.bfloat16)), mode=ctypes.RTLD_GLOBAL)
+        from sonicmoe.functional import forward
+        dev = torch.device("cuda:0")
+        T, H, I, E = 512, 256, 128, 2
+        g = torch.Generator().manual_seed(1)
+        x = torch.randn(T, H, generator=g).half().to(dev)
+        w1 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).half().to(dev)
+        off = torch.tensor([0, 200, T], dtype=torch.int32, device=dev)
+        gidx = torch.randperm(T, generator=g).to(torch.int32).to(dev)
+        z = torch.empty(T, 2 * I, dtype=torch.float16, device=dev)
+        y1 = torch.empty(T, I, dtype=torch.float16, device=dev)
+        forward._up_projection_forward(x, w1.permute(1, 2, 0), z, y1, None, off, None, gidx,
+                                       torch.cuda.current_stream().cuda_stream, "swiglu", True, False)
+        xg = x[gidx.long()].float()
+        ref = torch.cat([xg[:200] @ w1[0].float().t(), xg[200:] @ w1[1].float().t()])
+        err = float((z.float() - ref).norm() / ref.norm())
+        print("rel-L2", err)
+        assert err < 1.5e-3, err
+    """) % (str(ROOT / "sonic-moe_amd"), str(ROOT))
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=110)
+    assert res.returncode == 0, res.stdout + res.stderr
