@@ -88,7 +88,7 @@ def kernel_breakdown(cfg, x, wr, w1, w2, dout, steps, only=None, gemms_only=Fals
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     TK = T * K
     dev = x.device
-    bf = torch.bfloat16
+    bf = x.dtype
     stream = torch.cuda.current_stream().cuda_stream
     with torch.no_grad():
         logits = torch.nn.functional.linear(x, wr)
@@ -277,10 +277,10 @@ def recorded_traffic(kernel: str, config: str):
         return None
 
 
-def pmc_target(cfg, op_name, dev):
+def pmc_target(cfg, op_name, dev, dtype=torch.bfloat16):
     """Workload for the counter passes: 3 launches of one operator's kernel and one 1 GiB device-to-device copy whose
     FETCH_SIZE / WRITE_SIZE readings calibrate the counters."""
-    x, wr, w1, w2, dout = make_inputs(cfg, dev)
+    x, wr, w1, w2, dout = make_inputs(cfg, dev, dtype=dtype)
     a = torch.empty(1 << 28, dtype=torch.float32, device=dev).normal_()
     b = torch.empty_like(a)
     b.copy_(a)
@@ -468,6 +468,8 @@ def main():
     ap.add_argument("--no-breakdown", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the extra lines (C3, C4 layer times; per-kernel rows of the short-contraction shapes)")
+    ap.add_argument("--pmc-dtype", default="bf16", choices=["bf16", "fp16"],
+                    help="element type of the --pmc-target workload (fp16 = the second build of the library)")
     ap.add_argument("--pmc-target", default=None, choices=sorted(SINGLE_KERNEL_OPS),
                     help="run only this operator (3 launches) and a 1 GiB copy: the workload of the rocprofv3 --pmc passes")
     a = ap.parse_args()
@@ -481,7 +483,7 @@ def main():
     cfg = CONFIGS[a.config]
     dev = torch.device("cuda:0")
     if a.pmc_target:
-        pmc_target(cfg, a.pmc_target, dev)
+        pmc_target(cfg, a.pmc_target, dev, torch.float16 if a.pmc_dtype == "fp16" else torch.bfloat16)
         return
     T, H, I, E, K = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["K"]
     rec, t = measure_layer(cfg, a.config, dev, a.steps, a.warmup)
